@@ -1,0 +1,5 @@
+from .pages import PAGE_TOKENS, PagePool, CacheFull, CacheError, pages_for
+from .sequence_cache import SequenceCache, KvLayerView, StateLayerView
+
+__all__ = ["PAGE_TOKENS", "PagePool", "CacheFull", "CacheError", "pages_for", "SequenceCache", "KvLayerView",
+           "StateLayerView"]

@@ -1,0 +1,6 @@
+from .qwen3 import ConfigError, Qwen3Config
+from .registry import (Architecture, register_architecture, resolve_architecture, known_architectures,
+                       load_config, read_config_json)
+
+__all__ = ["ConfigError", "Qwen3Config", "Architecture", "register_architecture", "resolve_architecture",
+           "known_architectures", "load_config", "read_config_json"]

@@ -1,0 +1,86 @@
+// Shared device helpers for the gfx950 kernels: types, conversions, wave and block
+// reductions, and the error channel of the C entry points.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#define SYN_WAVE 64
+#define SYN_PAGE 64  // tokens per cache page; the host side asserts the same number
+
+typedef __bf16 bf16;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) short short4_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+// ---- error channel: every entry point returns 0, or a code after syn_set_error ----
+// One translation unit of each library places SYN_DEFINE_ERROR_CHANNEL at file scope.
+#define SYN_EXPORT extern "C" __attribute__((visibility("default")))
+SYN_EXPORT const char* syn_last_error();
+void syn_set_error(const char* fmt, ...);
+#define SYN_DEFINE_ERROR_CHANNEL                                   \
+  static thread_local char syn_error_text[512];                    \
+  SYN_EXPORT const char* syn_last_error() { return syn_error_text; } \
+  void syn_set_error(const char* fmt, ...) {                       \
+    va_list ap;                                                    \
+    va_start(ap, fmt);                                             \
+    vsnprintf(syn_error_text, sizeof(syn_error_text), fmt, ap);    \
+    va_end(ap);                                                    \
+  }
+#define SYN_CHECK(cond, ...)            \
+  do {                                  \
+    if (!(cond)) {                      \
+      syn_set_error(__VA_ARGS__);       \
+      return 1;                         \
+    }                                   \
+  } while (0)
+#define SYN_LAUNCH_CHECK(name)                                          \
+  do {                                                                  \
+    hipError_t e_ = hipGetLastError();                                  \
+    if (e_ != hipSuccess) {                                             \
+      syn_set_error("%s: launch failed: %s", name, hipGetErrorString(e_)); \
+      return 2;                                                         \
+    }                                                                   \
+  } while (0)
+
+// ---- conversions ----
+template <typename T> __device__ __forceinline__ float to_f32(T v);
+template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ float to_f32<bf16>(bf16 v) { return (float)v; }
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16 from_f32<bf16>(float v) { return (bf16)v; }
+
+// a weight vector that is bf16 or float, chosen at run time
+__device__ __forceinline__ float load_gain(const void* w, int is_f32, int i) {
+  return is_f32 ? ((const float*)w)[i] : (float)((const bf16*)w)[i];
+}
+
+// ---- reductions over the 64 lanes of a wave ----
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, SYN_WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, SYN_WAVE));
+  return v;
+}
+
+// sum over a block of up to 1024 threads; `red` holds 16 floats of LDS; all threads get the result
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
+  const int nw = (blockDim.x + SYN_WAVE - 1) / SYN_WAVE;
+  __syncthreads();  // `red` may still be read from an earlier call
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nw; ++i) t += red[i];
+  return t;
+}

@@ -1,0 +1,243 @@
+// Row kernels that move little data per flop: embedding gather, RMSNorm with the
+// residual sum fused in, SwiGLU, and the fused per-head q/k norm + rotation + cache write.
+//
+// Reference counterparts (one kernel each there, several fused here):
+//   crates/synaptix-kernels-cuda/src/cu/embed/embed.cu:18-46
+//   crates/synaptix-kernels-cuda/src/cu/reduction/rms_norm.cu:65-98
+//   crates/synaptix-kernels-cuda/src/cu/fused/norm/rmsnorm_residual.cu:97-159
+//   crates/synaptix-kernels-cuda/src/cu/fused/mlp/silu_and_mul.cu:11-52
+//   crates/synaptix-kernels-cuda/src/cu/elementwise/rope.cu:27-70, kv_append.cu:32-78
+#include "common.h"
+
+SYN_DEFINE_ERROR_CHANNEL
+
+// ------------------------------------------------------------------ embedding
+// resid[n, :] = table[ids[n], :] widened to float.  Ids are checked on the host.
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids, float* __restrict__ resid,
+                             int H) {
+  const int n = blockIdx.x;
+  const T* row = table + (size_t)ids[n] * H;
+  float* out = resid + (size_t)n * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = to_f32<T>(row[i]);
+}
+
+SYN_EXPORT int syn_embed(const void* table, int table_is_f32, const int* ids, float* resid, int n_tokens, int H,
+                         hipStream_t stream) {
+  SYN_CHECK(n_tokens > 0 && H > 0, "embed: empty input (%d tokens, width %d)", n_tokens, H);
+  if (table_is_f32)
+    embed_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)table, ids, resid, H);
+  else
+    embed_kernel<bf16><<<n_tokens, 256, 0, stream>>>((const bf16*)table, ids, resid, H);
+  SYN_LAUNCH_CHECK("embed");
+  return 0;
+}
+
+// ------------------------------------------------------------------ residual sum + RMSNorm
+// rows == nullptr: for every row r: resid[r] += delta[r] (if delta), out[r] = norm(resid[r]).
+// rows != nullptr: out[i] = norm(resid[rows[i]] + delta[rows[i]]); resid stays as it is.
+// The sum, the mean of squares and the scaling are 32-bit; one rounding at the store.
+template <typename TOut>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const float* __restrict__ delta,
+                                   const int* __restrict__ rows, const void* __restrict__ gain, int gain_is_f32,
+                                   float eps, TOut* __restrict__ out, int H) {
+  __shared__ float red[16];
+  const int r = rows ? rows[blockIdx.x] : blockIdx.x;
+  float* x = resid + (size_t)r * H;
+  const float* d = delta ? delta + (size_t)r * H : nullptr;
+  TOut* o = out + (size_t)blockIdx.x * H;
+  const bool write_back = (rows == nullptr) && (d != nullptr);
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = x[i];
+    if (d) v += d[i];
+    if (write_back) x[i] = v;
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float inv = rsqrtf(ss / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = x[i];
+    if (d && !write_back) v += d[i];
+    o[i] = from_f32<TOut>(load_gain(gain, gain_is_f32, i) * v * inv);
+  }
+}
+
+SYN_EXPORT int syn_add_rmsnorm(float* resid, const float* delta, const int* rows, int n_out, const void* gain,
+                               int gain_is_f32, float eps, void* out, int out_is_f32, int H, hipStream_t stream) {
+  SYN_CHECK(n_out > 0 && H > 0, "add_rmsnorm: empty input (%d rows, width %d)", n_out, H);
+  int block = H >= 4096 ? 1024 : (H >= 1024 ? 512 : 256);
+  if (out_is_f32)
+    add_rmsnorm_kernel<float><<<n_out, block, 0, stream>>>(resid, delta, rows, gain, gain_is_f32, eps, (float*)out, H);
+  else
+    add_rmsnorm_kernel<bf16><<<n_out, block, 0, stream>>>(resid, delta, rows, gain, gain_is_f32, eps, (bf16*)out, H);
+  SYN_LAUNCH_CHECK("add_rmsnorm");
+  return 0;
+}
+
+// ------------------------------------------------------------------ RMSNorm of rows of any width
+// One wave a row.
+template <typename T>
+__global__ void rmsnorm_rows_kernel(const T* __restrict__ x, const void* __restrict__ gain, int gain_is_f32, float eps,
+                                    T* __restrict__ out, int n_rows, int width) {
+  const int row = blockIdx.x * (blockDim.x / SYN_WAVE) + threadIdx.x / SYN_WAVE;
+  if (row >= n_rows) return;
+  const int lane = threadIdx.x % SYN_WAVE;
+  const T* xr = x + (size_t)row * width;
+  T* o = out + (size_t)row * width;
+  float ss = 0.f;
+  for (int i = lane; i < width; i += SYN_WAVE) {
+    float v = to_f32<T>(xr[i]);
+    ss += v * v;
+  }
+  ss = wave_sum(ss);
+  const float inv = rsqrtf(ss / (float)width + eps);
+  for (int i = lane; i < width; i += SYN_WAVE)
+    o[i] = from_f32<T>(load_gain(gain, gain_is_f32, i) * to_f32<T>(xr[i]) * inv);
+}
+
+SYN_EXPORT int syn_rmsnorm_rows(const void* x, int is_f32, const void* gain, int gain_is_f32, float eps, void* out,
+                                int n_rows, int width, hipStream_t stream) {
+  SYN_CHECK(n_rows > 0 && width > 0, "rmsnorm_rows: empty input (%d rows, width %d)", n_rows, width);
+  const int wpb = 4;
+  const int grid = (n_rows + wpb - 1) / wpb;
+  if (is_f32)
+    rmsnorm_rows_kernel<float><<<grid, wpb * SYN_WAVE, 0, stream>>>((const float*)x, gain, gain_is_f32, eps,
+                                                                    (float*)out, n_rows, width);
+  else
+    rmsnorm_rows_kernel<bf16><<<grid, wpb * SYN_WAVE, 0, stream>>>((const bf16*)x, gain, gain_is_f32, eps,
+                                                                   (bf16*)out, n_rows, width);
+  SYN_LAUNCH_CHECK("rmsnorm_rows");
+  return 0;
+}
+
+// ------------------------------------------------------------------ SwiGLU on a fused [gate | up] row
+// out[n, i] = silu(gu[n, i]) * gu[n, I + i], silu(z) = z / (1 + exp(-z)), in 32-bit.
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int n_rows, int I) {
+  const size_t total = (size_t)n_rows * I;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t n = idx / I;
+    const int i = (int)(idx - n * I);
+    const float g = to_f32<T>(gu[n * 2 * I + i]);
+    const float u = to_f32<T>(gu[n * 2 * I + I + i]);
+    out[idx] = from_f32<T>(g / (1.f + expf(-g)) * u);
+  }
+}
+
+SYN_EXPORT int syn_swiglu(const void* gu, void* out, int is_f32, int n_rows, int I, hipStream_t stream) {
+  SYN_CHECK(n_rows > 0 && I > 0, "swiglu: empty input (%d rows, width %d)", n_rows, I);
+  const size_t total = (size_t)n_rows * I;
+  int grid = (int)((total + 255) / 256);
+  if (grid > 65536) grid = 65536;
+  if (is_f32)
+    swiglu_kernel<float><<<grid, 256, 0, stream>>>((const float*)gu, (float*)out, n_rows, I);
+  else
+    swiglu_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, n_rows, I);
+  SYN_LAUNCH_CHECK("swiglu");
+  return 0;
+}
+
+// ------------------------------------------------------------------ q/k norm + rotation + cache write
+// One wave for each (token, head) of the fused projection row [q heads | k heads | v heads].
+//   q: optional RMSNorm over the head, rotation at the token's position, stored to q_out[token, head, :]
+//   k: the same, stored to the cache page of the token's sequence: k_pages[page, kv_head, pos % 64, :]
+//   v: copied as it is, stored transposed inside the page:          v_pages[page, kv_head, :, pos % 64]
+// Rotation (half-split layout over the first `rot` dims, the rest passes through):
+//   d < rot/2:        o[d] = x[d] cos[p, d]         - x[d + rot/2] sin[p, d]
+//   rot/2 <= d < rot: o[d] = x[d] cos[p, d - rot/2] + x[d - rot/2] sin[p, d - rot/2]
+// All arithmetic is 32-bit; each value is rounded once when stored.
+template <typename T>
+__global__ void qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_pages,
+                                             T* __restrict__ v_pages, const int* __restrict__ page_table,
+                                             int table_stride, const int* __restrict__ tok_seq,
+                                             const int* __restrict__ tok_pos, const void* __restrict__ q_gain,
+                                             const void* __restrict__ k_gain, int gain_is_f32, float eps,
+                                             const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
+                                             int nh, int nkv, int hd, int write_kv) {
+  extern __shared__ float lds[];  // [waves][hd]
+  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
+  const int heads = nh + 2 * nkv;
+  const int tok = blockIdx.x;
+  const int head = blockIdx.y * (blockDim.x / SYN_WAVE) + wave;
+  // no early return: every wave reaches the barrier; a layer that reads another layer's cache
+  // (write_kv == 0) only needs its q heads
+  const bool active = head < (write_kv ? heads : nh);
+  float* xs = lds + wave * hd;
+  const int pos = tok_pos[tok];
+  const bool is_q = head < nh, is_k = !is_q && head < nh + nkv;
+  const void* gain = is_q ? q_gain : (is_k ? k_gain : nullptr);
+
+  if (active) {
+    const T* src = qkv + ((size_t)tok * heads + head) * hd;
+    float ss = 0.f;
+    for (int d = lane; d < hd; d += SYN_WAVE) {
+      const float v = to_f32<T>(src[d]);
+      xs[d] = v;
+      ss += v * v;
+    }
+    if (gain) {
+      ss = wave_sum(ss);
+      const float inv = rsqrtf(ss / (float)hd + eps);
+      for (int d = lane; d < hd; d += SYN_WAVE) xs[d] = load_gain(gain, gain_is_f32, d) * xs[d] * inv;
+    }
+  }
+  __syncthreads();  // lanes read what other lanes of their wave wrote
+  if (!active) return;
+
+  T* dst;
+  size_t dst_stride = 1;
+  if (is_q) {
+    dst = q_out + ((size_t)tok * nh + head) * hd;
+  } else {
+    const int kvh = is_k ? head - nh : head - nh - nkv;
+    const int page = page_table[(size_t)tok_seq[tok] * table_stride + pos / SYN_PAGE];
+    const size_t base = ((size_t)page * nkv + kvh) * SYN_PAGE * hd;
+    if (is_k) {
+      dst = k_pages + base + (size_t)(pos % SYN_PAGE) * hd;
+    } else {
+      dst = v_pages + base + (pos % SYN_PAGE);
+      dst_stride = SYN_PAGE;
+    }
+  }
+  const bool rotate = (is_q || is_k) && cos_t != nullptr;
+  const int half = rot / 2;
+  for (int d = lane; d < hd; d += SYN_WAVE) {
+    float o = xs[d];
+    if (rotate && d < rot) {
+      if (d < half) {
+        const float c = cos_t[(size_t)pos * half + d], s = sin_t[(size_t)pos * half + d];
+        o = xs[d] * c - xs[d + half] * s;
+      } else {
+        const float c = cos_t[(size_t)pos * half + d - half], s = sin_t[(size_t)pos * half + d - half];
+        o = xs[d] * c + xs[d - half] * s;
+      }
+    }
+    dst[(size_t)d * dst_stride] = from_f32<T>(o);
+  }
+}
+
+SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, void* q_out, void* k_pages, void* v_pages, int is_f32,
+                                         const int* page_table, int table_stride, const int* tok_seq,
+                                         const int* tok_pos, const void* q_gain, const void* k_gain, int gain_is_f32,
+                                         float eps, const float* cos_t, const float* sin_t, int rot, int n_tokens,
+                                         int nh, int nkv, int hd, int write_kv, hipStream_t stream) {
+  SYN_CHECK(n_tokens > 0 && nh > 0 && nkv > 0 && hd > 0, "qk_norm_rope_kv_write: empty input");
+  SYN_CHECK(rot % 2 == 0 && rot >= 0 && rot <= hd, "qk_norm_rope_kv_write: rotary size %d does not fit head size %d",
+            rot, hd);
+  SYN_CHECK((cos_t == nullptr) == (sin_t == nullptr), "qk_norm_rope_kv_write: cos and sin come together");
+  const int wpb = 4;
+  const int heads = nh + 2 * nkv;
+  dim3 grid(n_tokens, (heads + wpb - 1) / wpb);
+  const size_t lds = (size_t)wpb * hd * sizeof(float);
+  if (is_f32)
+    qk_norm_rope_kv_write_kernel<float><<<grid, wpb * SYN_WAVE, lds, stream>>>(
+        (const float*)qkv, (float*)q_out, (float*)k_pages, (float*)v_pages, page_table, table_stride, tok_seq,
+        tok_pos, q_gain, k_gain, gain_is_f32, eps, cos_t, sin_t, rot, nh, nkv, hd, write_kv);
+  else
+    qk_norm_rope_kv_write_kernel<bf16><<<grid, wpb * SYN_WAVE, lds, stream>>>(
+        (const bf16*)qkv, (bf16*)q_out, (bf16*)k_pages, (bf16*)v_pages, page_table, table_stride, tok_seq, tok_pos,
+        q_gain, k_gain, gain_is_f32, eps, cos_t, sin_t, rot, nh, nkv, hd, write_kv);
+  SYN_LAUNCH_CHECK("qk_norm_rope_kv_write");
+  return 0;
+}

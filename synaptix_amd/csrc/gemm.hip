@@ -1,0 +1,268 @@
+// out[M, N] = x[M, K] . W[N, K]^T with 32-bit accumulation (both operands K-contiguous).
+//
+//   gemm_simt      any shape and type; plain FMA.  The whole 32-bit path, and bf16 shapes that
+//                  the MFMA kernels refuse (K not a multiple of 8, unaligned rows).
+//   gemm_skinny    bf16, M <= 64: the weight matrix is streamed once from HBM through
+//                  v_mfma_f32_16x16x32_bf16; the waves of a workgroup split K and sum in LDS.
+//   gemm_tiled     bf16, M > 64: 128x128x32 tiles in LDS, 2x2 waves of 64x64,
+//                  v_mfma_f32_32x32x16_bf16.
+//
+// Reference counterparts: crates/synaptix-kernels-cuda/src/best_cu/gemm/gemm_bf16.cu (TN family,
+// mma.sync m16n8k16), best_cu/gemv/mma_gemv.cu:19-133 (M == 1), best_cu/gemm/gemm_f32.cu (SIMT).
+// The tilings here are made for 64-lane waves and MFMA operand layouts, not translated.
+#include "common.h"
+
+// ------------------------------------------------------------------ SIMT, any type
+#define SIMT_BM 64
+#define SIMT_BN 64
+#define SIMT_BK 16
+
+template <typename TIn, typename TOut>
+__global__ void __launch_bounds__(256)
+gemm_simt_kernel(const TIn* __restrict__ x, const TIn* __restrict__ w, TOut* __restrict__ out, int M, int N, int K) {
+  __shared__ float xs[SIMT_BK][SIMT_BM + 1];
+  __shared__ float ws[SIMT_BK][SIMT_BN + 1];
+  const int tid = threadIdx.x;
+  const int m0 = blockIdx.y * SIMT_BM, n0 = blockIdx.x * SIMT_BN;
+  const int tm = (tid / 16) * 4, tn = (tid % 16) * 4;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += SIMT_BK) {
+    // 64 rows x 16 k for each operand: 1024 values, 4 a thread
+    for (int e = tid; e < SIMT_BM * SIMT_BK; e += 256) {
+      const int r = e / SIMT_BK, kk = e % SIMT_BK;
+      const int gm = m0 + r, gn = n0 + r, gk = k0 + kk;
+      xs[kk][r] = (gm < M && gk < K) ? to_f32<TIn>(x[(size_t)gm * K + gk]) : 0.f;
+      ws[kk][r] = (gn < N && gk < K) ? to_f32<TIn>(w[(size_t)gn * K + gk]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < SIMT_BK; ++kk) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = xs[kk][tm + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = ws[kk][tn + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int gm = m0 + tm + i, gn = n0 + tn + j;
+      if (gm < M && gn < N) out[(size_t)gm * N + gn] = from_f32<TOut>(acc[i][j]);
+    }
+}
+
+// ------------------------------------------------------------------ skinny, bf16, M <= 64
+// MFMA 16x16x32: A = x rows (m), B = W rows (n), D[m = 4*(lane/16)+j][n = lane%16].
+// Both operands: lane holds row lane%16, k = 8*(lane/16) .. +8, one 16-byte load.
+// A workgroup owns RT*16 rows of W; its WAVES waves take k-chunks of 32 round-robin, so that at
+// any moment the workgroup reads WAVES*64 contiguous bytes of each row.
+template <int MB, int RT, int WAVES>
+__global__ void __launch_bounds__(WAVES * SYN_WAVE)
+gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
+                   int M, int N, int K) {
+  extern __shared__ float part[];  // [WAVES][MB*RT*4][64]
+  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
+  const int r16 = lane % 16, kq = (lane / 16) * 8;
+  const int n0 = blockIdx.x * (RT * 16);
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  const bf16* wrow[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) wrow[r] = w + (size_t)min(n0 + r * 16 + r16, N - 1) * K;
+  const bf16* xrow[MB];
+  bool xok[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) {
+    xok[b] = b * 16 + r16 < M;
+    xrow[b] = x + (size_t)min(b * 16 + r16, M - 1) * K;
+  }
+  f32x4 acc[MB][RT];
+#pragma unroll
+  for (int b = 0; b < MB; ++b)
+#pragma unroll
+    for (int r = 0; r < RT; ++r) acc[b][r] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  for (int k0 = wave * 32; k0 < K; k0 += WAVES * 32) {
+    const int k = k0 + kq;
+    const bool kin = k < K;  // K is a multiple of 8: a chunk of 8 lies inside or outside as a whole
+    bf16x8 bw[RT], ax[MB];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) bw[r] = kin ? *(const bf16x8*)(wrow[r] + k) : zero;
+#pragma unroll
+    for (int b = 0; b < MB; ++b) ax[b] = (kin && xok[b]) ? *(const bf16x8*)(xrow[b] + k) : zero;
+#pragma unroll
+    for (int b = 0; b < MB; ++b)
+#pragma unroll
+      for (int r = 0; r < RT; ++r) acc[b][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[b], bw[r], acc[b][r], 0, 0, 0);
+  }
+
+  // sum the waves' partial tiles in a fixed order
+  constexpr int SLOTS = MB * RT * 4;
+#pragma unroll
+  for (int b = 0; b < MB; ++b)
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) part[((size_t)wave * SLOTS + (b * RT + r) * 4 + j) * 64 + lane] = acc[b][r][j];
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < SLOTS * 64; idx += WAVES * SYN_WAVE) {
+    float s = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv) s += part[(size_t)wv * SLOTS * 64 + idx];
+    const int slot = idx / 64, ln = idx % 64;
+    const int j = slot % 4, r = (slot / 4) % RT, b = slot / (4 * RT);
+    const int m = b * 16 + 4 * (ln / 16) + j, n = n0 + r * 16 + ln % 16;
+    if (m < M && n < N) {
+      if (out_is_f32)
+        ((float*)out)[(size_t)m * N + n] = s;
+      else
+        ((bf16*)out)[(size_t)m * N + n] = (bf16)s;
+    }
+  }
+}
+
+template <int MB, int RT, int WAVES>
+static void launch_skinny(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
+                          hipStream_t stream) {
+  const int grid = (N + RT * 16 - 1) / (RT * 16);
+  const size_t lds = (size_t)WAVES * MB * RT * 4 * 64 * sizeof(float);
+  gemm_skinny_kernel<MB, RT, WAVES><<<grid, WAVES * SYN_WAVE, lds, stream>>>(x, w, out, out_is_f32, M, N, K);
+}
+
+// ------------------------------------------------------------------ tiled, bf16, large M
+// Block tile 128 (m) x 128 (n) x 32 (k); 4 waves as 2x2, each 64x64 = 2x2 MFMA 32x32x16 tiles.
+// MFMA 32x32x16: A = x rows, B = W rows; lane holds row lane%32, k = 8*(lane/32) .. +8;
+// D[m = 8*(j/4) + 4*(lane/32) + j%4][n = lane%32], j = 0..15.
+#define TG_BM 128
+#define TG_BN 128
+#define TG_BK 32
+#define TG_LD (TG_BK + 8)  // padded row of the LDS tiles, in bf16 elements (80 bytes)
+
+__global__ void __launch_bounds__(256)
+gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
+                  int M, int N, int K) {
+  __shared__ __attribute__((aligned(16))) bf16 xs[2][TG_BM * TG_LD];
+  __shared__ __attribute__((aligned(16))) bf16 ws[2][TG_BN * TG_LD];
+  const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE;
+  const int wm = (wave / 2) * 64, wn = (wave % 2) * 64;
+  const int m0 = blockIdx.y * TG_BM, n0 = blockIdx.x * TG_BN;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  // global -> LDS: each tile is 128 rows x 4 chunks of 8; 512 chunks, 2 a thread
+  const int lrow = tid / 4, lchunk = (tid % 4) * 8;  // rows lrow and lrow + 64
+  const bf16* xg0 = x + (size_t)min(m0 + lrow, M - 1) * K + lchunk;
+  const bf16* xg1 = x + (size_t)min(m0 + lrow + 64, M - 1) * K + lchunk;
+  const bf16* wg0 = w + (size_t)min(n0 + lrow, N - 1) * K + lchunk;
+  const bf16* wg1 = w + (size_t)min(n0 + lrow + 64, N - 1) * K + lchunk;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const int nk = (K + TG_BK - 1) / TG_BK;
+  bf16x8 rx0, rx1, rw0, rw1;
+  auto fetch = [&](int kt) {
+    const int k = kt * TG_BK + lchunk;
+    const bool kin = k < K;
+    rx0 = kin ? *(const bf16x8*)(xg0 + (size_t)kt * TG_BK) : zero;
+    rx1 = kin ? *(const bf16x8*)(xg1 + (size_t)kt * TG_BK) : zero;
+    rw0 = kin ? *(const bf16x8*)(wg0 + (size_t)kt * TG_BK) : zero;
+    rw1 = kin ? *(const bf16x8*)(wg1 + (size_t)kt * TG_BK) : zero;
+  };
+  auto stash = [&](int buf) {
+    *(bf16x8*)(&xs[buf][lrow * TG_LD + lchunk]) = rx0;
+    *(bf16x8*)(&xs[buf][(lrow + 64) * TG_LD + lchunk]) = rx1;
+    *(bf16x8*)(&ws[buf][lrow * TG_LD + lchunk]) = rw0;
+    *(bf16x8*)(&ws[buf][(lrow + 64) * TG_LD + lchunk]) = rw1;
+  };
+
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  const int fr = lane % 32, fk = (lane / 32) * 8;
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < nk) fetch(kt + 1);
+#pragma unroll
+    for (int ks = 0; ks < TG_BK; ks += 16) {
+      bf16x8 a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) a[i] = *(const bf16x8*)(&xs[buf][(wm + i * 32 + fr) * TG_LD + ks + fk]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) b[j] = *(const bf16x8*)(&ws[buf][(wn + j * 32 + fr) * TG_LD + ks + fk]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < nk) stash(buf ^ 1);  // the other buffer was last read before the previous barrier
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = m0 + wm + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+        const int n = n0 + wn + j * 32 + lane % 32;
+        if (m < M && n < N) {
+          if (out_is_f32)
+            ((float*)out)[(size_t)m * N + n] = acc[i][j][e];
+          else
+            ((bf16*)out)[(size_t)m * N + n] = (bf16)acc[i][j][e];
+        }
+      }
+}
+
+// ------------------------------------------------------------------ entry point
+// dtype: 0 = float in, float out; 1 = bf16 in, bf16 out; 2 = bf16 in, float out.
+SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int M, int N, int K, int force_simt,
+                        hipStream_t stream) {
+  SYN_CHECK(M > 0 && N > 0 && K > 0, "gemm: empty shape M=%d N=%d K=%d", M, N, K);
+  SYN_CHECK(dtype >= 0 && dtype <= 2, "gemm: unknown dtype code %d", dtype);
+  const dim3 simt_grid((N + SIMT_BN - 1) / SIMT_BN, (M + SIMT_BM - 1) / SIMT_BM);
+  if (dtype == 0) {
+    gemm_simt_kernel<float, float><<<simt_grid, 256, 0, stream>>>((const float*)x, (const float*)w, (float*)out, M, N, K);
+    SYN_LAUNCH_CHECK("gemm_simt");
+    return 0;
+  }
+  const int out_is_f32 = dtype == 2;
+  const bool aligned = (K % 8 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
+  if (force_simt || !aligned) {
+    if (out_is_f32)
+      gemm_simt_kernel<bf16, float><<<simt_grid, 256, 0, stream>>>((const bf16*)x, (const bf16*)w, (float*)out, M, N, K);
+    else
+      gemm_simt_kernel<bf16, bf16><<<simt_grid, 256, 0, stream>>>((const bf16*)x, (const bf16*)w, (bf16*)out, M, N, K);
+    SYN_LAUNCH_CHECK("gemm_simt");
+    return 0;
+  }
+  const bf16* xb = (const bf16*)x;
+  const bf16* wb = (const bf16*)w;
+  if (M <= 16) {
+    launch_skinny<1, 1, 8>(xb, wb, out, out_is_f32, M, N, K, stream);
+  } else if (M <= 32) {
+    launch_skinny<2, 2, 8>(xb, wb, out, out_is_f32, M, N, K, stream);
+  } else if (M <= 48) {
+    launch_skinny<3, 2, 8>(xb, wb, out, out_is_f32, M, N, K, stream);
+  } else if (M <= 64) {
+    launch_skinny<4, 2, 8>(xb, wb, out, out_is_f32, M, N, K, stream);
+  } else {
+    const dim3 grid((N + TG_BN - 1) / TG_BN, (M + TG_BM - 1) / TG_BM);
+    gemm_tiled_kernel<<<grid, 256, 0, stream>>>(xb, wb, out, out_is_f32, M, N, K);
+  }
+  SYN_LAUNCH_CHECK("gemm");
+  return 0;
+}

@@ -1,0 +1,189 @@
+"""The engine: a model on the GPU, its cache, and one step function.
+
+`step` runs only the tokens it is given, as one packed batch, from the cache that earlier
+steps left, and returns the logits at the wanted places.  Prompts of unequal lengths go in one
+step; later steps bring one token for each sequence that is still alive.  Nothing is padded,
+so a sequence's results cannot depend on its neighbours beyond the rounding of reductions.
+
+The reference's forward takes [B, S] ids with one shared length
+(crates/synaptix-models/llm/common/src/model.rs:1107-1117,1169-1172); unequal lengths, slots and
+their reuse are this engine's own.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from ..cache import SequenceCache, CacheFull, CacheError, PAGE_TOKENS, pages_for
+from ..config.registry import load_config, resolve_architecture
+from ..kernels import ops
+from ..weights import FolderSource, RandomSource, load_weights
+from .batch import StepLayout, StepContext, fill_host_buffer
+
+assert ops.PAGE_TOKENS == PAGE_TOKENS
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "f32": torch.float32,
+           torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
+
+
+class StepError(ValueError):
+    """A step that cannot be run: bad token id, unknown slot, empty entry, ..."""
+
+
+def parse_dtype(dtype) -> torch.dtype:
+    if dtype not in _DTYPES:
+        raise ValueError(f"dtype {dtype!r}: expected bfloat16 or float32")
+    return _DTYPES[dtype]
+
+
+class Engine:
+    def __init__(self, model, dtype, max_tokens: int, max_slots: int | None = None):
+        """`model` has its weights loaded on a GPU."""
+        self.model = model
+        self.dtype = parse_dtype(dtype)
+        self.device = model.device
+        self._require_gpu()
+        self.vocab = model.vocab
+        max_positions = getattr(model.config, "max_position_embeddings", None)
+        for b in model.blocks:
+            cap = getattr(getattr(b.mixer, "position", None), "capacity", None)
+            if cap is not None:
+                max_positions = cap if max_positions is None else min(max_positions, cap)
+        self.max_positions = max_positions
+        self.cache = SequenceCache(model.cache_needs(), max_tokens, max_slots, self.dtype, self.device,
+                                   max_positions=max_positions)
+        self._scratch = {}
+        self._host = None
+        self._dev = None
+
+    # ------------------------------------------------------------------ construction
+    @classmethod
+    def load(cls, folder: str, dtype="bfloat16", max_tokens: int = 8192, max_slots: int | None = None,
+             max_seq: int | None = None, device="cuda:0", strict: bool = True) -> "Engine":
+        """A model folder (config.json + safetensors); the model class is chosen by config.json."""
+        arch, cfg = load_config(folder)
+        model = arch.build(cfg, max_positions=max_seq)
+        load_weights(model, FolderSource(folder), parse_dtype(dtype), device, strict=strict)
+        return cls(model, dtype, max_tokens, max_slots)
+
+    @classmethod
+    def from_config(cls, config, seed: int = 0, dtype="bfloat16", max_tokens: int = 8192,
+                    max_slots: int | None = None, max_seq: int | None = None, device="cuda:0") -> "Engine":
+        """Random weights drawn on the device (for measurements; no files are written)."""
+        arch = resolve_architecture(config.to_dict())
+        model = arch.build(config, max_positions=max_seq)
+        dt = parse_dtype(dtype)
+        src = RandomSource(model.tensor_specs(), seed, store_dtype=dt, device=device)
+        load_weights(model, src, dt, device)
+        return cls(model, dtype, max_tokens, max_slots)
+
+    # ------------------------------------------------------------------ slots
+    def acquire(self) -> int:
+        return self.cache.acquire()
+
+    def release(self, slot: int) -> None:
+        self.cache.release(slot)
+
+    def length(self, slot: int) -> int:
+        return self.cache.length(slot)
+
+    # ------------------------------------------------------------------ the step
+    def _require_gpu(self):
+        if self.device is None or self.device.type != "cuda":
+            raise RuntimeError("the engine runs on the GPU only; load the model's weights on a cuda device")
+
+    _RING = 4
+
+    def _buffers(self, total: int):
+        """A pinned host buffer whose last copy has left, and the device buffer of the step."""
+        if self._host is None or self._host[0].numel() < total:
+            n = max(2 * total, 4096)
+            self._host = [torch.empty(n, dtype=torch.int32, pin_memory=True) for _ in range(self._RING)]
+            self._dev = [torch.empty(n, dtype=torch.int32, device=self.device) for _ in range(self._RING)]
+            self._copied = [None] * self._RING
+            self._turn = 0
+        i = self._turn
+        self._turn = (i + 1) % self._RING
+        if self._copied[i] is not None:
+            self._copied[i].synchronize()
+        return i, self._host[i], self._dev[i]
+
+    def prepare(self, entries, want) -> tuple:
+        """Check a step, hold its pages, and write its arrays to the device.  Returns (ctx, n_want)."""
+        if not entries:
+            raise StepError("a step needs at least one sequence")
+        slots = [e[0] for e in entries]
+        token_lists = [np.asarray(e[1], dtype=np.int64).reshape(-1) for e in entries]
+        if len(set(slots)) != len(slots):
+            raise StepError("a slot appears twice in one step")
+        past = []
+        for sid, toks in zip(slots, token_lists):
+            past.append(self.cache.length(sid))          # raises CacheError for an unknown slot
+            if toks.size == 0:
+                raise StepError(f"slot {sid}: a step brings at least one token for each of its sequences")
+            if toks.min() < 0 or toks.max() >= self.vocab:
+                raise StepError(f"slot {sid}: token id outside the vocabulary [0, {self.vocab})")
+            if self.max_positions is not None and past[-1] + toks.size > self.max_positions:
+                raise CacheError(f"KV overflow: slot {sid} holds {past[-1]} tokens, {toks.size} more exceed "
+                                 f"the position range {self.max_positions}")
+        starts = np.concatenate([[0], np.cumsum([t.size for t in token_lists])])
+        if want is None:
+            want_rows = []
+        elif isinstance(want, str) and want == "last":
+            want_rows = [int(starts[i + 1]) - 1 for i in range(len(entries))]
+        elif isinstance(want, str) and want == "all":
+            want_rows = list(range(int(starts[-1])))
+        else:
+            if len(want) != len(entries):
+                raise StepError("`want` needs one list of places for each sequence of the step")
+            want_rows = []
+            for i, places in enumerate(want):
+                for p in places:
+                    if not (0 <= p < token_lists[i].size):
+                        raise StepError(f"slot {slots[i]}: wanted place {p} is outside its {token_lists[i].size} tokens")
+                    want_rows.append(int(starts[i]) + int(p))
+        # all pages of the step, or none
+        need = sum(self.cache.pages_needed(s, t.size) for s, t in zip(slots, token_lists))
+        for g in self.cache.groups:
+            if g.pool.free_pages < need:
+                raise CacheFull(f"the step needs {need} more pages, {g.pool.free_pages} of {g.pool.n_pages} are free")
+        for s, t in zip(slots, token_lists):
+            self.cache.reserve(s, t.size)
+
+        tables = [self.cache.page_table(gi, slots) for gi in range(len(self.cache.groups))]
+        layout = StepLayout(int(starts[-1]), len(entries), len(want_rows), [t.shape[1] for t in tables])
+        dev = self._upload(layout, token_lists, past, slots, want_rows, tables)
+        ctx = StepContext(layout, dev, self.dtype, slots, past, [t.size for t in token_lists], self._scratch)
+        return ctx, len(want_rows)
+
+    def _upload(self, layout, token_lists, past, slots, want_rows, tables) -> torch.Tensor:
+        """The step's arrays on the device, through a pinned buffer and one asynchronous copy."""
+        i, host, dev = self._buffers(layout.total)
+        fill_host_buffer(layout, host.numpy(), token_lists, past, slots, want_rows, tables)
+        dev[:layout.total].copy_(host[:layout.total], non_blocking=True)
+        self._copied[i] = torch.cuda.Event()
+        self._copied[i].record()
+        return dev
+
+    def step(self, entries, want="last") -> torch.Tensor:
+        """entries: [(slot, tokens), ...]; want: "last", "all", None or a list of places for each
+        entry.  Returns float logits [wanted, vocab] on the device, in the order of the entries and
+        of their places."""
+        ctx, n_want = self.prepare(entries, want)
+        with torch.no_grad():
+            logits = self.model.forward(ctx, ctx.tokens, ctx.want if n_want else None, self.cache)
+        for s, n in zip(ctx.slots, ctx.new_counts):
+            self.cache.commit(s, n)
+        if logits is None:
+            logits = torch.empty((0, self.vocab), dtype=torch.float32, device=self.device)
+        return logits
+
+    def sample(self, logits, temperatures=None, uniforms=None) -> torch.Tensor:
+        """Token ids (int32, device) for rows of logits; see kernels.ops.sample_rows."""
+        out = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device)
+        t = u = None
+        if temperatures is not None:
+            t = torch.as_tensor(temperatures, dtype=torch.float32).to(logits.device)
+            u = torch.as_tensor(uniforms, dtype=torch.float32).to(logits.device)
+        ops.sample_rows(logits, t, u, out)
+        return out

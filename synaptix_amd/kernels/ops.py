@@ -1,0 +1,249 @@
+"""The kernels as Python functions over torch tensors on the GPU.
+
+Every function checks on the host that shapes, types and layouts are what its kernel and grid
+assume, then launches on torch's current stream.  There is no other implementation behind
+these names: without the built library, or with tensors that are not on the GPU, they raise.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from .build import load_library
+
+PAGE_TOKENS = 64          # tokens in a cache page; the kernels are compiled with the same number
+MAX_HEAD_DIM = 256
+_F32, _BF16, _I32 = torch.float32, torch.bfloat16, torch.int32
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(0) if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _need(t, name, dtypes, shape=None):
+    if not isinstance(t, torch.Tensor):
+        raise KernelError(f"{name}: expected a tensor, got {type(t).__name__}")
+    if t.device.type != "cuda":
+        raise KernelError(f"{name}: tensor lies on {t.device}; the kernels of synaptix_amd run on the GPU only")
+    if not isinstance(dtypes, (tuple, list)):
+        dtypes = (dtypes,)
+    if t.dtype not in dtypes:
+        raise KernelError(f"{name}: dtype {t.dtype}, expected {' or '.join(str(d) for d in dtypes)}")
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: tensor is not contiguous")
+    if shape is not None:
+        if len(shape) != t.dim() or any(s is not None and s != g for s, g in zip(shape, t.shape)):
+            raise KernelError(f"{name}: shape {list(t.shape)}, expected {[('*' if s is None else s) for s in shape]}")
+
+
+def _call(lib, fn, *args):
+    rc = getattr(lib, fn)(*args)
+    if rc != 0:
+        raise KernelError(lib.syn_last_error().decode(errors="replace"))
+
+
+def _is_f32(t):
+    return 1 if t.dtype == _F32 else 0
+
+
+# ----------------------------------------------------------------------------- rows
+
+def embed(table, ids, resid):
+    """resid[n, :] = table[ids[n], :] as float.  table [V, H] bf16|f32, ids [N] int32, resid [N, H] f32."""
+    _need(table, "embed.table", (_BF16, _F32), (None, None))
+    V, H = table.shape
+    _need(ids, "embed.ids", _I32, (None,))
+    _need(resid, "embed.resid", _F32, (ids.shape[0], H))
+    _call(load_library("core"), "syn_embed", _ptr(table), _is_f32(table), _ptr(ids), _ptr(resid),
+          ids.shape[0], H, _stream())
+
+
+def add_rmsnorm(resid, delta, gain, eps, out, rows=None):
+    """rows is None:  resid += delta (when given), out = RMSNorm(resid) * gain, for every row.
+    rows [n] int32: out[i] = RMSNorm(resid[rows[i]] + delta[rows[i]]) * gain; resid is not written."""
+    _need(resid, "add_rmsnorm.resid", _F32, (None, None))
+    N, H = resid.shape
+    if delta is not None:
+        _need(delta, "add_rmsnorm.delta", _F32, (N, H))
+    _need(gain, "add_rmsnorm.gain", (_BF16, _F32), (H,))
+    n_out = N
+    if rows is not None:
+        _need(rows, "add_rmsnorm.rows", _I32, (None,))
+        n_out = rows.shape[0]
+    _need(out, "add_rmsnorm.out", (_BF16, _F32), (n_out, H))
+    _call(load_library("core"), "syn_add_rmsnorm", _ptr(resid), _ptr(delta), _ptr(rows), n_out, _ptr(gain),
+          _is_f32(gain), ctypes.c_float(eps), _ptr(out), _is_f32(out), H, _stream())
+
+
+def rmsnorm_rows(x, gain, eps, out):
+    """out = RMSNorm(x) * gain over the last axis; x [..., D] bf16|f32, out like x."""
+    _need(x, "rmsnorm_rows.x", (_BF16, _F32))
+    D = x.shape[-1]
+    _need(gain, "rmsnorm_rows.gain", (_BF16, _F32), (D,))
+    _need(out, "rmsnorm_rows.out", x.dtype, tuple(x.shape))
+    _call(load_library("core"), "syn_rmsnorm_rows", _ptr(x), _is_f32(x), _ptr(gain), _is_f32(gain),
+          ctypes.c_float(eps), _ptr(out), x.numel() // D, D, _stream())
+
+
+def swiglu(gate_up, out):
+    """out[n, i] = silu(gate_up[n, i]) * gate_up[n, I + i]."""
+    _need(gate_up, "swiglu.gate_up", (_BF16, _F32), (None, None))
+    N, I2 = gate_up.shape
+    if I2 % 2:
+        raise KernelError(f"swiglu: fused width {I2} is odd")
+    _need(out, "swiglu.out", gate_up.dtype, (N, I2 // 2))
+    _call(load_library("core"), "syn_swiglu", _ptr(gate_up), _ptr(out), _is_f32(gate_up), N, I2 // 2, _stream())
+
+
+# ----------------------------------------------------------------------------- matrix product
+
+def gemm(x, w, out, force_simt=False):
+    """out[M, N] = x[M, K] . w[N, K]^T with 32-bit accumulation.
+    float x float -> float (plain FMA); bf16 x bf16 -> bf16 or float (MFMA)."""
+    _need(x, "gemm.x", (_BF16, _F32), (None, None))
+    M, K = x.shape
+    _need(w, "gemm.w", x.dtype, (None, K))
+    N = w.shape[0]
+    if x.dtype == _F32:
+        _need(out, "gemm.out", _F32, (M, N))
+        code = 0
+    else:
+        _need(out, "gemm.out", (_BF16, _F32), (M, N))
+        code = 2 if out.dtype == _F32 else 1
+    _call(load_library("core"), "syn_gemm", _ptr(x), _ptr(w), _ptr(out), code, M, N, K, 1 if force_simt else 0,
+          _stream())
+
+
+# ----------------------------------------------------------------------------- attention
+
+def _check_pages(k_pages, v_pages, dtype, nkv, hd, name):
+    _need(k_pages, name + ".k_pages", dtype, (None, nkv, PAGE_TOKENS, hd))
+    _need(v_pages, name + ".v_pages", dtype, (k_pages.shape[0], nkv, hd, PAGE_TOKENS))
+
+
+def qk_norm_rope_kv_write(qkv, q_out, k_pages, v_pages, page_table, tok_seq, tok_pos, q_gain, k_gain, eps,
+                          cos, sin, n_heads, n_kv_heads, head_dim, write_kv=True):
+    """Split a fused [q | k | v] projection row into heads; RMSNorm q and k heads (if gains are
+    given), rotate them at tok_pos (if tables are given; their width is rotary_dim / 2), write q to
+    q_out [N, nh*hd], k and v into the cache pages of sequence tok_seq[n] at position tok_pos[n]
+    (not with write_kv False: a layer that reads a cache which another layer writes)."""
+    nh, nkv, hd = n_heads, n_kv_heads, head_dim
+    _need(qkv, "qk_norm_rope_kv_write.qkv", (_BF16, _F32), (None, (nh + 2 * nkv) * hd))
+    N = qkv.shape[0]
+    _need(q_out, "qk_norm_rope_kv_write.q_out", qkv.dtype, (N, nh * hd))
+    _check_pages(k_pages, v_pages, qkv.dtype, nkv, hd, "qk_norm_rope_kv_write")
+    _need(page_table, "qk_norm_rope_kv_write.page_table", _I32, (None, None))
+    _need(tok_seq, "qk_norm_rope_kv_write.tok_seq", _I32, (N,))
+    _need(tok_pos, "qk_norm_rope_kv_write.tok_pos", _I32, (N,))
+    if hd > MAX_HEAD_DIM:
+        raise KernelError(f"qk_norm_rope_kv_write: head size {hd} exceeds {MAX_HEAD_DIM}")
+    gain_f32 = 0
+    if (q_gain is None) != (k_gain is None):
+        raise KernelError("qk_norm_rope_kv_write: q and k gains come together")
+    if q_gain is not None:
+        _need(q_gain, "qk_norm_rope_kv_write.q_gain", (_BF16, _F32), (hd,))
+        _need(k_gain, "qk_norm_rope_kv_write.k_gain", q_gain.dtype, (hd,))
+        gain_f32 = _is_f32(q_gain)
+    rot = 0
+    if cos is not None:
+        _need(cos, "qk_norm_rope_kv_write.cos", _F32, (None, None))
+        _need(sin, "qk_norm_rope_kv_write.sin", _F32, tuple(cos.shape))
+        rot = 2 * cos.shape[1]
+        if rot > hd:
+            raise KernelError(f"qk_norm_rope_kv_write: rotary size {rot} exceeds head size {hd}")
+    _call(load_library("core"), "syn_qk_norm_rope_kv_write", _ptr(qkv), _ptr(q_out), _ptr(k_pages), _ptr(v_pages),
+          _is_f32(qkv), _ptr(page_table), page_table.shape[1], _ptr(tok_seq), _ptr(tok_pos), _ptr(q_gain), _ptr(k_gain),
+          gain_f32, ctypes.c_float(eps), _ptr(cos), _ptr(sin), rot, N, nh, nkv, hd, 1 if write_kv else 0, _stream())
+
+
+def attention_f32(q, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale, window, n_heads, n_kv_heads,
+                  head_dim):
+    """True 32-bit attention of every token (prefill and decode alike)."""
+    nh, nkv, hd = n_heads, n_kv_heads, head_dim
+    _need(q, "attention_f32.q", _F32, (None, nh * hd))
+    N = q.shape[0]
+    _check_pages(k_pages, v_pages, _F32, nkv, hd, "attention_f32")
+    _need(page_table, "attention_f32.page_table", _I32, (None, None))
+    _need(tok_seq, "attention_f32.tok_seq", _I32, (N,))
+    _need(tok_pos, "attention_f32.tok_pos", _I32, (N,))
+    _need(out, "attention_f32.out", _F32, (N, nh * hd))
+    _call(load_library("core"), "syn_attention_f32", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
+          page_table.shape[1], _ptr(tok_seq), _ptr(tok_pos), _ptr(out), ctypes.c_float(scale), int(window or 0),
+          N, nh, nkv, hd, _stream())
+
+
+def _attn_lib(hd):
+    if hd % 16 != 0 or not (16 <= hd <= MAX_HEAD_DIM):
+        raise KernelError(f"bf16 attention: head size {hd} is not one of 16, 32, ..., {MAX_HEAD_DIM}")
+    return load_library(f"attn_hd{hd}")
+
+
+def attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, seq_past, out, scale, window, n_heads,
+                           n_kv_heads, head_dim):
+    """Causal attention of the new tokens of each sequence over its cache (which already holds them).
+    seq_start [B+1]: offsets of the sequences' new tokens in q; seq_past [B]: tokens cached before."""
+    nh, nkv, hd = n_heads, n_kv_heads, head_dim
+    _need(q, "attention_prefill.q", _BF16, (None, nh * hd))
+    N = q.shape[0]
+    _check_pages(k_pages, v_pages, _BF16, nkv, hd, "attention_prefill")
+    _need(page_table, "attention_prefill.page_table", _I32, (None, None))
+    _need(seq_start, "attention_prefill.seq_start", _I32, (None,))
+    B = seq_start.shape[0] - 1
+    _need(seq_past, "attention_prefill.seq_past", _I32, (B,))
+    if page_table.shape[0] < B:
+        raise KernelError(f"attention_prefill: page table has {page_table.shape[0]} rows for {B} sequences")
+    _need(out, "attention_prefill.out", _BF16, (N, nh * hd))
+    _call(_attn_lib(hd), "syn_attention_prefill_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
+          page_table.shape[1], _ptr(seq_start), _ptr(seq_past), B, N, _ptr(out), ctypes.c_float(scale),
+          int(window or 0), nh, nkv, hd, _stream())
+
+
+def decode_splits(n_seqs, n_kv_heads, max_pages):
+    """How many ways the keys of a sequence are split in decode: enough waves to fill the chip."""
+    want = max(1, 2048 // max(1, n_seqs * n_kv_heads))
+    return int(max(1, min(want, max_pages, 64)))
+
+
+def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
+                          n_heads, n_kv_heads, head_dim):
+    """One query for each sequence (its last token, already in the cache); seq_len [B] counts it.
+    workspace: float [B * nh * n_splits * (hd + 2)]."""
+    nh, nkv, hd = n_heads, n_kv_heads, head_dim
+    _need(q, "attention_decode.q", _BF16, (None, nh * hd))
+    B = q.shape[0]
+    _check_pages(k_pages, v_pages, _BF16, nkv, hd, "attention_decode")
+    _need(page_table, "attention_decode.page_table", _I32, (None, None))
+    if page_table.shape[0] < B:
+        raise KernelError(f"attention_decode: page table has {page_table.shape[0]} rows for {B} sequences")
+    _need(seq_len, "attention_decode.seq_len", _I32, (B,))
+    _need(out, "attention_decode.out", _BF16, (B, nh * hd))
+    _need(workspace, "attention_decode.workspace", _F32)
+    if workspace.numel() < B * nh * n_splits * (hd + 2):
+        raise KernelError(f"attention_decode: workspace of {workspace.numel()} floats is too small")
+    _call(_attn_lib(hd), "syn_attention_decode_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
+          page_table.shape[1], _ptr(seq_len), B, _ptr(out), _ptr(workspace), int(n_splits), ctypes.c_float(scale),
+          int(window or 0), nh, nkv, hd, _stream())
+
+
+# ----------------------------------------------------------------------------- sampling
+
+def sample_rows(logits, temperature, uniform, out):
+    """out[r] = argmax (last of equal maxima) where temperature[r] <= 0 or temperature is None,
+    else a draw from softmax(logits[r] / temperature[r]) by inverse CDF with uniform[r]."""
+    _need(logits, "sample_rows.logits", _F32, (None, None))
+    R, V = logits.shape
+    if temperature is not None:
+        _need(temperature, "sample_rows.temperature", _F32, (R,))
+        _need(uniform, "sample_rows.uniform", _F32, (R,))
+    _need(out, "sample_rows.out", _I32, (R,))
+    _call(load_library("core"), "syn_sample_rows", _ptr(logits), _ptr(temperature),
+          _ptr(uniform if temperature is not None else None), _ptr(out), R, V, _stream())

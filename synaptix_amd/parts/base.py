@@ -1,0 +1,39 @@
+"""What every part of a layer has in common.
+
+A part owns the names, shapes and storage of its tensors and the launches that compute it.
+It receives its sizes and constants as parameters and its tensor-name prefix as a string; it
+does not know which model it is in (the reference produces tensor names the same way, from
+the layer: crates/synaptix-models/llm/common/src/model.rs:780).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+
+class Part:
+    """Base of norms, position encodings, mixers, feed-forwards and blocks."""
+
+    def tensor_specs(self) -> dict:
+        """name -> TensorSpec of every tensor this part reads from the weight source."""
+        return {}
+
+    def load(self, get) -> None:
+        """Fetch the tensors; `get(name)` returns the tensor on the device in its kept type."""
+
+
+@dataclass(frozen=True)
+class KvNeed:
+    """A mixer that keeps keys and values of the tokens it has seen: all of them, or a window."""
+    kv_heads: int
+    head_dim: int
+    window: Optional[int] = None      # None: all keys
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """A mixer that keeps a state of fixed size for each sequence, zero when the sequence starts."""
+    shape: tuple
+    dtype: torch.dtype = torch.float32

@@ -1,0 +1,47 @@
+"""Feed-forward parts.  Here: the gated MLP  down( act(gate(h)) * up(h) ), dense.
+
+crates/synaptix-models/llm/common/src/model.rs:1670-1691; activation silu(z) = z / (1 + e^-z) in
+32-bit as crates/synaptix-kernels-cuda/src/cu/fused/mlp/silu_and_mul.cu:11-52.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..weights.source import TensorSpec
+from .base import Part
+from .linear import linear
+
+
+class FeedForward(Part):
+    """Interface: forward(h [N, hidden] activation type, ctx) -> residual delta [N, hidden] float."""
+
+    def forward(self, h, ctx):
+        raise NotImplementedError
+
+
+class GatedMlp(FeedForward):
+    def __init__(self, prefix: str, hidden: int, intermediate: int, activation: str = "silu"):
+        if activation not in ("silu", "swish"):
+            raise ValueError(f"activation {activation!r} is not built (silu only)")
+        self.prefix, self.hidden, self.intermediate = prefix, hidden, intermediate
+        self.w_gate_up = self.w_down = None
+
+    def tensor_specs(self):
+        p = self.prefix
+        return {
+            p + "gate_proj.weight": TensorSpec((self.intermediate, self.hidden)),
+            p + "up_proj.weight": TensorSpec((self.intermediate, self.hidden)),
+            p + "down_proj.weight": TensorSpec((self.hidden, self.intermediate)),
+        }
+
+    def load(self, get):
+        p = self.prefix
+        self.w_gate_up = torch.cat([get(p + "gate_proj.weight"), get(p + "up_proj.weight")], 0)
+        self.w_down = get(p + "down_proj.weight")
+
+    def forward(self, h, ctx):
+        gu = linear(h, self.w_gate_up, h.dtype)
+        m = torch.empty((h.shape[0], self.intermediate), dtype=h.dtype, device=h.device)
+        ops.swiglu(gu, m)
+        return linear(m, self.w_down, torch.float32)

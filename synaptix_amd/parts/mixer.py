@@ -1,0 +1,103 @@
+"""Token mixers.  Here: grouped-query attention over the paged cache.
+
+GqaAttention: q/k/v projections (one fused product), optional per-head RMSNorm of q and k,
+a position encoding, cache write, causal attention (optionally a window), output projection.
+Order and formulas as crates/synaptix-models/llm/common/src/model.rs:1715-1734 (projections,
+q/k norm before the rotation, the layer's eps), 1781-1782 (cache write), 1740-1869
+(scores, scale, mask, softmax, PV), 1872-1878 (merge heads, o_proj).
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..kernels import ops
+from ..weights.source import TensorSpec
+from .base import Part, KvNeed
+from .linear import linear
+from .position import Position, NoPosition
+
+
+class Mixer(Part):
+    """Interface of a token mixer.
+
+    cache_need(): KvNeed, StateNeed or None: what it keeps for each sequence.
+    forward(h, ctx, cache, owner): h [N, hidden] in the activation type, ctx the step's
+    StepContext, cache the view of its cache layer (None without a need); owner is False when the
+    layer reads a cache that another layer writes.  Returns the residual delta [N, hidden] float.
+    """
+
+    def cache_need(self):
+        return None
+
+    def forward(self, h, ctx, cache, owner=True):
+        raise NotImplementedError
+
+
+class GqaAttention(Mixer):
+    def __init__(self, prefix: str, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, *,
+                 position: Position | None = None, qk_norm_eps: float | None = None, scale: float | None = None,
+                 window: int | None = None):
+        if n_kv_heads <= 0 or n_heads % n_kv_heads:
+            raise ValueError(f"{n_heads} heads do not divide into {n_kv_heads} kv heads")
+        self.prefix = prefix
+        self.hidden, self.nh, self.nkv, self.hd = hidden, n_heads, n_kv_heads, head_dim
+        self.position = position or NoPosition()
+        self.qk_norm_eps = qk_norm_eps
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        self.window = window
+        self.w_qkv = self.w_o = self.q_gain = self.k_gain = None
+
+    def tensor_specs(self):
+        p, hd = self.prefix, self.hd
+        specs = {
+            p + "q_proj.weight": TensorSpec((self.nh * hd, self.hidden)),
+            p + "k_proj.weight": TensorSpec((self.nkv * hd, self.hidden)),
+            p + "v_proj.weight": TensorSpec((self.nkv * hd, self.hidden)),
+            p + "o_proj.weight": TensorSpec((self.hidden, self.nh * hd)),
+        }
+        if self.qk_norm_eps is not None:
+            specs[p + "q_norm.weight"] = TensorSpec((hd,), "gain")
+            specs[p + "k_norm.weight"] = TensorSpec((hd,), "gain")
+        return specs
+
+    def load(self, get):
+        p = self.prefix
+        # one product for q, k and v: rows of the three matrices one after another
+        self.w_qkv = torch.cat([get(p + "q_proj.weight"), get(p + "k_proj.weight"), get(p + "v_proj.weight")], 0)
+        self.w_o = get(p + "o_proj.weight")
+        if self.qk_norm_eps is not None:
+            self.q_gain = get(p + "q_norm.weight")
+            self.k_gain = get(p + "k_norm.weight").to(self.q_gain.dtype)
+
+    def cache_need(self):
+        return KvNeed(self.nkv, self.hd, self.window)
+
+    def forward(self, h, ctx, cache, owner=True):
+        nh, nkv, hd = self.nh, self.nkv, self.hd
+        N, act = h.shape[0], h.dtype
+        cap = self.position.capacity
+        if cap is not None and ctx.max_position >= cap:
+            raise ValueError(f"position {ctx.max_position} is beyond the position encoding's capacity {cap}")
+        qkv = linear(h, self.w_qkv, act)
+        q = torch.empty((N, nh * hd), dtype=act, device=h.device)
+        cos, sin = self.position.tables(h.device)
+        table = ctx.page_table(cache.group)
+        ops.qk_norm_rope_kv_write(qkv, q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos,
+                                  self.q_gain, self.k_gain, self.qk_norm_eps or 0.0, cos, sin, nh, nkv, hd,
+                                  write_kv=owner)
+        o = torch.empty((N, nh * hd), dtype=act, device=h.device)
+        window = self.window or 0
+        if act == torch.float32:
+            ops.attention_f32(q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos, o, self.scale, window,
+                              nh, nkv, hd)
+        elif ctx.one_token_each:
+            splits = ctx.decode_splits(nkv, cache.group)
+            work = ctx.scratch("attention_decode", N * nh * splits * (hd + 2))
+            ops.attention_decode_bf16(q, cache.k_pages, cache.v_pages, table, ctx.seq_len, o, work, splits,
+                                      self.scale, window, nh, nkv, hd)
+        else:
+            ops.attention_prefill_bf16(q, cache.k_pages, cache.v_pages, table, ctx.seq_start, ctx.seq_past, o,
+                                       self.scale, window, nh, nkv, hd)
+        return linear(o, self.w_o, torch.float32)

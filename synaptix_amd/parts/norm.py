@@ -1,0 +1,43 @@
+"""RMSNorm as a part: y = gain * x * rsqrt(mean(x^2) + eps), arithmetic in 32-bit.
+
+Formula and order of the product as in crates/synaptix-ops/src/norm/rms_norm.rs:16-26 and
+crates/synaptix-kernels-cuda/src/cu/reduction/rms_norm.cu:65-98 (plain gain `w`, not `1 + w`).
+The residual sum of the block is fused in (`add_apply`), as the reference's graph path does with
+crates/synaptix-kernels-cuda/src/cu/fused/norm/rmsnorm_residual.cu:97-159; here the residual stream
+itself stays in 32-bit.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..weights.source import TensorSpec
+from .base import Part
+
+
+class RmsNorm(Part):
+    def __init__(self, name: str, dim: int, eps: float):
+        self.name = name          # full tensor name of the gain
+        self.dim = dim
+        self.eps = float(eps)
+        self.gain = None
+
+    def tensor_specs(self):
+        return {self.name: TensorSpec((self.dim,), "gain")}
+
+    def load(self, get):
+        self.gain = get(self.name)
+
+    def add_apply(self, resid, delta, out_dtype, rows=None):
+        """resid [N, dim] float: with rows None, resid += delta (if any) in place and every row is
+        normed; with rows [n] int32 only those rows of resid + delta are normed and resid is kept."""
+        n = resid.shape[0] if rows is None else rows.shape[0]
+        out = torch.empty((n, self.dim), dtype=out_dtype, device=resid.device)
+        ops.add_rmsnorm(resid, delta, self.gain, self.eps, out, rows)
+        return out
+
+    def apply(self, x):
+        """Norm over the last axis of a tensor in the activation type."""
+        out = torch.empty_like(x)
+        ops.rmsnorm_rows(x, self.gain, self.eps, out)
+        return out

@@ -1,0 +1,173 @@
+"""Stand-ins for the GPU kernels, written with torch CPU ops, for tests that run without a GPU.
+
+They let the engine's own logic (packing of a step, the cache, page tables, the order of layers,
+the generation loop) run on the CPU against the plain implementation.  They are test equipment:
+nothing in the package imports them, and the package has no CPU path of its own.
+Each function has the signature and the meaning of its namesake in synaptix_amd.kernels.ops.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import torch
+
+from synaptix_amd.engine.engine import Engine
+from synaptix_amd.engine.batch import fill_host_buffer
+
+PAGE = 64
+F32 = torch.float32
+
+
+def embed(table, ids, resid):
+    resid.copy_(table[ids.long()].to(F32))
+
+
+def add_rmsnorm(resid, delta, gain, eps, out, rows=None):
+    if rows is None:
+        if delta is not None:
+            resid.add_(delta)
+        x = resid
+    else:
+        x = resid[rows.long()]
+        if delta is not None:
+            x = x + delta[rows.long()]
+    inv = torch.rsqrt((x * x).mean(-1, keepdim=True) + eps)
+    out.copy_((gain.to(F32) * x * inv).to(out.dtype))
+
+
+def rmsnorm_rows(x, gain, eps, out):
+    xf = x.to(F32)
+    inv = torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps)
+    out.copy_((gain.to(F32) * xf * inv).to(out.dtype))
+
+
+def swiglu(gate_up, out):
+    I = gate_up.shape[1] // 2
+    g, u = gate_up[:, :I].to(F32), gate_up[:, I:].to(F32)
+    out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
+
+
+def gemm(x, w, out, force_simt=False):
+    out.copy_((x.to(F32) @ w.to(F32).T).to(out.dtype))
+
+
+def qk_norm_rope_kv_write(qkv, q_out, k_pages, v_pages, page_table, tok_seq, tok_pos, q_gain, k_gain, eps,
+                          cos, sin, n_heads, n_kv_heads, head_dim, write_kv=True):
+    nh, nkv, hd = n_heads, n_kv_heads, head_dim
+    N = qkv.shape[0]
+    x = qkv.to(F32).view(N, nh + 2 * nkv, hd)
+    q, k, v = x[:, :nh], x[:, nh:nh + nkv], x[:, nh + nkv:]
+
+    def norm(t, g):
+        if g is None:
+            return t
+        return g.to(F32) * t * torch.rsqrt((t * t).mean(-1, keepdim=True) + eps)
+
+    def rope(t):
+        if cos is None:
+            return t
+        half = cos.shape[1]
+        c, s = cos[tok_pos.long()][:, None, :], sin[tok_pos.long()][:, None, :]
+        a, b, rest = t[..., :half], t[..., half:2 * half], t[..., 2 * half:]
+        return torch.cat([a * c - b * s, b * c + a * s, rest], -1)
+
+    q_out.copy_(rope(norm(q, q_gain)).reshape(N, nh * hd).to(q_out.dtype))
+    if not write_kv:
+        return
+    k = rope(norm(k, k_gain))
+    for n in range(N):
+        p = int(tok_pos[n])
+        page = int(page_table[int(tok_seq[n]), p // PAGE])
+        k_pages[page, :, p % PAGE, :] = k[n].to(k_pages.dtype)
+        v_pages[page, :, :, p % PAGE] = v[n].to(v_pages.dtype)
+
+
+def _attend(qrow, k_pages, v_pages, table_row, pos, scale, window, nh, nkv, hd):
+    T = pos + 1
+    pages = table_row[:(T + PAGE - 1) // PAGE].long()
+    K = k_pages[pages].to(F32).permute(1, 0, 2, 3).reshape(nkv, -1, hd)[:, :T]          # [nkv, T, hd]
+    V = v_pages[pages].to(F32).permute(1, 2, 0, 3).reshape(nkv, hd, -1)[:, :, :T]       # [nkv, hd, T]
+    lo = max(0, pos - window + 1) if window and window > 0 else 0
+    g = nh // nkv
+    out = torch.empty(nh, hd)
+    for h in range(nh):
+        s = (K[h // g, lo:] @ qrow[h]) * scale
+        p = torch.softmax(s, 0)
+        out[h] = V[h // g][:, lo:] @ p
+    return out
+
+
+def attention_f32(q, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale, window, n_heads, n_kv_heads,
+                  head_dim):
+    N = q.shape[0]
+    qf = q.to(F32).view(N, n_heads, head_dim)
+    for n in range(N):
+        o = _attend(qf[n], k_pages, v_pages, page_table[int(tok_seq[n])], int(tok_pos[n]), scale, window,
+                    n_heads, n_kv_heads, head_dim)
+        out[n] = o.reshape(-1).to(out.dtype)
+
+
+def attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, seq_past, out, scale, window, n_heads,
+                           n_kv_heads, head_dim):
+    N = q.shape[0]
+    qf = q.to(F32).view(N, n_heads, head_dim)
+    for b in range(seq_past.shape[0]):
+        for n in range(int(seq_start[b]), int(seq_start[b + 1])):
+            pos = int(seq_past[b]) + n - int(seq_start[b])
+            o = _attend(qf[n], k_pages, v_pages, page_table[b], pos, scale, window, n_heads, n_kv_heads, head_dim)
+            out[n] = o.reshape(-1).to(out.dtype)
+
+
+def decode_splits(n_seqs, n_kv_heads, max_pages):
+    return 1
+
+
+def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
+                          n_heads, n_kv_heads, head_dim):
+    B = q.shape[0]
+    qf = q.to(F32).view(B, n_heads, head_dim)
+    for b in range(B):
+        o = _attend(qf[b], k_pages, v_pages, page_table[b], int(seq_len[b]) - 1, scale, window, n_heads,
+                    n_kv_heads, head_dim)
+        out[b] = o.reshape(-1).to(out.dtype)
+
+
+def sample_rows(logits, temperature, uniform, out):
+    for r in range(logits.shape[0]):
+        x = logits[r]
+        T = 0.0 if temperature is None else float(temperature[r])
+        if not T > 0:
+            m = x.max()
+            out[r] = int(torch.nonzero(x == m)[-1])
+            continue
+        if T != 1.0:
+            x = x / torch.tensor(T, dtype=F32)
+        p = torch.softmax(x, 0)
+        hit = torch.nonzero(float(uniform[r]) < torch.cumsum(p, 0))
+        out[r] = int(hit[0]) if hit.numel() else x.numel() - 1
+
+
+ALL = ["embed", "add_rmsnorm", "rmsnorm_rows", "swiglu", "gemm", "qk_norm_rope_kv_write", "attention_f32",
+       "attention_prefill_bf16", "decode_splits", "attention_decode_bf16", "sample_rows"]
+
+
+def install(monkeypatch):
+    """Replace the kernels by the stand-ins for the duration of a test."""
+    from synaptix_amd.kernels import ops
+    import sys
+    me = sys.modules[__name__]
+    for name in ALL:
+        monkeypatch.setattr(ops, name, getattr(me, name))
+
+
+class CpuEngine(Engine):
+    """The engine with the two places that need a GPU (the device check, the pinned upload) replaced."""
+
+    def _require_gpu(self):
+        pass
+
+    def _upload(self, layout, token_lists, past, slots, want_rows, tables):
+        host = np.zeros(layout.total, dtype=np.int32)
+        fill_host_buffer(layout, host, token_lists, past, slots, want_rows, tables)
+        return torch.from_numpy(host)

@@ -1,0 +1,421 @@
+"""Each HIP kernel alone against a plain torch float32 statement of the same operation
+(tests/cpu_kernels.py), at sizes other than the engine's test models use, with sizes that are
+no multiple of any tile.  Tolerances follow the reference's ladder for its CUDA kernels
+(crates/synaptix-kernels-cuda/tests/*: float32 1e-5 .. 1e-4, bf16 around 1e-2 on O(1) data)."""
+import math
+
+import pytest
+import torch
+
+import cpu_kernels as ref
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+F32, BF16, I32 = torch.float32, torch.bfloat16, torch.int32
+
+
+@pytest.fixture(scope="module")
+def ops():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from synaptix_amd.kernels import ops as o
+    return o
+
+
+def rnd(shape, seed, dtype=F32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def close(got, want, atol, rtol=0.0, what=""):
+    got, want = got.detach().cpu().to(F32), want.detach().cpu().to(F32)
+    assert torch.isfinite(got).all(), f"{what}: non-finite values"
+    err = (got - want).abs()
+    bound = atol + rtol * want.abs()
+    bad = err > bound
+    assert not bad.any(), f"{what}: max abs err {err.max():.3e} (allowed {atol:.1e} + {rtol:.1e}|x|), {int(bad.sum())} values off"
+
+
+# ----------------------------------------------------------------------------- rows
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("V,H,N", [(100, 24, 7), (1000, 4100, 3)])
+def test_embed(ops, dtype, V, H, N):
+    table = rnd((V, H), 1, dtype)
+    ids = torch.tensor([(i * 37 + V - 1) % V for i in range(N)], dtype=I32)
+    out = torch.empty((N, H), dtype=F32, device=DEV)
+    ops.embed(table.to(DEV), ids.to(DEV), out)
+    assert torch.equal(out.cpu(), table[ids.long()].to(F32))  # a copy: exact
+
+
+@pytest.mark.parametrize("out_dtype,gain_dtype", [(F32, F32), (BF16, BF16), (BF16, F32)])
+@pytest.mark.parametrize("N,H", [(5, 72), (3, 4096), (2, 5000)])
+def test_add_rmsnorm(ops, out_dtype, gain_dtype, N, H):
+    eps = 1e-5
+    resid, delta = rnd((N, H), 2), rnd((N, H), 3)
+    gain = (1 + 0.1 * rnd((H,), 4)).to(gain_dtype)
+    want_resid = resid.clone()
+    want = torch.empty((N, H), dtype=out_dtype)
+    ref.add_rmsnorm(want_resid, delta, gain, eps, want)
+    r = resid.to(DEV)
+    out = torch.empty((N, H), dtype=out_dtype, device=DEV)
+    ops.add_rmsnorm(r, delta.to(DEV), gain.to(DEV), eps, out)
+    close(r, want_resid, 1e-6, what="residual sum")
+    close(out, want, 1e-5 if out_dtype == F32 else 2e-2, 1e-5 if out_dtype == F32 else 1e-2, "normed")
+    # without a delta the residual stays; with rows only those rows are normed and nothing is written
+    r2 = resid.to(DEV)
+    ops.add_rmsnorm(r2, None, gain.to(DEV), eps, out)
+    assert torch.equal(r2.cpu(), resid)
+    rows = torch.tensor([N - 1, 0], dtype=I32)
+    out2 = torch.empty((2, H), dtype=out_dtype, device=DEV)
+    want2 = torch.empty((2, H), dtype=out_dtype)
+    ref.add_rmsnorm(resid.clone(), delta, gain, eps, want2, rows)
+    ops.add_rmsnorm(r2, delta.to(DEV), gain.to(DEV), eps, out2, rows.to(DEV))
+    assert torch.equal(r2.cpu(), resid)
+    close(out2, want2, 1e-5 if out_dtype == F32 else 2e-2, 1e-5 if out_dtype == F32 else 1e-2, "gathered rows")
+
+
+def test_rmsnorm_eps_sits_inside_the_root(ops):
+    # tiny x: sqrt(mean + eps) and sqrt(mean) + eps differ by orders of magnitude
+    x = torch.full((1, 64), 1e-4)
+    gain = torch.ones(64)
+    out = torch.empty((1, 64), device=DEV)
+    ops.rmsnorm_rows(x.to(DEV), gain.to(DEV), 1e-6, out)
+    want = 1e-4 / math.sqrt(1e-8 + 1e-6)
+    close(out, torch.full((1, 64), want), 1e-6, what="eps inside the root")
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("R,D", [(9, 16), (5, 80), (3, 200)])
+def test_rmsnorm_rows(ops, dtype, R, D):
+    x, gain = rnd((R, D), 5, dtype), (1 + 0.1 * rnd((D,), 6)).to(dtype)
+    want = torch.empty_like(x)
+    ref.rmsnorm_rows(x, gain, 1e-6, want)
+    out = torch.empty((R, D), dtype=dtype, device=DEV)
+    ops.rmsnorm_rows(x.to(DEV), gain.to(DEV), 1e-6, out)
+    close(out, want, 1e-5 if dtype == F32 else 2e-2, 0 if dtype == F32 else 1e-2)
+
+
+def test_rmsnorm_reference_vector(ops):
+    """The vector of crates/synaptix-ops/tests/rms_norm.rs:76-95, against the float64 closed form."""
+    x = torch.tensor([i * 0.1 - 1.0 for i in range(24)], dtype=F32).view(6, 4)
+    w = torch.tensor([0.5, -0.25, 1.0, 2.0])
+    out = torch.empty((6, 4), device=DEV)
+    ops.rmsnorm_rows(x.to(DEV), w.to(DEV), 1e-6, out)
+    xd = x.double()
+    want = xd / torch.sqrt((xd * xd).mean(-1, keepdim=True) + 1e-6) * w.double()
+    close(out, want.float(), 1e-5)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_swiglu(ops, dtype):
+    N, I = 7, 176
+    gu = rnd((N, 2 * I), 7, dtype, 2.0)
+    want = torch.empty((N, I), dtype=dtype)
+    ref.swiglu(gu, want)
+    out = torch.empty((N, I), dtype=dtype, device=DEV)
+    ops.swiglu(gu.to(DEV), out)
+    close(out, want, 5e-6 if dtype == F32 else 1.5e-2, 0 if dtype == F32 else 1e-2)
+    # swapping gate and up must change the result (a swapped fused layout would not be seen otherwise)
+    swapped = torch.cat([gu[:, I:], gu[:, :I]], 1).contiguous()
+    out2 = torch.empty((N, I), dtype=dtype, device=DEV)
+    ops.swiglu(swapped.to(DEV), out2)
+    assert (out2.cpu().float() - want.float()).abs().max() > 0.1
+
+
+# ----------------------------------------------------------------------------- matrix product
+
+@pytest.mark.parametrize("M,N,K", [(1, 33, 40), (7, 100, 72), (64, 64, 64), (65, 130, 100), (200, 70, 300)])
+def test_gemm_f32(ops, M, N, K):
+    x, w = rnd((M, K), 8), rnd((N, K), 9)
+    out = torch.empty((M, N), device=DEV)
+    ops.gemm(x.to(DEV), w.to(DEV), out)
+    want = (x.double() @ w.double().T).float()
+    close(out, want, 1e-4, 1e-5, f"gemm f32 {M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("out_dtype", [BF16, F32])
+@pytest.mark.parametrize("M,N,K", [
+    (1, 48, 64), (3, 1000, 176), (16, 100, 320), (17, 40, 72), (33, 1000, 128), (48, 70, 2048), (64, 4096, 512),
+    (65, 130, 104), (128, 128, 32), (200, 300, 1000), (513, 257, 4096),
+    (5, 30, 20), (70, 50, 36),          # K no multiple of 8: the plain kernel takes them
+])
+def test_gemm_bf16(ops, out_dtype, M, N, K):
+    x, w = rnd((M, K), 10, BF16), rnd((N, K), 11, BF16)
+    out = torch.empty((M, N), dtype=out_dtype, device=DEV)
+    ops.gemm(x.to(DEV), w.to(DEV), out)
+    want = (x.double() @ w.double().T).float()
+    # float accumulation of exact bf16 products: the only error is the order of the sum and the last rounding
+    atol = 1e-3 * math.sqrt(K)
+    close(out, want, atol if out_dtype == F32 else atol + 0.02, 0 if out_dtype == F32 else 1e-2, f"gemm bf16 {M}x{N}x{K}")
+
+
+def test_gemm_bf16_paths_agree(ops):
+    """The MFMA kernels and the plain kernel compute the same sums."""
+    for M in (4, 40, 300):
+        x, w = rnd((M, 256), 12, BF16).to(DEV), rnd((96, 256), 13, BF16).to(DEV)
+        a = torch.empty((M, 96), dtype=F32, device=DEV)
+        b = torch.empty((M, 96), dtype=F32, device=DEV)
+        ops.gemm(x, w, a)
+        ops.gemm(x, w, b, force_simt=True)
+        close(a, b, 2e-4, what=f"mfma vs plain, M={M}")
+
+
+# ----------------------------------------------------------------------------- cache write + attention
+
+def make_cache(n_pages, nkv, hd, dtype, seed, fill="garbage"):
+    """Pages filled with large values: whatever a kernel reads beyond a sequence's end shows."""
+    k = rnd((n_pages, nkv, 64, hd), seed, dtype, 50.0)
+    v = rnd((n_pages, nkv, hd, 64), seed + 1, dtype, 50.0)
+    if fill == "nan":
+        k[:], v[:] = float("nan"), float("nan")
+    return k, v
+
+
+def step_arrays(past, new):
+    tok_seq, tok_pos, starts = [], [], [0]
+    for i, (p, n) in enumerate(zip(past, new)):
+        tok_seq += [i] * n
+        tok_pos += list(range(p, p + n))
+        starts.append(starts[-1] + n)
+    t = lambda a: torch.tensor(a, dtype=I32)
+    return t(tok_seq), t(tok_pos), t(starts), t(past), t([p + n for p, n in zip(past, new)])
+
+
+def shuffled_table(n_seqs, width, seed):
+    """Each sequence's pages lie scattered over the pool."""
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(n_seqs * width, generator=g).to(I32)
+    return perm.view(n_seqs, width).contiguous()
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("nh,nkv,hd,rot,norm", [(4, 2, 16, 16, True), (6, 3, 48, 32, True), (8, 1, 128, 128, False),
+                                                (3, 3, 80, 0, True)])
+def test_qk_norm_rope_kv_write(ops, dtype, nh, nkv, hd, rot, norm):
+    past, new = [3, 70, 0], [5, 1, 66]
+    tok_seq, tok_pos, _, _, _ = step_arrays(past, new)
+    N = len(tok_seq)
+    table = shuffled_table(3, 3, 1)
+    qkv = rnd((N, (nh + 2 * nkv) * hd), 20, dtype)
+    qg = (1 + 0.1 * rnd((hd,), 21)).to(dtype) if norm else None
+    kg = (1 + 0.1 * rnd((hd,), 22)).to(dtype) if norm else None
+    cos = sin = None
+    if rot:
+        ang = torch.arange(200, dtype=F32)[:, None] * (10000.0 ** (-torch.arange(rot // 2, dtype=F32) * 2 / rot))[None]
+        cos, sin = torch.cos(ang), torch.sin(ang)
+    k0, v0 = make_cache(9, nkv, hd, dtype, 23)
+    kw, vw, qw = k0.clone(), v0.clone(), torch.empty((N, nh * hd), dtype=dtype)
+    ref.qk_norm_rope_kv_write(qkv, qw, kw, vw, table, tok_seq, tok_pos, qg, kg, 1e-5, cos, sin, nh, nkv, hd)
+    d = lambda t: None if t is None else t.to(DEV)
+    kd, vd, qd = k0.to(DEV), v0.to(DEV), torch.empty((N, nh * hd), dtype=dtype, device=DEV)
+    ops.qk_norm_rope_kv_write(d(qkv), qd, kd, vd, d(table), d(tok_seq), d(tok_pos), d(qg), d(kg), 1e-5, d(cos), d(sin),
+                              nh, nkv, hd)
+    tol = dict(atol=1e-5, rtol=1e-5) if dtype == F32 else dict(atol=3e-2, rtol=1e-2)
+    close(qd, qw, what="q", **tol)
+    close(kd, kw, what="k pages", **tol)
+    assert torch.equal(vd.cpu(), vw), "v is a copy"
+    # untouched places of the pages stay as they were
+    untouched = (kw == k0)
+    assert torch.equal(kd.cpu()[untouched], k0[untouched])
+    # a reader of another layer's cache writes nothing
+    kd2, vd2 = k0.to(DEV), v0.to(DEV)
+    ops.qk_norm_rope_kv_write(d(qkv), qd, kd2, vd2, d(table), d(tok_seq), d(tok_pos), d(qg), d(kg), 1e-5, d(cos), d(sin),
+                              nh, nkv, hd, write_kv=False)
+    assert torch.equal(kd2.cpu(), k0) and torch.equal(vd2.cpu(), v0)
+    close(qd, qw, what="q without cache write", **tol)
+
+
+def fill_sequences(k, v, table, lens, nkv, hd, dtype, seed):
+    """Write O(1) keys and values for positions below each length; the rest stays garbage."""
+    for b, T in enumerate(lens):
+        kk = rnd((T, nkv, hd), seed + 10 * b, dtype)
+        vv = rnd((T, nkv, hd), seed + 10 * b + 1, dtype)
+        for t in range(T):
+            page = int(table[b, t // 64])
+            k[page, :, t % 64, :] = kk[t]
+            v[page, :, :, t % 64] = vv[t]
+
+
+ATTN_SHAPES = [
+    # nh, nkv, hd, past, new, window
+    (4, 2, 16, [0, 0, 0], [5, 17, 70], 0),
+    (8, 1, 32, [0, 100, 63], [130, 1, 2], 0),
+    (6, 3, 48, [10, 0], [40, 200], 0),
+    (8, 2, 64, [600, 0], [1, 8], 0),            # the reference's decode shape (2,8,2,1,600,64) beside a short one
+    (32, 8, 128, [0], [300], 0),
+    (4, 4, 128, [0, 40], [33, 1], 0),
+    (4, 2, 96, [0, 5], [150, 100], 37),          # a window that ends inside pages
+    (5, 5, 16, [200], [1], 64),
+]
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("nh,nkv,hd,past,new,window", ATTN_SHAPES)
+def test_attention_prefill(ops, dtype, nh, nkv, hd, past, new, window):
+    B = len(past)
+    lens = [p + n for p, n in zip(past, new)]
+    width = max((T + 63) // 64 for T in lens) + 1
+    table = shuffled_table(B, width, 3)
+    k, v = make_cache(B * width, nkv, hd, dtype, 30)
+    fill_sequences(k, v, table, lens, nkv, hd, dtype, 31)
+    tok_seq, tok_pos, starts, past_t, len_t = step_arrays(past, new)
+    N = len(tok_seq)
+    q = rnd((N, nh * hd), 32, dtype)
+    scale = 1 / math.sqrt(hd)
+    want = torch.empty((N, nh * hd), dtype=F32)
+    ref.attention_f32(q.float(), k.float(), v.float(), table, tok_seq, tok_pos, want, scale, window, nh, nkv, hd)
+    d = lambda t: t.to(DEV)
+    out = torch.empty((N, nh * hd), dtype=dtype, device=DEV)
+    if dtype == F32:
+        ops.attention_f32(d(q), d(k), d(v), d(table), d(tok_seq), d(tok_pos), out, scale, window, nh, nkv, hd)
+        close(out, want, 1e-4, what="attention f32")
+    else:
+        ops.attention_prefill_bf16(d(q), d(k), d(v), d(table), d(starts), d(past_t), out, scale, window, nh, nkv, hd)
+        close(out, want, 2e-2, 1e-2, what="attention prefill bf16")
+
+
+@pytest.mark.parametrize("nh,nkv,hd,lens,window,splits", [
+    (8, 2, 64, [600, 3], 0, 4),                 # crates/synaptix-kernels-cuda/tests/cuda_flash_decode.rs:101 GQA, Tkv=600
+    (4, 4, 128, [40], 0, 8),                    # more splits than pages (empty splits), ibid. 130-183
+    (40, 2, 32, [129, 64, 65, 1], 0, 3),        # 20 heads a group: two chunks of 16
+    (8, 1, 16, [1000, 77], 0, 16),
+    (4, 2, 96, [500, 30], 100, 5),
+    (32, 8, 128, [2100] * 3, 0, 11),
+])
+def test_attention_decode_bf16(ops, nh, nkv, hd, lens, window, splits):
+    B = len(lens)
+    width = max((T + 63) // 64 for T in lens) + 2
+    table = shuffled_table(B, width, 4)
+    k, v = make_cache(B * width, nkv, hd, BF16, 40, fill="nan" if hd == 64 else "garbage")
+    fill_sequences(k, v, table, lens, nkv, hd, BF16, 41)
+    tok_seq = torch.arange(B, dtype=I32)
+    tok_pos = torch.tensor([T - 1 for T in lens], dtype=I32)
+    q = rnd((B, nh * hd), 42, BF16)
+    scale = 1 / math.sqrt(hd)
+    want = torch.empty((B, nh * hd), dtype=F32)
+    kf, vf = torch.nan_to_num(k.float()), torch.nan_to_num(v.float())
+    ref.attention_f32(q.float(), kf, vf, table, tok_seq, tok_pos, want, scale, window, nh, nkv, hd)
+    d = lambda t: t.to(DEV)
+    out = torch.empty((B, nh * hd), dtype=BF16, device=DEV)
+    work = torch.empty(B * nh * splits * (hd + 2), dtype=F32, device=DEV)
+    ops.attention_decode_bf16(d(q), d(k), d(v), d(table), d(torch.tensor(lens, dtype=I32)), out, work, splits, scale,
+                              window, nh, nkv, hd)
+    close(out, want, 2e-2, 1e-2, what="attention decode bf16")
+
+
+def test_attention_far_key_stands_out(ops):
+    """One key among hundreds is made to dominate: the output must be that key's value, in every
+    kernel.  A kernel that loses a page, a split or the cache's start would not show it with
+    random data."""
+    nh, nkv, hd, T = 4, 2, 64, 700
+    scale = 1 / math.sqrt(hd)
+    for far in (0, 63, 64, 350, T - 1):
+        table = shuffled_table(1, 12, far)
+        k, v = make_cache(12, nkv, hd, BF16, 50)
+        fill_sequences(k, v, table, [T], nkv, hd, BF16, 51)
+        q = rnd((1, nh * hd), 52, BF16)
+        page = int(table[0, far // 64])
+        for h in range(nkv):   # the far key is 20 x the query of the group's first head
+            k[page, h, far % 64, :] = (q.view(nh, hd)[h * 2] * 20).to(BF16)
+        want = v[page, :, :, far % 64].float()            # [nkv, hd]
+        d = lambda t: t.to(DEV)
+        lens = torch.tensor([T], dtype=I32)
+        out = torch.empty((1, nh * hd), dtype=BF16, device=DEV)
+        work = torch.empty(nh * 6 * (hd + 2), dtype=F32, device=DEV)
+        ops.attention_decode_bf16(d(q), d(k), d(v), d(table), d(lens), out, work, 6, scale, 0, nh, nkv, hd)
+        got = out.cpu().float().view(nh, hd)
+        for h in range(nkv):
+            close(got[h * 2], want[h], 3e-2, 2e-2, f"decode, far key {far}")
+        outp = torch.empty((1, nh * hd), dtype=BF16, device=DEV)
+        ops.attention_prefill_bf16(d(q), d(k), d(v), d(table), d(torch.tensor([0, 1], dtype=I32)),
+                                   d(torch.tensor([T - 1], dtype=I32)), outp, scale, 0, nh, nkv, hd)
+        gotp = outp.cpu().float().view(nh, hd)
+        for h in range(nkv):
+            close(gotp[h * 2], want[h], 3e-2, 2e-2, f"prefill, far key {far}")
+        o32 = torch.empty((1, nh * hd), dtype=F32, device=DEV)
+        ops.attention_f32(d(q.float()), d(k.float()), d(v.float()), d(table), d(torch.zeros(1, dtype=I32)),
+                          d(torch.tensor([T - 1], dtype=I32)), o32, scale, 0, nh, nkv, hd)
+        got32 = o32.cpu().view(nh, hd)
+        for h in range(nkv):
+            close(got32[h * 2], want[h], 1e-3, 1e-3, f"f32, far key {far}")
+
+
+def test_attention_window_edge(ops):
+    """The key just outside the window dominates if it is seen: it must not be."""
+    nh, nkv, hd, T, W = 2, 1, 32, 300, 100
+    scale = 1 / math.sqrt(hd)
+    table = shuffled_table(1, 6, 9)
+    k, v = make_cache(6, nkv, hd, BF16, 60)
+    fill_sequences(k, v, table, [T], nkv, hd, BF16, 61)
+    q = rnd((1, nh * hd), 62, BF16)
+    edge = T - 1 - W          # the last key outside: visible keys are j > T-1-W
+    page = int(table[0, edge // 64])
+    k[page, 0, edge % 64, :] = (q.view(nh, hd)[0] * 20).to(BF16)
+    tok_seq, tok_pos = torch.zeros(1, dtype=I32), torch.tensor([T - 1], dtype=I32)
+    want = torch.empty((1, nh * hd), dtype=F32)
+    ref.attention_f32(q.float(), k.float(), v.float(), table, tok_seq, tok_pos, want, scale, W, nh, nkv, hd)
+    seen = torch.empty((1, nh * hd), dtype=F32)
+    ref.attention_f32(q.float(), k.float(), v.float(), table, tok_seq, tok_pos, seen, scale, W + 1, nh, nkv, hd)
+    assert (want - seen).abs().max() > 1.0, "the test's key does not dominate"
+    d = lambda t: t.to(DEV)
+    out = torch.empty((1, nh * hd), dtype=BF16, device=DEV)
+    work = torch.empty(nh * 3 * (hd + 2), dtype=F32, device=DEV)
+    ops.attention_decode_bf16(d(q), d(k), d(v), d(table), d(torch.tensor([T], dtype=I32)), out, work, 3, scale, W, nh,
+                              nkv, hd)
+    close(out, want, 2e-2, 1e-2, "decode at the window's edge")
+    ops.attention_prefill_bf16(d(q), d(k), d(v), d(table), d(torch.tensor([0, 1], dtype=I32)),
+                               d(torch.tensor([T - 1], dtype=I32)), out, scale, W, nh, nkv, hd)
+    close(out, want, 2e-2, 1e-2, "prefill at the window's edge")
+    o32 = torch.empty((1, nh * hd), dtype=F32, device=DEV)
+    ops.attention_f32(d(q.float()), d(k.float()), d(v.float()), d(table), d(tok_seq), d(tok_pos), o32, scale, W, nh, nkv,
+                      hd)
+    close(o32, want, 1e-4, what="f32 at the window's edge")
+
+
+# ----------------------------------------------------------------------------- sampling
+
+def test_sample_rows_greedy_and_ties(ops):
+    V = 1000
+    x = rnd((5, V), 70)
+    x[1, 17] = x[1, 900] = 9.0           # the last of equal maxima wins
+    x[2, :] = 0.0                        # all equal: the last index
+    out = torch.empty(5, dtype=I32, device=DEV)
+    ops.sample_rows(x.to(DEV), None, None, out)
+    want = [int(x[0].argmax()), 900, V - 1, int(x[3].argmax()), int(x[4].argmax())]
+    assert out.cpu().tolist() == want
+
+
+def test_sample_rows_temperature(ops):
+    V, R = 333, 64
+    x = rnd((R, V), 71, scale=3.0)
+    temps = torch.tensor([0.7, 1.0, 0.0, 1.5] * (R // 4))
+    g = torch.Generator().manual_seed(5)
+    u = torch.rand(R, generator=g)
+    want = torch.empty(R, dtype=I32)
+    ref.sample_rows(x, temps, u, want)
+    out = torch.empty(R, dtype=I32, device=DEV)
+    ops.sample_rows(x.to(DEV), temps.to(DEV), u.to(DEV), out)
+    got = out.cpu()
+    # a draw falls on the other side of a boundary only if u is within rounding of the CDF there
+    differ = int((got != want).sum())
+    assert differ <= 1, f"{differ} of {R} draws differ"
+    # u = 1 can never be below the last cumulative sum of rounded probabilities: the last index
+    ops.sample_rows(x.to(DEV), torch.ones(R).to(DEV), torch.full((R,), 1.5).to(DEV), out)
+    assert out.cpu().tolist() == [V - 1] * R
+
+
+def test_sample_rows_frequencies(ops):
+    """Frequencies of many draws lie within 0.01 of the probabilities
+    (as crates/synaptix-infer/tests/ref_infer.rs:114-166, with fewer draws)."""
+    V, R = 50, 20000
+    logits = rnd((1, V), 72, scale=1.5)
+    x = logits.expand(R, V).contiguous()
+    g = torch.Generator().manual_seed(6)
+    u = torch.rand(R, generator=g)
+    out = torch.empty(R, dtype=I32, device=DEV)
+    ops.sample_rows(x.to(DEV), torch.full((R,), 0.8).to(DEV), u.to(DEV), out)
+    freq = torch.bincount(out.cpu().long(), minlength=V).float() / R
+    p = torch.softmax(logits[0] / 0.8, 0)
+    assert (freq - p).abs().max() < 0.012
