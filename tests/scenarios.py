@@ -1,0 +1,158 @@
+"""Scenarios that compare an engine with the plain implementation; the engine is made by a
+factory, so the same scenarios run with the stand-in kernels on the CPU and with the HIP
+kernels on the GPU."""
+from __future__ import annotations
+
+import torch
+
+from helpers import CONFIGS, plain_logits, plain_model, random_tokens, assert_logits_close, model_folder
+from synaptix_amd.engine.generate import generate, GenerationConfig
+import plain_qwen3 as P
+
+
+def lengths_for(name):
+    # the batches of BASELINE's tiny configurations, plus lengths around a page's edge
+    return {"A": [5, 17, 11, 64, 65], "B": [1, 33, 7, 64, 130], "C": [3, 70, 129, 40, 200]}[name]
+
+
+def requests_for(name, tail=0):
+    V = CONFIGS[name]["vocab_size"]
+    return {f"r{i}": random_tokens(V, n + tail, 100 + i) for i, n in enumerate(lengths_for(name))}
+
+
+def whole(make_engine, name, dtype, sharp=False):
+    """Each request alone and whole: one step, every position wanted."""
+    eng = make_engine(name, dtype, 1024, sharp)
+    for rid, toks in requests_for(name).items():
+        s = eng.acquire()
+        got = eng.step([(s, toks)], want="all")
+        assert_logits_close(got, plain_logits(name, toks, sharp), dtype, f"{name} {dtype} {rid} whole")
+        eng.release(s)
+    eng.cache.check()
+
+
+def last_tokens_one_by_one(make_engine, name, dtype, tail=32, sharp=False):
+    """The same requests with their last `tail` tokens decoded one by one."""
+    eng = make_engine(name, dtype, 2048, sharp)
+    for rid, toks in requests_for(name, tail).items():
+        want = plain_logits(name, toks, sharp)
+        s = eng.acquire()
+        head = len(toks) - tail
+        got = [eng.step([(s, toks[:head])], want="all")]
+        for t in toks[head:]:
+            got.append(eng.step([(s, [t])], want="last"))
+        assert_logits_close(torch.cat(got), want, dtype, f"{name} {dtype} {rid} last {tail} one by one")
+        eng.release(s)
+    eng.cache.check()
+
+
+def unequal_batches(make_engine, name, dtype, sharp=False, decode=12):
+    """Batches of unequal lengths whose shorter requests end earlier, one batch after another so
+    that slots and pages are used again; the second batch's order differs from the first's."""
+    reqs = requests_for(name, tail=0)
+    ids = list(reqs)
+    batches = [ids[:3], ids[3:] + ids[:1], list(reversed(ids))]
+    eng = make_engine(name, dtype, 64 * 12, sharp)
+    for batch in batches:
+        slots = {r: eng.acquire() for r in batch}
+        head = {r: max(1, len(reqs[r]) - decode) for r in batch}
+        got = {r: [] for r in batch}
+        lg = eng.step([(slots[r], reqs[r][:head[r]]) for r in batch], want="all")
+        off = 0
+        for r in batch:
+            got[r].append(lg[off:off + head[r]])
+            off += head[r]
+        fed = dict(head)
+        live = [r for r in batch if fed[r] < len(reqs[r])]
+        for r in batch:
+            if r not in live:
+                eng.release(slots[r])
+        while live:
+            lg = eng.step([(slots[r], [reqs[r][fed[r]]]) for r in live], want="last")
+            for i, r in enumerate(live):
+                got[r].append(lg[i:i + 1])
+                fed[r] += 1
+            for r in [r for r in live if fed[r] == len(reqs[r])]:
+                eng.release(slots[r])                       # leaves the batch; the others go on
+            live = [r for r in live if fed[r] < len(reqs[r])]
+        for r in batch:
+            assert_logits_close(torch.cat(got[r]), plain_logits(name, reqs[r], sharp), dtype,
+                                f"{name} {dtype} {r} in batch {batch}")
+        eng.cache.check()
+    assert eng.cache.free_slots == eng.cache.max_slots
+
+
+def long_decoding(make_engine, name, dtype, n_decode):
+    """A short prompt, then many single tokens: positions cross several pages."""
+    V = CONFIGS[name]["vocab_size"]
+    toks = random_tokens(V, 3 + n_decode, 7)
+    want = plain_logits(name, toks)
+    eng = make_engine(name, dtype, 1024, False)
+    s = eng.acquire()
+    got = [eng.step([(s, toks[:3])], want="all")]
+    for t in toks[3:]:
+        got.append(eng.step([(s, [t])], want="last"))
+    got = torch.cat(got)
+    assert_logits_close(got, want, dtype, f"{name} {dtype} long decoding")
+    # the last positions alone, so that an error that grows with the position is not averaged away
+    assert_logits_close(got[-8:], want[-8:], dtype, f"{name} {dtype} long decoding, last positions")
+
+
+def first_tokens(make_engine, name, dtype):
+    """Prompts of one and two tokens; the very first position; a chunk that starts at position 1."""
+    V = CONFIGS[name]["vocab_size"]
+    eng = make_engine(name, dtype, 512, False)
+    toks = random_tokens(V, 4, 8)
+    want = plain_logits(name, toks)
+    a, b, c = eng.acquire(), eng.acquire(), eng.acquire()
+    lg = eng.step([(a, toks[:1]), (b, toks[:2]), (c, toks)], want=[[0], [0, 1], [0, 3]])
+    assert_logits_close(lg[0:1], want[0:1], dtype, "one token")
+    assert_logits_close(lg[1:3], want[0:2], dtype, "two tokens")
+    assert_logits_close(lg[3:5], want[[0, 3]], dtype, "places 0 and 3")
+    lg = eng.step([(a, toks[1:])], want="all")                 # positions 1..3 in one step after position 0
+    assert_logits_close(lg, want[1:], dtype, "a chunk from position 1")
+    lg = eng.step([(b, toks[2:3])], want=None)                 # nothing wanted: the cache still advances
+    assert lg.shape[0] == 0 and eng.length(b) == 3
+    lg = eng.step([(b, toks[3:])], want="last")
+    assert_logits_close(lg, want[3:], dtype, "after a step that wanted nothing")
+
+
+def greedy_generation(make_engine, name, dtype, n_new=8):
+    """Greedy generation through the generation loop equals the plain implementation's."""
+    V = CONFIGS[name]["vocab_size"]
+    prompts = [random_tokens(V, n, 200 + i) for i, n in enumerate(lengths_for(name)[:4])]
+    plain = plain_model(name)
+    want = [P.generate(plain, p, n_new) for p in prompts]
+    eng = make_engine(name, dtype, 2048, False)
+    outs, stats = generate(eng, prompts, GenerationConfig(max_new_tokens=n_new), max_batch=3)
+    assert stats.batches == 2
+    for p, o, w in zip(prompts, outs, want):
+        if dtype == "float32":
+            assert o.tokens == w
+        else:
+            check_greedy_path(plain, p, o.tokens, w)
+    eng.cache.check()
+
+
+def check_greedy_path(plain, prompt, got, want, margin=2e-2):
+    """bfloat16 may leave the plain greedy path, but only where the plain logits nearly tie."""
+    for i, (g, w) in enumerate(zip(got, want)):
+        if g != w:
+            row = plain.forward(list(prompt) + want[:i])[-1]
+            assert float(row[w] - row[g]) <= margin * max(1.0, float(row.abs().max())), \
+                f"token {i}: engine {g}, plain {w}, and the plain logits do not tie"
+            return
+
+
+def sampled_generation(make_engine, name, dtype):
+    """Temperature sampling with per-sequence streams: BASELINE's tiny B case (T = 0.7, seed 1)."""
+    V = CONFIGS[name]["vocab_size"]
+    prompts = [random_tokens(V, n, 300 + i) for i, n in enumerate(lengths_for(name)[:4])]
+    plain = plain_model(name)
+    eng = make_engine(name, dtype, 2048, False)
+    outs, _ = generate(eng, prompts, GenerationConfig(max_new_tokens=12, temperature=0.7, seed=1))
+    same = 0
+    for i, (p, o) in enumerate(zip(prompts, outs)):
+        same += o.tokens == P.generate(plain, p, 12, seed=1 + i, temperature=0.7)
+    # a draw can fall on the other side of a CDF boundary by rounding; that is rare
+    assert same >= len(prompts) - 1

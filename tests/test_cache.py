@@ -1,0 +1,153 @@
+"""The cache's bookkeeping (no GPU): no slot or page lost, held twice or freed twice."""
+import random
+
+import pytest
+import torch
+
+from synaptix_amd.cache import SequenceCache, PagePool, CacheFull, CacheError, PAGE_TOKENS, pages_for
+from synaptix_amd.parts import KvNeed, StateNeed
+
+
+def make(max_tokens=640, max_slots=None, needs=None, max_positions=None):
+    needs = needs if needs is not None else [KvNeed(2, 16)] * 3
+    return SequenceCache(needs, max_tokens, max_slots, torch.float32, "cpu", max_positions=max_positions)
+
+
+def test_page_pool():
+    p = PagePool(4)
+    a = p.take(3)
+    assert a == [0, 1, 2] and p.free_pages == 1
+    with pytest.raises(CacheFull):
+        p.take(2)
+    assert p.free_pages == 1                        # nothing was taken
+    p.give_back([1])
+    with pytest.raises(CacheError, match="not held"):
+        p.give_back([1])                            # freed twice
+    with pytest.raises(CacheError):
+        p.give_back([9])
+    p.check()
+    assert sorted(p.take(2)) == [1, 3]
+    p.check()
+
+
+def test_groups_and_storage():
+    c = make(needs=[KvNeed(2, 16), KvNeed(1, 32), KvNeed(2, 16), StateNeed((3, 5)), None, KvNeed(2, 16, window=100)])
+    assert [g.layers for g in c.groups] == [[0, 2], [1], [5]]
+    assert c.groups[0].k.shape == (2, 10, 2, 64, 16) and c.groups[0].v.shape == (2, 10, 2, 16, 64)
+    assert c.groups[1].k.shape == (1, 10, 1, 64, 32)
+    v0, v2, v3 = c.layer_view(0), c.layer_view(2), c.layer_view(3)
+    assert v0.group == v2.group == 0 and v0.k_pages.data_ptr() != v2.k_pages.data_ptr()
+    assert v3.state.shape == (10, 3, 5) and c.layer_view(4) is None
+    assert c.bytes_per_token() == 2 * 4 * (2 * 2 * 16 + 1 * 32 + 2 * 16)
+
+
+def test_slot_life_cycle_and_errors():
+    c = make(max_tokens=256, max_slots=2)
+    a, b = c.acquire(), c.acquire()
+    assert {a, b} == {0, 1} and c.free_slots == 0
+    with pytest.raises(CacheFull, match="slots"):
+        c.acquire()
+    c.reserve(a, 70)
+    c.commit(a, 70)
+    assert c.length(a) == 70 and c.groups[0].pool.free_pages == 2
+    c.reserve(a, 1)                                  # 71 tokens still fit two pages
+    assert c.groups[0].pool.free_pages == 2
+    with pytest.raises(CacheError, match="commit without reserve"):
+        c.commit(a, 5)
+    c.commit(a, 1)
+    c.reserve(b, 128)
+    with pytest.raises(CacheFull):
+        c.reserve(a, 100)                            # would need a third page; nothing changes
+    assert c.groups[0].pool.free_pages == 0 and c.length(a) == 71
+    c.check()
+    c.release(a)
+    with pytest.raises(CacheError, match="not live"):
+        c.release(a)                                 # freed twice
+    with pytest.raises(CacheError, match="not live"):
+        c.length(a)
+    with pytest.raises(CacheError):
+        c.reserve(7, 1)
+    with pytest.raises(CacheError, match="at least one token"):
+        c.reserve(b, 0)
+    assert c.acquire() == a and c.length(a) == 0     # the slot is used again, empty
+    c.check()
+
+
+def test_position_range():
+    c = make(max_tokens=1024, max_positions=100)
+    s = c.acquire()
+    c.reserve(s, 100)
+    c.commit(s, 100)
+    with pytest.raises(CacheError, match="KV overflow"):
+        c.reserve(s, 1)
+
+
+def test_page_table_follows_each_sequence():
+    c = make(max_tokens=64 * 8)
+    a, b = c.acquire(), c.acquire()
+    c.reserve(a, 65); c.commit(a, 65)
+    c.reserve(b, 10); c.commit(b, 10)
+    c.reserve(a, 64); c.commit(a, 64)                # a grows after b took a page: its pages are not adjacent
+    t = c.page_table(0, [b, a])
+    assert t.shape == (2, 3) and t.dtype.name == "int32"
+    assert t[1].tolist() == [0, 1, 3] and t[0].tolist()[0] == 2
+    assert c.page_table(0, [a], width=5).shape == (1, 5)
+    with pytest.raises(CacheError):
+        c.page_table(0, [a], width=2)
+
+
+def test_window_group_gives_pages_back_early():
+    c = make(max_tokens=64 * 6, needs=[KvNeed(1, 16), KvNeed(1, 16, window=70)])
+    s = c.acquire()
+    c.reserve(s, 200); c.commit(s, 200)
+    full, win = c.groups[0].pool, c.groups[1].pool
+    assert full.free_pages == 2
+    # the next query sits at 200 and sees keys 131..200: pages 0 and 1 (keys 0..127) are out of reach
+    assert win.free_pages == 4
+    assert c.page_table(1, [s])[0].tolist() == [0, 0, 2, 3] or c.page_table(1, [s])[0].tolist()[2:] == [2, 3]
+    c.check()
+    c.release(s)
+    assert full.free_pages == win.free_pages == 6
+    c.check()
+
+
+def test_state_is_zeroed_when_a_slot_is_taken():
+    c = make(needs=[StateNeed((4,))], max_slots=2)
+    s = c.acquire()
+    c.layer_view(0).state[s] += 5
+    c.release(s)
+    s2 = c.acquire()
+    assert s2 == s and float(c.layer_view(0).state[s2].abs().sum()) == 0.0
+
+
+def test_random_walk_keeps_every_invariant():
+    rng = random.Random(0)
+    c = make(max_tokens=64 * 40, max_slots=12, needs=[KvNeed(2, 16), KvNeed(2, 16, window=130)])
+    live = {}
+    for _ in range(3000):
+        op = rng.random()
+        if op < 0.25 and c.free_slots:
+            live[c.acquire()] = 0
+        elif op < 0.45 and live:
+            s = rng.choice(list(live))
+            c.release(s)
+            del live[s]
+        elif live:
+            s = rng.choice(list(live))
+            n = rng.choice([1, 1, 1, 5, 64, 100])
+            try:
+                c.reserve(s, n)
+                c.commit(s, n)
+                live[s] += n
+            except CacheFull:
+                pass
+        assert sorted(live) == c.live_slots
+        for s, n in live.items():
+            assert c.length(s) == n
+    c.check()
+    held = sum(pages_for(n) for n in live.values())
+    assert c.groups[0].pool.free_pages <= 40 - held       # reserved pages may exceed the committed ones
+    for s in list(live):
+        c.release(s)
+    c.check()
+    assert c.free_slots == 12 and all(g.pool.free_pages == 40 for g in c.groups)

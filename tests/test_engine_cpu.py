@@ -1,0 +1,89 @@
+"""The engine's own logic (packing, page tables, slots, order of layers, generation) with the
+stand-in kernels on the CPU, against the plain implementation."""
+import pytest
+import torch
+
+import cpu_kernels
+import scenarios
+from helpers import model_folder, CONFIGS
+from synaptix_amd import StepError, CacheError, CacheFull
+
+
+@pytest.fixture(autouse=True)
+def kernels_on_cpu(monkeypatch):
+    cpu_kernels.install(monkeypatch)
+
+
+def make_engine(name, dtype, max_tokens, sharp=False, max_slots=None):
+    return cpu_kernels.CpuEngine.load(model_folder(name, sharp), dtype=dtype, max_tokens=max_tokens, device="cpu",
+                                      max_slots=max_slots)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_whole(name):
+    scenarios.whole(make_engine, name, "float32")
+
+
+def test_whole_sharp_attention():
+    scenarios.whole(make_engine, "C", "float32", sharp=True)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_last_tokens_one_by_one(name):
+    scenarios.last_tokens_one_by_one(make_engine, name, "float32", tail=8)
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("B", "bfloat16")])
+def test_unequal_batches(name, dtype):
+    scenarios.unequal_batches(make_engine, name, dtype, decode=5)
+
+
+def test_first_tokens():
+    scenarios.first_tokens(make_engine, "B", "float32")
+
+
+def test_greedy_and_sampled_generation():
+    scenarios.greedy_generation(make_engine, "A", "float32", n_new=5)
+    scenarios.sampled_generation(make_engine, "B", "float32")
+
+
+def test_step_errors():
+    eng = make_engine("A", "float32", 256, max_slots=2)
+    s = eng.acquire()
+    with pytest.raises(StepError, match="vocabulary"):
+        eng.step([(s, [1, 512])])
+    with pytest.raises(StepError, match="vocabulary"):
+        eng.step([(s, [-1])])
+    with pytest.raises(StepError, match="at least one token"):
+        eng.step([(s, [])])
+    with pytest.raises(StepError, match="at least one sequence"):
+        eng.step([])
+    with pytest.raises(StepError, match="twice"):
+        eng.step([(s, [1]), (s, [2])])
+    with pytest.raises(CacheError, match="not live"):
+        eng.step([(1, [1])])
+    with pytest.raises(StepError, match="place 3"):
+        eng.step([(s, [1, 2, 3])], want=[[3]])
+    with pytest.raises(StepError, match="one list of places"):
+        eng.step([(s, [1, 2, 3])], want=[[0], [1]])
+    assert eng.length(s) == 0                                   # nothing of the above touched the cache
+    with pytest.raises(CacheError, match="KV overflow"):
+        eng.step([(s, [1] * 257)])                              # max_position_embeddings = 256
+    t = eng.acquire()
+    eng.step([(s, [1] * 200)])
+    with pytest.raises(CacheFull):
+        eng.step([(t, [1] * 65)])                               # 4 pages in all; s holds 4... none left
+    assert eng.length(t) == 0 and eng.length(s) == 200
+    eng.cache.check()
+
+
+def test_batch_rows_do_not_depend_on_their_neighbours():
+    """Permuting a batch permutes its logits bit for bit (no padding, nothing shared between rows)."""
+    eng = make_engine("A", "float32", 1024)
+    V = CONFIGS["A"]["vocab_size"]
+    prompts = [scenarios.random_tokens(V, n, 50 + n) for n in (9, 2, 30)]
+    a = [eng.acquire() for _ in prompts]
+    x = eng.step(list(zip(a, prompts)), want="last")
+    b = [eng.acquire() for _ in prompts]
+    y = eng.step(list(zip(b, prompts))[::-1], want="last")
+    assert torch.equal(x, y.flip(0))

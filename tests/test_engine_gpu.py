@@ -1,0 +1,142 @@
+"""The engine on the GPU against the plain implementation, in 32-bit and in bfloat16: each
+request alone and whole; with the last 32 tokens one by one; in batches of unequal lengths one
+after another (slots used again); long decoding; the first tokens; generation; the replay
+program as a user runs it."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import scenarios
+from helpers import (model_folder, CONFIGS, plain_logits, random_tokens, assert_logits_close, run_trace,
+                     batched_trace)
+
+pytestmark = pytest.mark.gpu
+DTYPES = ["float32", "bfloat16"]
+
+
+@pytest.fixture(scope="module", autouse=True)
+def need_gpu():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+
+
+_engines = {}
+
+
+def make_engine(name, dtype, max_tokens, sharp=False, max_slots=None):
+    from synaptix_amd import Engine
+    return Engine.load(model_folder(name, sharp), dtype=dtype, max_tokens=max_tokens, max_slots=max_slots)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole(name, dtype):
+    scenarios.whole(make_engine, name, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_whole_with_peaked_attention(dtype):
+    """q/k gains 3 x larger: attention picks single keys, so a wrong key or page shows."""
+    scenarios.whole(make_engine, "C", dtype, sharp=True)
+    scenarios.unequal_batches(make_engine, "B", dtype, sharp=True)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_last_32_tokens_one_by_one(name, dtype):
+    scenarios.last_tokens_one_by_one(make_engine, name, dtype, tail=32)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_unequal_batches_one_after_another(name, dtype):
+    scenarios.unequal_batches(make_engine, name, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,n", [("A", 250), ("B", 400), ("C", 300)])
+def test_long_decoding(name, n, dtype):
+    scenarios.long_decoding(make_engine, name, dtype, n)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_first_tokens(name, dtype):
+    scenarios.first_tokens(make_engine, name, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation(name, dtype):
+    scenarios.greedy_generation(make_engine, name, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sampled_generation(dtype):
+    scenarios.sampled_generation(make_engine, "B", dtype)
+
+
+def test_batch_rows_do_not_depend_on_their_neighbours():
+    """The same request alone, and between others in another slot and other pages."""
+    for dtype in DTYPES:
+        eng = make_engine("B", dtype, 4096)
+        V = CONFIGS["B"]["vocab_size"]
+        mine = random_tokens(V, 77, 1)
+        s = eng.acquire()
+        alone = eng.step([(s, mine)], want="all")
+        others = [random_tokens(V, n, 2 + n) for n in (130, 5)]
+        a, b, c = eng.acquire(), eng.acquire(), eng.acquire()
+        lg = eng.step([(a, others[0]), (b, mine), (c, others[1])], want=[[], list(range(77)), []])
+        # no padding and no shared reductions: the rows of a request are the same numbers
+        assert float((lg - alone).abs().max()) <= (1e-5 if dtype == "float32" else 2e-2)
+
+
+# ----------------------------------------------------------------------------- the replay program
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_trace_run_whole_one_by_one_and_batched(tmp_path, dtype):
+    """bin/trace_run as a user starts it: requests whole; with their last 32 tokens one by one;
+    and in batches of unequal lengths, one batch after another, with max-tokens so tight that
+    the second batch needs the pages of the first."""
+    name = "B"
+    folder = model_folder(name)
+    V = CONFIGS[name]["vocab_size"]
+    reqs = {f"q{i}": random_tokens(V, n, 400 + i) for i, n in enumerate([40, 97, 33, 150, 64])}
+    # whole
+    steps = [{"step": i, "entries": [{"id": r, "tokens": t, "want": list(range(len(t)))}], "end": [r]}
+             for i, (r, t) in enumerate(reqs.items())]
+    out = run_trace(folder, dtype, steps, 192, str(tmp_path / "whole"))
+    for i, (r, t) in enumerate(reqs.items()):
+        assert_logits_close(out[i], plain_logits(name, t), dtype, f"trace whole {r}")
+    # last 32 one by one, each request alone
+    steps, where = batched_trace(reqs, [[r] for r in reqs], decode=32)
+    out = run_trace(folder, dtype, steps, 192, str(tmp_path / "tail"))
+    for r, t in reqs.items():
+        got = np.stack([out[where[(r, p)][0]][where[(r, p)][1]] for p in range(len(t))])
+        assert_logits_close(got, plain_logits(name, t), dtype, f"trace last 32 {r}")
+    # unequal batches; q3 (150 tokens, 3 pages) + q0 + q1 (1 + 2 pages) fill 6 pages exactly
+    batches = [["q3", "q0", "q1"], ["q2", "q4", "q1"], ["q4", "q3"]]
+    steps, where = batched_trace(reqs, batches, decode=32)
+    out = run_trace(folder, dtype, steps, 64 * 6, str(tmp_path / "batched"))
+    for batch in batches:
+        pass
+    seen = set()
+    for (r, p), (st, row) in where.items():
+        seen.add(r)
+    for r in seen:
+        t = reqs[r]
+        got = np.stack([out[where[(r, p)][0]][where[(r, p)][1]] for p in range(len(t))])
+        assert_logits_close(got, plain_logits(name, t), dtype, f"trace batched {r}")
+
+
+def test_trace_run_steps_without_wants_write_no_file(tmp_path):
+    folder = model_folder("A")
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": [1, 2, 3], "want": []}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": [4], "want": [0]}], "end": ["x"]},
+             {"step": 2, "entries": [], "end": []}]
+    out = run_trace(folder, "float32", steps, 64, str(tmp_path / "o"))
+    assert sorted(out) == [1]
+    assert_logits_close(out[1], plain_logits("A", [1, 2, 3, 4])[3:], "float32", "after a silent step")
+    assert not os.path.exists(tmp_path / "o" / "0.f32")

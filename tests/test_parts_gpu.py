@@ -1,0 +1,224 @@
+"""Each part alone against the plain implementation's function for it, and the framework's
+openness: a toy mixer with a state of its own, defined here, is registered, built and stepped
+without a change to the package."""
+import math
+
+import pytest
+import torch
+
+import plain_qwen3 as P
+from helpers import assert_logits_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+F32, BF16 = torch.float32, torch.bfloat16
+
+
+@pytest.fixture(scope="module", autouse=True)
+def need_gpu():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+
+
+def rnd(shape, seed, scale=1.0):
+    return torch.randn(shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+def tol(dtype):
+    return dict(atol=1e-5, rtol=1e-5) if dtype == F32 else dict(atol=3e-2, rtol=2e-2)
+
+
+def one_sequence_ctx(cache, slot, n_new, dtype):
+    """A StepContext for one sequence that brings n_new tokens, as the engine builds it."""
+    import numpy as np
+    from synaptix_amd.engine.batch import StepLayout, StepContext, fill_host_buffer
+    past = cache.length(slot)
+    cache.reserve(slot, n_new)
+    tables = [cache.page_table(g, [slot]) for g in range(len(cache.groups))]
+    layout = StepLayout(n_new, 1, 0, [t.shape[1] for t in tables])
+    host = np.zeros(layout.total, dtype=np.int32)
+    fill_host_buffer(layout, host, [np.zeros(n_new, dtype=np.int64)], [past], [slot], [], tables)
+    return StepContext(layout, torch.from_numpy(host).to(DEV), dtype, [slot], [past], [n_new], {})
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_rms_norm_part(dtype):
+    from synaptix_amd.parts import RmsNorm
+    n = RmsNorm("g", 72, 1e-5)
+    gain = 1 + 0.1 * rnd((72,), 1)
+    n.load(lambda name: gain.to(dtype).to(DEV))
+    resid, delta = rnd((5, 72), 2), rnd((5, 72), 3)
+    r = resid.to(DEV)
+    out = n.add_apply(r, delta.to(DEV), dtype)
+    want = P.rms_norm(resid + delta, gain.to(dtype).float(), 1e-5)
+    assert torch.allclose(out.float().cpu(), want, **tol(dtype))
+    assert torch.allclose(r.cpu(), resid + delta, atol=1e-6)
+    x = rnd((4, 3, 72), 4).to(dtype)
+    assert torch.allclose(n.apply(x.to(DEV)).float().cpu(), P.rms_norm(x.float(), gain.to(dtype).float(), 1e-5),
+                          **tol(dtype))
+
+
+def test_rotary_part_tables():
+    from synaptix_amd.parts import RotaryHalfSplit
+    r = RotaryHalfSplit(1e6, 32, 300)
+    cos, sin = r.tables(DEV)
+    c, s = P.rope_tables(32, 300, 1e6)
+    assert cos.shape == (300, 16)
+    assert torch.allclose(cos.cpu(), c, atol=1e-6) and torch.allclose(sin.cpu(), s, atol=1e-6)
+    with pytest.raises(ValueError):
+        RotaryHalfSplit(1e4, 15, 10)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("nh,nkv,hd,rot,qk_norm,window", [(4, 2, 16, 16, True, None), (6, 2, 48, 32, False, None),
+                                                           (3, 1, 32, 32, True, 20), (4, 4, 64, 0, True, None)])
+def test_attention_part_alone(dtype, nh, nkv, hd, rot, qk_norm, window):
+    """GqaAttention with its own sizes and options (partial rotation, no q/k norm, a window, no
+    rotation at all), a prompt and then single tokens, against the plain functions."""
+    from synaptix_amd.parts import GqaAttention, RotaryHalfSplit, NoPosition
+    from synaptix_amd.cache import SequenceCache
+    H, S, eps = 40, 90, 1e-5
+    pos = RotaryHalfSplit(1e4, rot, 256) if rot else NoPosition()
+    att = GqaAttention("a.", H, nh, nkv, hd, position=pos, qk_norm_eps=eps if qk_norm else None, window=window)
+    w = {n: (rnd(s.shape, 10 + i, 0.3) if s.kind != "gain" else 1 + 0.1 * rnd(s.shape, 10 + i)).to(dtype)
+         for i, (n, s) in enumerate(att.tensor_specs().items())}
+    att.load(lambda name: w[name].to(DEV))
+    x = rnd((S, H), 30).to(dtype)
+
+    # the plain statement of the same part
+    xf = x.float()
+    q = (xf @ w["a.q_proj.weight"].float().T).view(S, nh, hd)
+    k = (xf @ w["a.k_proj.weight"].float().T).view(S, nkv, hd)
+    v = (xf @ w["a.v_proj.weight"].float().T).view(S, nkv, hd)
+    if qk_norm:
+        q, k = P.rms_norm(q, w["a.q_norm.weight"].float(), eps), P.rms_norm(k, w["a.k_norm.weight"].float(), eps)
+    if rot:
+        cos, sin = P.rope_tables(rot, S, 1e4)
+        q = torch.cat([P.apply_rope(q[..., :rot], cos, sin, range(S)), q[..., rot:]], -1)
+        k = torch.cat([P.apply_rope(k[..., :rot], cos, sin, range(S)), k[..., rot:]], -1)
+    want = P.attention(q, k, v, 1 / math.sqrt(hd), list(range(S)), window=window).reshape(S, nh * hd) \
+        @ w["a.o_proj.weight"].float().T
+
+    cache = SequenceCache([att.cache_need()], 256, 2, dtype, DEV)
+    slot = cache.acquire()
+    got = []
+    for lo, hi in [(0, 70)] + [(i, i + 1) for i in range(70, S)]:
+        ctx = one_sequence_ctx(cache, slot, hi - lo, dtype)
+        got.append(att.forward(x[lo:hi].to(DEV), ctx, cache.layer_view(0)))
+        cache.commit(slot, hi - lo)
+    got = torch.cat(got).cpu()
+    assert got.dtype == F32
+    err = (got - want).abs().max()
+    assert err <= (2e-4 if dtype == F32 else 4e-2) * max(1.0, float(want.abs().max())), float(err)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_gated_mlp_part_alone(dtype):
+    from synaptix_amd.parts import GatedMlp
+    ff = GatedMlp("m.", 56, 200)
+    w = {n: rnd(s.shape, 40 + i, 0.2).to(dtype) for i, (n, s) in enumerate(ff.tensor_specs().items())}
+    ff.load(lambda name: w[name].to(DEV))
+    x = rnd((9, 56), 50).to(dtype)
+    got = ff.forward(x.to(DEV), None).cpu()
+    want = P.swiglu_mlp(x.float(), w["m.gate_proj.weight"].float(), w["m.up_proj.weight"].float(),
+                        w["m.down_proj.weight"].float())
+    assert (got - want).abs().max() <= (1e-4 if dtype == F32 else 3e-2)
+    with pytest.raises(ValueError, match="gelu"):
+        GatedMlp("m.", 8, 8, "gelu")
+
+
+# ----------------------------------------------------------------------------- a toy architecture
+def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
+    """A decayed running mean of the inputs as 'mixer': state [hidden] for each sequence, zero at
+    the start.  It is defined, registered under a name of its own, built from its own config.json,
+    loaded and stepped here; whole prompts and single tokens must agree, which they only do if the
+    state is kept for each slot, zeroed when a slot is taken, and carried across steps."""
+    from dataclasses import dataclass, asdict
+    import json
+    from synaptix_amd import register_architecture, Engine
+    from synaptix_amd.models import DecoderModel, LayerRun, TokenEmbedding, OutputHead
+    from synaptix_amd.parts import Mixer, StateNeed, RmsNorm, GatedMlp, PreNormBlock, GqaAttention, RotaryHalfSplit
+    from synaptix_amd.weights import TensorSpec, save_file, RandomSource
+
+    class RunningMean(Mixer):
+        def __init__(self, prefix, hidden, decay):
+            self.prefix, self.hidden, self.decay = prefix, hidden, decay
+            self.scale = None
+
+        def tensor_specs(self):
+            return {self.prefix + "scale": TensorSpec((self.hidden,), "gain")}
+
+        def load(self, get):
+            self.scale = get(self.prefix + "scale").float()
+
+        def cache_need(self):
+            return StateNeed((self.hidden,), torch.float32)
+
+        def forward(self, h, ctx, cache, owner=True):
+            out = torch.empty(h.shape, dtype=torch.float32, device=h.device)
+            start = 0
+            for slot, n in zip(ctx.slots, ctx.new_counts):       # tokens of a sequence in order
+                s = cache.state[slot]
+                for t in range(start, start + n):
+                    s.mul_(self.decay).add_(h[t].float())
+                    out[t] = s * self.scale
+                start += n
+            return out
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        vocab_size: int = 97
+        hidden_size: int = 48
+        intermediate_size: int = 80
+        decay: float = 0.5
+        max_position_embeddings: int = 128
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(**{k: d[k] for k in cls.__dataclass_fields__ if k in d})
+
+        def to_dict(self):
+            return {**asdict(self), "architectures": ["ToyRunningMean"]}
+
+    def build(cfg, max_positions=None):
+        emb = TokenEmbedding("emb", cfg.vocab_size, cfg.hidden_size)
+        rope = RotaryHalfSplit(1e4, 16, cfg.max_position_embeddings)
+        blocks = [
+            PreNormBlock(RmsNorm("l0.n1", cfg.hidden_size, 1e-5), RunningMean("l0.mix.", cfg.hidden_size, cfg.decay),
+                         RmsNorm("l0.n2", cfg.hidden_size, 1e-5), GatedMlp("l0.ff.", cfg.hidden_size, cfg.intermediate_size)),
+            PreNormBlock(RmsNorm("l1.n1", cfg.hidden_size, 1e-5),
+                         GqaAttention("l1.att.", cfg.hidden_size, 3, 1, 16, position=rope),
+                         RmsNorm("l1.n2", cfg.hidden_size, 1e-5), GatedMlp("l1.ff.", cfg.hidden_size, cfg.intermediate_size)),
+        ]
+        # the stateful block runs twice, each run with a state of its own; the attention block runs once
+        schedule = [LayerRun(0, 0), LayerRun(1, 1), LayerRun(0, 2)]
+        return DecoderModel(cfg, emb, blocks, schedule, RmsNorm("norm", cfg.hidden_size, 1e-5),
+                            OutputHead("head", cfg.vocab_size, cfg.hidden_size))
+
+    register_architecture("ToyRunningMean", ToyConfig, build)
+    cfg = ToyConfig()
+    model = build(cfg)
+    src = RandomSource(model.tensor_specs(), 5, std=0.2)
+    save_file({n: src.tensor(n) for n in src.names()}, str(tmp_path / "model.safetensors"))
+    (tmp_path / "config.json").write_text(json.dumps(cfg.to_dict()))
+
+    for dtype in ("float32", "bfloat16"):
+        eng = Engine.load(str(tmp_path), dtype=dtype, max_tokens=512, max_slots=3)
+        assert [type(n).__name__ for n in eng.model.cache_needs()] == ["StateNeed", "KvNeed", "StateNeed"]
+        toks = [[5, 9, 33, 2, 70, 11, 8], [90, 1, 4]]
+        a, b = eng.acquire(), eng.acquire()
+        whole = eng.step([(a, toks[0]), (b, toks[1])], want="all")
+        eng.release(a), eng.release(b)
+        b2, a2 = eng.acquire(), eng.acquire()                   # the same slots again, the other way round
+        got = {0: [], 1: []}
+        lg = eng.step([(a2, toks[0][:2]), (b2, toks[1][:1])], want="all")
+        got[0].append(lg[:2]), got[1].append(lg[2:])
+        for i in range(2, 7):
+            ent = [(a2, [toks[0][i]])] + ([(b2, [toks[1][i - 1]])] if i - 1 < 3 else [])
+            lg = eng.step(ent, want="last")
+            got[0].append(lg[:1])
+            if len(ent) > 1:
+                got[1].append(lg[1:])
+        tolerance = 1e-4 if dtype == "float32" else 5e-2
+        assert (torch.cat(got[0]) - whole[:7]).abs().max() <= tolerance
+        assert (torch.cat(got[1]) - whole[7:]).abs().max() <= tolerance

@@ -1,0 +1,225 @@
+"""What fixes the plain implementation beside the reference's text: vectors the reference's own
+tests hold, special cases that reduce to a library routine, and invariants.  Each is chosen so
+that a plausible mistake (a wrong sign or pairing, eps outside the root, a norm in the wrong
+place) fails it."""
+import math
+
+import pytest
+import torch
+
+import plain_qwen3 as P
+from helpers import plain_model, random_tokens, CONFIGS
+
+F64 = torch.float64
+
+
+def rnd(shape, seed, dtype=torch.float32):
+    return torch.randn(shape, generator=torch.Generator().manual_seed(seed)).to(dtype)
+
+
+# ----------------------------------------------------------------------------- RMSNorm
+def test_rms_norm_reference_vector():
+    """crates/synaptix-ops/tests/rms_norm.rs:76-95: shape [2,3,4], x_i = 0.1 i - 1, w = [0.5,-0.25,1,2]."""
+    x = torch.tensor([i * 0.1 - 1.0 for i in range(24)]).view(2, 3, 4)
+    w = torch.tensor([0.5, -0.25, 1.0, 2.0])
+    got = P.rms_norm(x, w, 1e-6)
+    xd = x.double()
+    want = xd * (1.0 / torch.sqrt((xd * xd).mean(-1, keepdim=True) + 1e-6)) * w.double()
+    assert (got.double() - want).abs().max() < 1e-5
+    # first row by hand: x = [-1, -.9, -.8, -.7], mean x^2 = 0.735
+    r = 1 / math.sqrt(0.735 + 1e-6)
+    assert torch.allclose(got[0, 0], torch.tensor([-1 * r * 0.5, 0.9 * r * 0.25, -0.8 * r, -0.7 * r * 2]), atol=1e-6)
+
+
+def test_rms_norm_properties():
+    x = rnd((5, 32), 1)
+    y = P.rms_norm(x, torch.ones(32), 1e-12)
+    assert torch.allclose((y * y).mean(-1), torch.ones(5), atol=1e-5)            # unit RMS with unit gain
+    assert torch.allclose(P.rms_norm(7.0 * x, torch.ones(32), 1e-12), y, atol=1e-5)  # scale invariance
+    # eps inside the root: tiny x separates sqrt(m + eps) from sqrt(m) + eps and from no eps at all
+    t = torch.full((1, 8), 1e-4)
+    assert abs(float(P.rms_norm(t, torch.ones(8), 1e-6)[0, 0]) - 1e-4 / math.sqrt(1e-8 + 1e-6)) < 1e-9
+    # plain gain, not 1 + w
+    assert torch.allclose(P.rms_norm(x, torch.zeros(32), 1e-6), torch.zeros(5, 32))
+
+
+# ----------------------------------------------------------------------------- rotation
+def test_rope_position_zero_and_norm():
+    """crates/synaptix-ops/tests/pos.rs:11-57: position 0 is the identity; norms are kept."""
+    cos, sin = P.rope_tables(16, 50, 1e4)
+    x = rnd((6, 3, 16), 2)
+    assert torch.allclose(P.apply_rope(x, cos, sin, [0] * 6), x, atol=1e-7)
+    y = P.apply_rope(x, cos, sin, [3, 7, 11, 19, 30, 49])
+    assert torch.allclose((y * y).sum(-1), (x * x).sum(-1), rtol=1e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("theta,hd", [(1e4, 16), (1e6, 32)])
+def test_rope_is_complex_multiplication_of_split_pairs(theta, hd):
+    """Pair (d, d + hd/2) turns by p * theta^(-2d/hd): (x_d + i x_{d+hd/2}) * e^{i p f_d}.
+    An interleaved pairing, a wrong sign or a wrong exponent fails."""
+    cos, sin = P.rope_tables(hd, 40, theta, F64)
+    x = rnd((1, 1, hd), 3, F64)
+    p = 17
+    y = P.apply_rope(x, cos, sin, [p])[0, 0]
+    half = hd // 2
+    z = torch.complex(x[0, 0, :half], x[0, 0, half:])
+    f = torch.tensor([theta ** (-2.0 * d / hd) for d in range(half)], dtype=F64)
+    zr = z * torch.exp(1j * p * f)
+    assert torch.allclose(y[:half], zr.real, atol=1e-12) and torch.allclose(y[half:], zr.imag, atol=1e-12)
+
+
+def test_rope_scores_depend_on_distance_only():
+    cos, sin = P.rope_tables(32, 200, 1e6, F64)
+    q, k = rnd((1, 1, 32), 4, F64), rnd((1, 1, 32), 5, F64)
+    def score(pq, pk):
+        return float((P.apply_rope(q, cos, sin, [pq]) * P.apply_rope(k, cos, sin, [pk])).sum())
+    assert abs(score(10, 3) - score(110, 103)) < 1e-9
+    assert abs(score(10, 3) - score(3, 10)) > 1e-3      # not symmetric: the sign of the angle matters
+
+
+# ----------------------------------------------------------------------------- attention
+def test_attention_reduces_to_library_softmax_attention():
+    """One kv head a q head, no mask effect on the last query: equals torch's SDPA with a causal mask."""
+    S, nh, hd = 9, 3, 8
+    q, k, v = rnd((S, nh, hd), 6), rnd((S, nh, hd), 7), rnd((S, nh, hd), 8)
+    got = P.attention(q, k, v, 1 / math.sqrt(hd), list(range(S)))
+    want = torch.nn.functional.scaled_dot_product_attention(q.transpose(0, 1), k.transpose(0, 1), v.transpose(0, 1),
+                                                            is_causal=True).transpose(0, 1)
+    assert torch.allclose(got, want, atol=1e-5)
+
+
+def test_attention_special_cases():
+    hd = 4
+    q, k, v = rnd((1, 2, hd), 9), rnd((1, 1, hd), 10), rnd((1, 1, hd), 11)
+    # one key: the output is its value, for every head of the group
+    o = P.attention(q, k, v, 0.5, [0])
+    assert torch.allclose(o[0, 0], v[0, 0]) and torch.allclose(o[0, 1], v[0, 0])
+    # equal scores: the mean of the visible values
+    T = 6
+    kk, vv = torch.zeros(T, 1, hd), rnd((T, 1, hd), 12)
+    o = P.attention(rnd((1, 1, hd), 13), kk, vv, 1.0, [3])
+    assert torch.allclose(o[0, 0], vv[:4, 0].mean(0), atol=1e-6)
+    # a window of 2 sees keys p-1 and p only
+    o = P.attention(rnd((1, 1, hd), 13), kk, vv, 1.0, [3], window=2)
+    assert torch.allclose(o[0, 0], vv[2:4, 0].mean(0), atol=1e-6)
+
+
+def test_attention_gqa_is_mha_with_repeated_kv():
+    """crates/synaptix-models/llm/common/src/model.rs:2569-2579: kv heads repeated g times, head h -> h // g."""
+    S, nh, nkv, hd = 7, 6, 2, 8
+    q, k, v = rnd((S, nh, hd), 14), rnd((S, nkv, hd), 15), rnd((S, nkv, hd), 16)
+    a = P.attention(q, k, v, 0.3, list(range(S)))
+    b = P.attention(q, k.repeat_interleave(3, 1), v.repeat_interleave(3, 1), 0.3, list(range(S)))
+    assert torch.allclose(a, b, atol=1e-6)
+
+
+def test_attention_decode_shape_of_the_reference():
+    """(b,nh,nkv,Tq,Tkv,d) = (1,4,2,8,200,64), a chunk of 8 queries at the end of 200 keys:
+    q_pos = Tkv - Tq + i (crates/synaptix-kernels-cuda/tests/cuda_flash_decode.rs:32-90,185-240)."""
+    nh, nkv, Tq, T, hd = 4, 2, 8, 200, 64
+    q, k, v = rnd((Tq, nh, hd), 17), rnd((T, nkv, hd), 18), rnd((T, nkv, hd), 19)
+    got = P.attention(q, k, v, 1 / 8.0, [T - Tq + i for i in range(Tq)])
+    # the host reference of that test, restated directly
+    for i in (0, 7):
+        for h in (0, 3):
+            qp = T - Tq + i
+            s = (k[:qp + 1, h // 2] @ q[i, h]) / 8.0
+            want = torch.softmax(s, 0) @ v[:qp + 1, h // 2]
+            assert torch.allclose(got[i, h], want, atol=1e-5)
+
+
+# ----------------------------------------------------------------------------- feed-forward
+def test_swiglu():
+    z = rnd((20,), 20)
+    assert torch.allclose(P.silu(z), z * torch.sigmoid(z), atol=1e-6)
+    H, I = 6, 10
+    h, wg, wu, wd = rnd((3, H), 21), rnd((I, H), 22), rnd((I, H), 23), rnd((H, I), 24)
+    want = (torch.nn.functional.silu(h @ wg.T) * (h @ wu.T)) @ wd.T
+    assert torch.allclose(P.swiglu_mlp(h, wg, wu, wd), want, atol=1e-5)
+    assert not torch.allclose(P.swiglu_mlp(h, wu, wg, wd), want, atol=1e-3)    # gate and up are not symmetric
+
+
+# ----------------------------------------------------------------------------- whole model
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_zeroed_projections_leave_embedding_norm_head(name):
+    """o_proj = down_proj = 0: x passes through, logits = RMSNorm(E[id]) . W_out^T: one line that
+    checks embedding, final norm, tied or separate output."""
+    m = plain_model(name)
+    w = dict(m.w)
+    for n in list(w):
+        if n.endswith("o_proj.weight") or n.endswith("down_proj.weight"):
+            w[n] = torch.zeros_like(w[n])
+    z = P.PlainQwen3(m.cfg, w)
+    ids = random_tokens(m.cfg["vocab_size"], 6, 1)
+    E = w["model.embed_tokens.weight"]
+    out = E if m.cfg["tie_word_embeddings"] else w["lm_head.weight"]
+    want = P.rms_norm(E[ids], w["model.norm.weight"], m.eps) @ out.T
+    assert torch.allclose(z.forward(ids), want, atol=1e-6)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_causality_and_prefix(name):
+    m = plain_model(name)
+    ids = random_tokens(m.cfg["vocab_size"], 12, 2)
+    full = m.forward(ids)
+    assert torch.allclose(m.forward(ids[:7]), full[:7], atol=1e-5)
+    other = ids[:7] + random_tokens(m.cfg["vocab_size"], 5, 3)
+    assert torch.allclose(m.forward(other)[:7], full[:7], atol=1e-5)
+
+
+def test_qk_norm_uses_the_layers_eps_and_sits_before_the_rotation():
+    """Config B has eps 1e-5 and q_norm != k_norm; swapping the two gains, or taking another eps
+    with tiny activations, changes the logits."""
+    m = plain_model("B")
+    ids = random_tokens(1000, 5, 4)
+    base = m.forward(ids)
+    w = dict(m.w)
+    a, b = "model.layers.0.self_attn.q_norm.weight", "model.layers.0.self_attn.k_norm.weight"
+    w[a], w[b] = m.w[b], m.w[a]
+    assert (P.PlainQwen3(m.cfg, w).forward(ids) - base).abs().max() > 1e-5
+
+
+def test_float64_agrees_with_float32():
+    m32 = plain_model("A")
+    m64 = P.PlainQwen3(m32.cfg, m32.w, dtype=F64)
+    ids = random_tokens(512, 20, 5)
+    assert (m32.forward(ids).double() - m64.forward(ids)).abs().max() < 2e-5
+
+
+# ----------------------------------------------------------------------------- sampling
+def test_philox_known_answer():
+    """crates/synaptix-ops/src/rng.rs:162-167: zero key, zero counter."""
+    assert P.philox4x32([0, 0, 0, 0], [0, 0]) == [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]
+    r = P.PlainPhilox(0)
+    assert [r.next_u32() for _ in range(4)] == [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]
+    assert r.counter == [1, 0, 0, 0]
+
+
+def test_greedy_takes_the_last_of_equal_maxima():
+    assert P.greedy(torch.tensor([1.0, 3.0, 2.0, 3.0, 0.0])) == 3
+    assert P.greedy(torch.tensor([5.0, 3.0])) == 0
+
+
+def test_repetition_vector_of_the_reference():
+    """crates/synaptix-infer/src/sampling/repetition.rs:88-97: penalty 2, last_n 2 -> [1,1,.5,.5]."""
+    got = P.repetition_penalty(torch.ones(4), [0, 1, 2, 3], 2.0, 2)
+    assert got.tolist() == [1.0, 1.0, 0.5, 0.5]
+    neg = P.repetition_penalty(torch.tensor([-1.0, 1.0]), [0, 0], 2.0, 0)
+    assert neg.tolist() == [-4.0, 1.0]                     # once for each occurrence
+    pf = P.presence_frequency(torch.zeros(3), [1, 1, 2], 0.5, 0.25, 0)
+    assert pf.tolist() == [0.0, -1.0, -0.75]
+
+
+def test_filters():
+    x = torch.tensor([1.0, 4.0, 2.0, 3.0])
+    assert P.top_k(x, 2).tolist() == [-math.inf, 4.0, -math.inf, 3.0]
+    # probabilities ~ [.03,.64,.09,.24]: p = .7 keeps 4.0 (sum before 0 <= .7) and 3.0 (.64 <= .7), drops the rest
+    assert P.top_p(x, 0.7).tolist() == [-math.inf, 4.0, -math.inf, 3.0]
+    assert P.min_p(x, 0.2).tolist() == [-math.inf, 4.0, -math.inf, 3.0]    # .24/.64 > .2 > .09/.64
+    assert P.multinomial(x, 0.0) == 0 and P.multinomial(x, 0.999999) == 3 and P.multinomial(x, 1.0) == 3
+
+
+def test_small_temperature_is_greedy():
+    x = rnd((50,), 30)
+    rng = P.PlainPhilox(3)
+    assert all(P.sample(x, [], rng, temperature=1e-3) == int(x.argmax()) for _ in range(5))
