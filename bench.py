@@ -1,0 +1,154 @@
+#!/usr/bin/env python3
+"""Throughput of the engine at the Qwen3-8B shape with random bf16 weights on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+
+A step is one decode step of `batch` sequences, each after a 2,048-token prompt of uniform ids,
+run through the same captured graph and host loop that generation uses.  One JSON line:
+decoded tokens a second at the batch, the prefill of one 2,048-token prompt (tokens a second and
+the fraction of the bf16 MFMA peak), the decode step against the HBM roofline (every weight it
+uses once plus the cache of the live requests, over its time), and decode at batch 1 and 64.
+
+Method after the reference's own harnesses (crates/synaptix-models/llm/qwen3/examples/format_perf.rs:41-122,
+crates/synaptix-cli/src/commands/bench.rs:35-96): synthetic ids, warm-up first, device synchronised
+at both ends of the timed region only.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X, published
+MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+QWEN3_8B = dict(num_hidden_layers=36, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                intermediate_size=12288, vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6,
+                max_position_embeddings=8192, tie_word_embeddings=False, eos_token_id=None, bos_token_id=None)
+PROMPT = 2048
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=QWEN3_8B["num_hidden_layers"],
+                    help="fewer layers than the model has (same layer sizes); both numbers are reported")
+    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    from synaptix_amd import Qwen3Config, Engine
+
+    torch.manual_seed(0)
+    cfg = Qwen3Config.from_dict({**QWEN3_8B, "num_hidden_layers": args.layers})
+    batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
+    new_tokens = args.warmup + args.steps + 8
+    per_seq = (PROMPT + new_tokens + 63) // 64 * 64
+    eng = Engine.from_config(cfg, seed=0, dtype="bfloat16", max_tokens=max(batches) * per_seq, max_seq=8192)
+    g = torch.Generator().manual_seed(0)
+
+    def prompt():
+        return torch.randint(0, cfg.vocab_size, (PROMPT,), generator=g).tolist()
+
+    L, H, I, V = cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    nh, nkv, hd = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    layer_params = H * (nh + 2 * nkv) * hd + nh * hd * H + 3 * H * I
+    weight_bytes = 2 * (L * (layer_params + 2 * H + 2 * hd) + H + V * H)      # every weight a decode step reads
+    kv_bytes_per_token = eng.cache.bytes_per_token()
+
+    # ---- prefill of one 2,048-token prompt
+    times = []
+    for i in range(5):
+        s = eng.acquire()
+        toks = prompt()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.step([(s, toks)], want="last")
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        eng.release(s)
+    pre_s = statistics.median(times[2:])
+    pre_flops = 2 * PROMPT * L * layer_params + L * 4 * hd * nh * PROMPT * (PROMPT + 1) // 2 + 2 * V * H
+    prefill = {"value": round(PROMPT / pre_s, 1), "tokens": PROMPT, "ms": round(pre_s * 1e3, 3),
+               "frac": round(pre_flops / pre_s / MFMA_PEAK["bf16"], 4)}
+
+    # ---- decode
+    def decode(batch: int, warmup: int, steps: int):
+        slots = [eng.acquire() for _ in range(batch)]
+        for lo in range(0, batch, 8):                       # prompts go in steps of 8 sequences
+            part = slots[lo:lo + 8]
+            lg = eng.step([(s, prompt()) for s in part], want="last")
+            first = eng.sample(lg).cpu().tolist()
+            if lo == 0:
+                tokens = []
+            tokens += first
+        longest = PROMPT + warmup + steps + 8
+
+        def one_step(tokens):
+            if args.no_graph:
+                lg = eng.step([(s, [t]) for s, t in zip(slots, tokens)], want="last")
+                return eng.sample(lg).cpu().tolist()
+            return eng.decode_runner(batch, longest).step(slots, tokens)[0]
+
+        for _ in range(warmup):
+            tokens = one_step(tokens)
+        torch.cuda.synchronize()
+        len0 = sum(eng.length(s) for s in slots)
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            tokens = one_step(tokens)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        mean_ctx = len0 / batch + (steps - 1) / 2 + 1       # tokens a sequence holds when a step reads it
+        for s in slots:
+            eng.release(s)
+        step_bytes = weight_bytes + batch * mean_ctx * kv_bytes_per_token
+        return batch * steps / dt, dt / steps, step_bytes
+
+    points = {}
+    main_rate = main_step = main_bytes = None
+    for b in batches:
+        k = args.steps if b == args.batch else max(16, min(args.steps, 64))
+        w = args.warmup if b == args.batch else max(4, min(args.warmup, 8))
+        rate, step_s, step_bytes = decode(b, w, k)
+        if b == args.batch:
+            main_rate, main_step, main_bytes = rate, step_s, step_bytes
+        if b in (1, 64):
+            points[f"decode_b{b}"] = round(rate, 1)
+            points[f"decode_b{b}_hbm_frac"] = round(step_bytes / step_s / 1e9 / HBM_PEAK_GBS, 4)
+
+    achieved = main_bytes / main_step / 1e9
+    line = {
+        "metric": "decode tok/s at batch 8 (+ batch 1/64 in points) and prefill tok/s at 2048 tokens, Qwen3-8B shape bf16",
+        "value": round(main_rate, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(main_step * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic: seeded uniform token ids, random-init weights N(0, 0.02)",
+        "config": {"model": "Qwen3-8B shape", "layers": L, "model_layers": QWEN3_8B["num_hidden_layers"],
+                   "hidden": H, "heads": nh, "kv_heads": nkv, "head_dim": hd, "intermediate": I, "vocab": V,
+                   "global_batch": args.batch, "seq_len": PROMPT, "context": 8192, "new_tokens": args.steps,
+                   "tie_word_embeddings": False, "rope_theta": 1e6, "rms_norm_eps": 1e-6, "parallelism": "single GPU",
+                   "graph": not args.no_graph},
+        "prefill": prefill,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -46,6 +46,7 @@ class _Group:
     pool: PagePool
     k: torch.Tensor = None
     v: torch.Tensor = None
+    spare_page: int = 0               # a page beyond the pool that no sequence owns (padding rows write there)
 
 
 @dataclass
@@ -92,8 +93,9 @@ class SequenceCache:
         for g in self.groups:
             n, nd = len(g.layers), g.need
             # zeros: what a kernel may touch beyond a sequence's end is at least a number
-            g.k = torch.zeros((n, self.n_pages, nd.kv_heads, PAGE_TOKENS, nd.head_dim), dtype=dtype, device=self.device)
-            g.v = torch.zeros((n, self.n_pages, nd.kv_heads, nd.head_dim, PAGE_TOKENS), dtype=dtype, device=self.device)
+            g.spare_page = self.n_pages
+            g.k = torch.zeros((n, self.n_pages + 1, nd.kv_heads, PAGE_TOKENS, nd.head_dim), dtype=dtype, device=self.device)
+            g.v = torch.zeros((n, self.n_pages + 1, nd.kv_heads, nd.head_dim, PAGE_TOKENS), dtype=dtype, device=self.device)
         self._slots = [_Slot() for _ in range(self.max_slots)]
         self._free_slots = list(range(self.max_slots - 1, -1, -1))
 

@@ -55,6 +55,11 @@ class Engine:
         self._scratch = {}
         self._host = None
         self._dev = None
+        self._runners = {}
+        from ..parts.base import StateNeed
+        # a captured step is run more than once while it is recorded: only steps that write the
+        # same values again may be captured, which a mixer with a running state is not
+        self.graph_ok = not any(isinstance(n, StateNeed) for n in model.cache_needs())
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -177,6 +182,19 @@ class Engine:
         if logits is None:
             logits = torch.empty((0, self.vocab), dtype=torch.float32, device=self.device)
         return logits
+
+    def decode_runner(self, n_seqs: int, max_len: int):
+        """The captured decode step for up to n_seqs sequences of at most max_len tokens."""
+        from .graph import DecodeRunner, bucket_for
+        rows = bucket_for(n_seqs)
+        cap = max_len if self.max_positions is None else min(max_len, self.max_positions)
+        width = 1
+        while width < pages_for(cap):          # few distinct widths, so that graphs are shared
+            width *= 2
+        key = (rows, width)
+        if key not in self._runners:
+            self._runners[key] = DecodeRunner(self, rows, [width] * len(self.cache.groups))
+        return self._runners[key]
 
     def sample(self, logits, temperatures=None, uniforms=None) -> torch.Tensor:
         """Token ids (int32, device) for rows of logits; see kernels.ops.sample_rows."""

@@ -79,6 +79,25 @@ def plan_batch(waiting: list, prompt_lens: list, max_new: list, free_slots: int,
     return chosen
 
 
+def graph_step(engine, live, longest):
+    """One decode step through the captured graph; sampling runs inside it when every sequence
+    samples greedily or by temperature alone, else on the graph's logits."""
+    runner = engine.decode_runner(len(live), longest)
+    slots, last = [s.slot for s in live], [s.out[-1] for s in live]
+    if all(s.config.plain for s in live):
+        temps = [float(s.config.temperature) for s in live]
+        if all(t <= 0.0 for t in temps):
+            tokens, _ = runner.step(slots, last)
+        else:
+            u = [s.sampler.rng.next_multinomial_uniform() if t > 0.0 else 0.0 for s, t in zip(live, temps)]
+            tokens, _ = runner.step(slots, last, temps, u)
+        for s, t in zip(live, tokens):
+            s.sampler.commit(t)
+        return tokens
+    _, logits = runner.step(slots, last)
+    return sample_batch(logits, [s.sampler for s in live])
+
+
 class _Live:
     def __init__(self, request, slot, prompt, config, sampler):
         self.request, self.slot, self.prompt, self.config, self.sampler = request, slot, prompt, config, sampler
@@ -87,10 +106,12 @@ class _Live:
         self.finish = None
 
 
-def generate(engine, prompts, config=None, on_token=None, max_batch: int | None = None):
+def generate(engine, prompts, config=None, on_token=None, max_batch: int | None = None, use_graph: bool = True):
     """prompts: a list of token-id lists.  config: one GenerationConfig for all, or one each
     (with one for all, request i draws from the stream of seed + i).  on_token(request, token)
-    -> bool: False cancels that request.  Returns ([GenerationOutput], GenerationStats)."""
+    -> bool: False cancels that request.  use_graph: decode steps are replayed from a captured
+    graph where the engine allows it (the reference's --no-graph switches the same thing off).
+    Returns ([GenerationOutput], GenerationStats)."""
     if config is None:
         config = GenerationConfig()
     shared = isinstance(config, GenerationConfig)
@@ -156,6 +177,8 @@ def generate(engine, prompts, config=None, on_token=None, max_batch: int | None 
                     s.finish = "cancelled"
 
             # ---- one token a step for each live sequence
+            graph = use_graph and getattr(engine, "graph_ok", False)
+            longest = max(len(s.prompt) + max(s.config.max_new_tokens, 1) for s in live)
             t1 = time.perf_counter()
             while True:
                 still = []
@@ -178,8 +201,11 @@ def generate(engine, prompts, config=None, on_token=None, max_batch: int | None 
                 if not live:
                     break
                 ts = time.perf_counter()
-                lg = engine.step([(s.slot, [s.out[-1]]) for s in live], want="last")
-                tokens = sample_batch(lg, [s.sampler for s in live])
+                if graph:
+                    tokens = graph_step(engine, live, longest)
+                else:
+                    lg = engine.step([(s.slot, [s.out[-1]]) for s in live], want="last")
+                    tokens = sample_batch(lg, [s.sampler for s in live])
                 stats.step_ms.append((time.perf_counter() - ts) * 1000.0)
                 stats.decode_steps += 1
                 for s, t in zip(live, tokens):

@@ -1,0 +1,122 @@
+"""Decode steps replayed from a HIP graph.
+
+A decode step is some hundreds of small launches; launched one by one from the host they cost
+more than the step's work at small batch sizes.  The step for a fixed number of rows is
+therefore captured once and replayed; what changes from step to step (tokens, positions,
+lengths, page tables, temperatures, uniform numbers) lies in one device buffer that is
+refreshed by one copy before each replay.  The reference does the same for its single sequence
+(crates/synaptix-models/llm/qwen3/src/pipeline.rs:192-316, crates/synaptix-infer/src/graph_capture/capture.rs:24-122).
+
+Rows beyond the live sequences are padding: they run token 0 at position 0 against a spare
+cache page that no sequence owns, and their results are dropped.  No row reads another row's
+data, so padding changes no result.
+
+Captured are this package's kernels and torch's allocations only; no memset nodes.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from ..kernels import ops
+from .batch import StepLayout, StepContext
+
+
+def bucket_for(n: int) -> int:
+    """Row counts for which graphs are captured: powers of two up to 64, then multiples of 32."""
+    if n <= 64:
+        b = 1
+        while b < n:
+            b *= 2
+        return b
+    return (n + 31) // 32 * 32
+
+
+class DecodeRunner:
+    def __init__(self, engine, rows: int, widths: list):
+        self.engine, self.rows, self.widths = engine, rows, list(widths)
+        self.layout = StepLayout(rows, rows, rows, widths)
+        n_int = self.layout.total
+        self.total = n_int + 2 * rows                          # + temperatures and uniforms as float bits
+        dev = engine.device
+        self.dev = torch.zeros(self.total, dtype=torch.int32, device=dev)
+        self.host = [torch.zeros(self.total, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self.copied = [None, None]
+        self.turn = 0
+        self.temps = self.dev[n_int:n_int + rows].view(torch.float32)
+        self.uniforms = self.dev[n_int + rows:n_int + 2 * rows].view(torch.float32)
+        self.out_tokens = torch.zeros(rows, dtype=torch.int32, device=dev)
+        self.logits = None
+        self.graph = None
+        self.spare = [g.spare_page for g in engine.cache.groups]
+
+    def _fill(self, host: np.ndarray, slots, tokens, temps, uniforms):
+        lay, cache, R, B = self.layout, self.engine.cache, self.rows, len(slots)
+        o = lay.off
+        past = [cache.length(s) for s in slots]
+        host[o["tokens"][0]:o["tokens"][0] + R] = 0
+        host[o["tokens"][0]:o["tokens"][0] + B] = tokens
+        host[o["tok_seq"][0]:o["tok_seq"][0] + R] = np.arange(R, dtype=np.int32)
+        pos = np.zeros(R, dtype=np.int32)
+        pos[:B] = past
+        host[o["tok_pos"][0]:o["tok_pos"][0] + R] = pos
+        host[o["seq_start"][0]:o["seq_start"][0] + R + 1] = np.arange(R + 1, dtype=np.int32)
+        host[o["seq_past"][0]:o["seq_past"][0] + R] = pos
+        host[o["seq_len"][0]:o["seq_len"][0] + R] = pos + 1
+        sl = np.full(R, -1, dtype=np.int32)
+        sl[:B] = slots
+        host[o["seq_slot"][0]:o["seq_slot"][0] + R] = sl
+        host[o["want"][0]:o["want"][0] + R] = np.arange(R, dtype=np.int32)
+        for gi, ((off, n), w) in enumerate(zip(lay.table_off, lay.widths)):
+            tab = np.full((R, w), self.spare[gi], dtype=np.int32)
+            if B:
+                tab[:B] = cache.page_table(gi, slots, width=w)
+            host[off:off + n] = tab.reshape(-1)
+        f = host[lay.total:lay.total + 2 * R].view(np.float32)
+        f[:] = 0.0
+        if temps is not None:
+            f[:B] = temps
+            f[R:R + B] = uniforms
+        return past
+
+    def _forward(self, ctx):
+        eng = self.engine
+        logits = eng.model.forward(ctx, ctx.tokens, ctx.want, eng.cache)
+        ops.sample_rows(logits, self.temps, self.uniforms, self.out_tokens)
+        return logits
+
+    def step(self, slots, tokens, temps=None, uniforms=None):
+        """One token for each of `slots`; returns (sampled tokens as a host list, logits [B, V]).
+        temps None: greedy for every row."""
+        eng, B = self.engine, len(slots)
+        if B > self.rows:
+            raise ValueError(f"{B} sequences for a graph of {self.rows} rows")
+        for s in slots:
+            eng.cache.reserve(s, 1)
+        i = self.turn
+        self.turn ^= 1
+        if self.copied[i] is not None:
+            self.copied[i].synchronize()
+        past = self._fill(self.host[i].numpy(), slots, tokens, temps, uniforms)
+        self.dev.copy_(self.host[i], non_blocking=True)
+        self.copied[i] = torch.cuda.Event()
+        self.copied[i].record()
+        if self.graph is None:
+            ctx = StepContext(self.layout, self.dev, eng.dtype, [-1] * self.rows, [0] * self.rows, [1] * self.rows,
+                              eng._scratch)
+            ctx.max_position = eng.max_positions - 1 if eng.max_positions else 0   # checked on the host each step
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side), torch.no_grad():
+                for _ in range(2):                   # a decode step writes the same values again: repeatable
+                    self._forward(ctx)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.no_grad(), torch.cuda.graph(self.graph):
+                self.logits = self._forward(ctx)
+        self.graph.replay()
+        out = self.out_tokens[:B].cpu().tolist()      # waits for the step
+        for s in slots:
+            eng.cache.commit(s, 1)
+        return out, self.logits[:B]

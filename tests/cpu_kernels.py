@@ -164,6 +164,10 @@ def install(monkeypatch):
 class CpuEngine(Engine):
     """The engine with the two places that need a GPU (the device check, the pinned upload) replaced."""
 
+    def __init__(self, *args, **kw):
+        super().__init__(*args, **kw)
+        self.graph_ok = False            # graphs are a GPU matter
+
     def _require_gpu(self):
         pass
 

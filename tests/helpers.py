@@ -83,11 +83,19 @@ def random_tokens(vocab: int, n: int, seed: int) -> list:
     return torch.randint(0, vocab, (n,), generator=g).tolist()
 
 
-def assert_logits_close(got, want, dtype: str, what: str = "") -> None:
-    """float32: only the order of sums differs from the plain implementation.
-    bfloat16: weights are the same numbers; activations are rounded to 8 bits of mantissa at
-    every product's input, a few times a layer: the error is a fraction of a percent of the
-    logits' scale.  The bounds leave a factor of about five over what was measured."""
+def assert_logits_close(got, want, dtype: str, what: str = "", sharp: bool = False) -> None:
+    """float32: only the order of sums differs from the plain implementation: 2e-4 of the scale.
+
+    bfloat16: the weights are the same numbers; activations are rounded to 8 bits of mantissa at the
+    input of every product, a few times a layer.  What that rounding alone does was measured with
+    float32-accumulating torch operations that round at the same places (tests/cpu_kernels.py under
+    the engine): for the tiny configurations the error's RMS is 0.3 .. 0.55 % of the logits' RMS and
+    its maximum 0.2 .. 0.7 % of the largest logit.  The bounds are 2.5 % for both, a factor of four
+    to five.  With `sharp` weights (q/k gains x 3, scores of standard deviation ~9) the same
+    measurement gives 2.3 .. 6.9 % RMS and up to 15 % maximum, since a rounding of q or k moves
+    whole softmax weights; there the bounds are 20 % and 45 %, which still separates rounding from
+    a lost or wrong key (an error of the order of the logits themselves); the exact check of that
+    case is the float32 one."""
     got = torch.as_tensor(np.asarray(got), dtype=torch.float32) if not isinstance(got, torch.Tensor) else got.float().cpu()
     want = want.float()
     assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(want.shape)}"
@@ -97,9 +105,10 @@ def assert_logits_close(got, want, dtype: str, what: str = "") -> None:
     if dtype == "float32":
         assert float(err.max()) <= 2e-4 * scale, f"{what}: max err {float(err.max()):.3e} at scale {scale:.2f}"
     else:
-        rms = float(want.pow(2).mean().sqrt())
-        assert float(err.max()) <= 2.5e-2 * scale, f"{what}: max err {float(err.max()):.3e} at scale {scale:.2f}"
-        assert float(err.pow(2).mean().sqrt()) <= 8e-3 * max(rms, 0.1), \
+        rms = max(float(want.pow(2).mean().sqrt()), 0.05)
+        b_max, b_rms = (0.45, 0.20) if sharp else (2.5e-2, 2.5e-2)
+        assert float(err.max()) <= b_max * scale, f"{what}: max err {float(err.max()):.3e} at scale {scale:.2f}"
+        assert float(err.pow(2).mean().sqrt()) <= b_rms * rms, \
             f"{what}: rms err {float(err.pow(2).mean().sqrt()):.3e} vs rms {rms:.3f}"
 
 

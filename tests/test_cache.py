@@ -33,8 +33,8 @@ def test_page_pool():
 def test_groups_and_storage():
     c = make(needs=[KvNeed(2, 16), KvNeed(1, 32), KvNeed(2, 16), StateNeed((3, 5)), None, KvNeed(2, 16, window=100)])
     assert [g.layers for g in c.groups] == [[0, 2], [1], [5]]
-    assert c.groups[0].k.shape == (2, 10, 2, 64, 16) and c.groups[0].v.shape == (2, 10, 2, 16, 64)
-    assert c.groups[1].k.shape == (1, 10, 1, 64, 32)
+    assert c.groups[0].k.shape == (2, 11, 2, 64, 16) and c.groups[0].v.shape == (2, 11, 2, 16, 64)   # + a spare page
+    assert c.groups[1].k.shape == (1, 11, 1, 64, 32) and c.groups[1].spare_page == 10
     v0, v2, v3 = c.layer_view(0), c.layer_view(2), c.layer_view(3)
     assert v0.group == v2.group == 0 and v0.k_pages.data_ptr() != v2.k_pages.data_ptr()
     assert v3.state.shape == (10, 3, 5) and c.layer_view(4) is None

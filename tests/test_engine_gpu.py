@@ -140,3 +140,53 @@ def test_trace_run_steps_without_wants_write_no_file(tmp_path):
     assert sorted(out) == [1]
     assert_logits_close(out[1], plain_logits("A", [1, 2, 3, 4])[3:], "float32", "after a silent step")
     assert not os.path.exists(tmp_path / "o" / "0.f32")
+
+
+# ----------------------------------------------------------------------------- captured decode steps
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_graph_replays_equal_eager_steps(dtype):
+    """Every replay of the captured decode step is checked against the eager step, with eager work
+    and synchronisations of the program's own between the replays; rows of padding change nothing."""
+    name = "B"
+    V = CONFIGS[name]["vocab_size"]
+    prompts = [random_tokens(V, n, 500 + n) for n in (20, 70, 3)]
+    eager, graph = make_engine(name, dtype, 2048), make_engine(name, dtype, 2048)
+    es = [eager.acquire() for _ in prompts]
+    gs = [graph.acquire() for _ in prompts]
+    tok = eager.sample(eager.step(list(zip(es, prompts)), want="last")).cpu().tolist()
+    tok_g = graph.sample(graph.step(list(zip(gs, prompts)), want="last")).cpu().tolist()
+    assert tok == tok_g
+    runner = graph.decode_runner(3, 200)            # 4 rows: one of padding
+    assert runner.rows == 4
+    for step in range(70):                          # crosses a page edge for two of the sequences
+        want = eager.step([(s, [t]) for s, t in zip(es, tok)], want="last")
+        got_tokens, got = runner.step(gs, tok)
+        torch.cuda.synchronize()
+        assert float((got - want).abs().max()) <= (1e-5 if dtype == "float32" else 2e-2), f"replay {step}"
+        tok = eager.sample(want).cpu().tolist()
+        if dtype == "float32":
+            assert got_tokens == tok, f"replay {step}"
+        if step % 7 == 0:                           # eager work of another engine between replays
+            other = eager.acquire()
+            eager.step([(other, prompts[1])], want="last")
+            eager.release(other)
+    # a smaller live set in the same graph: the finished sequence's row becomes padding
+    want = eager.step([(es[0], [tok[0]]), (es[2], [tok[2]])], want="last")
+    _, got = runner.step([gs[0], gs[2]], [tok[0], tok[2]])
+    assert float((got - want).abs().max()) <= (1e-5 if dtype == "float32" else 2e-2)
+    for e in (eager, graph):
+        e.cache.check()
+
+
+def test_generation_with_and_without_graph_agree():
+    from synaptix_amd.engine.generate import generate, GenerationConfig
+    V = CONFIGS["A"]["vocab_size"]
+    prompts = [random_tokens(V, n, 600 + n) for n in (5, 40, 64, 9, 2)]
+    eng = make_engine("A", "float32", 4096)
+    cfgs = [GenerationConfig(max_new_tokens=n, temperature=t, seed=i) for i, (n, t) in
+            enumerate([(30, 0.0), (12, 0.8), (70, 0.0), (3, 1.0), (25, 0.0)])]
+    a, sa = generate(eng, prompts, cfgs, use_graph=True)
+    b, sb = generate(eng, prompts, cfgs, use_graph=False)
+    assert [o.tokens for o in a] == [o.tokens for o in b]
+    assert [len(o.tokens) for o in a] == [30, 12, 70, 3, 25]
+    eng.cache.check()

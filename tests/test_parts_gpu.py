@@ -64,7 +64,11 @@ def test_rotary_part_tables():
     cos, sin = r.tables(DEV)
     c, s = P.rope_tables(32, 300, 1e6)
     assert cos.shape == (300, 16)
-    assert torch.allclose(cos.cpu(), c, atol=1e-6) and torch.allclose(sin.cpu(), s, atol=1e-6)
+    # two float32 power routines may differ by one ulp in a frequency; times a position of up to
+    # 300 that is an angle error of 300 * 2^-23 ~ 4e-5
+    assert torch.allclose(cos.cpu(), c, atol=1e-4) and torch.allclose(sin.cpu(), s, atol=1e-4)
+    assert torch.equal(cos[0].cpu(), torch.ones(16)) and torch.equal(sin[0].cpu(), torch.zeros(16))
+    assert torch.allclose(cos[:4].cpu(), c[:4], atol=1e-6)
     with pytest.raises(ValueError):
         RotaryHalfSplit(1e4, 15, 10)
 
@@ -122,7 +126,8 @@ def test_gated_mlp_part_alone(dtype):
     got = ff.forward(x.to(DEV), None).cpu()
     want = P.swiglu_mlp(x.float(), w["m.gate_proj.weight"].float(), w["m.up_proj.weight"].float(),
                         w["m.down_proj.weight"].float())
-    assert (got - want).abs().max() <= (1e-4 if dtype == F32 else 3e-2)
+    # bf16: the activations silu(g) * u are rounded once (2^-9 relative) before the last product
+    assert (got - want).abs().max() <= (2e-5 if dtype == F32 else 2e-2) * float(want.abs().max())
     with pytest.raises(ValueError, match="gelu"):
         GatedMlp("m.", 8, 8, "gelu")
 
