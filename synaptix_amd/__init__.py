@@ -4,7 +4,11 @@ from .weights import WeightError, write_random_model
 from .cache import CacheFull, CacheError
 from . import models as _models  # registers the architectures
 from .engine import Engine, StepError
+from .engine.generate import generate, GenerationOutput, GenerationStats
+from .sampling import GenerationConfig
+from .pipeline import Pipeline, load
 
 __all__ = ["ConfigError", "Qwen3Config", "load_config", "register_architecture", "known_architectures",
-           "WeightError", "write_random_model", "CacheFull", "CacheError", "Engine", "StepError"]
+           "WeightError", "write_random_model", "CacheFull", "CacheError", "Engine", "StepError", "generate",
+           "GenerationOutput", "GenerationStats", "GenerationConfig", "Pipeline", "load"]
 __version__ = "0.1.0"

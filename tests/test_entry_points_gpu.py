@@ -1,0 +1,74 @@
+"""Greedy generation through the entry points a user has: the Python pipeline and the command line."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_qwen3 as P
+from helpers import ROOT, model_folder, plain_model, random_tokens, CONFIGS
+from scenarios import check_greedy_path
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def need_gpu():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_pipeline_generate(dtype):
+    import synaptix_amd
+    from synaptix_amd import GenerationConfig
+    name = "B"
+    plain = plain_model(name)
+    prompt = random_tokens(CONFIGS[name]["vocab_size"], 21, 9)
+    want = P.generate(plain, prompt, 10)
+    pipe = synaptix_amd.load(model_folder(name), device="cuda", dtype=dtype, max_seq=256)
+    ids, stats = pipe.generate(prompt, GenerationConfig(max_new_tokens=10))
+    assert stats.prompt_tokens == 21 and stats.new_tokens == 10
+    if dtype == "f32":
+        assert ids == want
+    else:
+        check_greedy_path(plain, prompt, ids, want)
+    # the stop token: make the third token of the plain path the stop token
+    ids, _ = pipe.generate(prompt, GenerationConfig(max_new_tokens=10, eos_token_id=want[2]))
+    if dtype == "f32":
+        assert ids == want[:3]
+    seen = []
+    pipe.generate_streaming(prompt, GenerationConfig(max_new_tokens=4), lambda t: seen.append(t) or True)
+    assert len(seen) == 4
+    outs, st = pipe.generate_batch([prompt, prompt[:5]], GenerationConfig(max_new_tokens=6))
+    assert [len(o.tokens) for o in outs] == [6, 6] and st.batches == 1
+    with pytest.raises(FileNotFoundError, match="tokenizer"):
+        pipe.encode("text")
+
+
+def test_command_line_run_and_bench():
+    name = "A"
+    folder = model_folder(name)
+    plain = plain_model(name)
+    prompt = random_tokens(CONFIGS[name]["vocab_size"], 12, 10)
+    want = P.generate(plain, prompt, 7)
+    cmd = [sys.executable, "-m", "synaptix_amd", "run", folder, "--prompt-ids", ",".join(map(str, prompt)),
+           "--max-tokens", "7", "--temperature", "0", "--compute-dtype", "f32", "--warmup"]
+    proc = subprocess.run(cmd, capture_output=True, text=True, cwd=ROOT, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [int(t) for t in proc.stdout.split()] == want
+    assert "12 prompt + 7 new tokens" in proc.stderr and "tok/s" in proc.stderr
+    cmd = [sys.executable, "-m", "synaptix_amd", "bench", folder, "--n-tokens", "16", "--prompt-tokens", "9",
+           "--batch-size", "3", "--warmup", "1"]
+    proc = subprocess.run(cmd, capture_output=True, text=True, cwd=ROOT, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    line = json.loads(proc.stdout.strip().splitlines()[-1])
+    assert line["new_tokens"] == 48 and line["prompt_tokens"] == 27 and line["decode_tok_s"] > 0
+
+
+def test_smoke_entry():
+    sys.path.insert(0, ROOT)
+    import __graft_entry__
+    __graft_entry__.smoke()
