@@ -14,8 +14,9 @@
 // is rounded once.
 //
 //   prefill: a workgroup of 4 waves takes 128 query rows of one (sequence, head); a wave 32 of them.
-//   decode : a wave takes (sequence, kv head, up to 16 heads of its group, one split of the keys);
-//            the heads of a group share every K/V load.  A second kernel merges the splits.
+//   decode : a workgroup takes (sequence, kv head, up to 16 heads of its group, one split of the keys);
+//            the heads of a group share every K/V load and the waves share the split's blocks.
+//            A second kernel merges the splits when there is more than one.
 // Reference counterparts: flash_splitq.cu (prefill), flash_decode.cu:92-205,340-387 (split + merge,
 // one block a q-head there, scalar dot products).
 #include "common.h"
@@ -27,15 +28,20 @@ SYN_DEFINE_ERROR_CHANNEL
 
 constexpr int HD = SYN_HD;
 static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head sizes in steps of 16 up to 256");
-constexpr int KS32 = HD / 32;
 constexpr bool TAIL16 = (HD % 32) != 0;
 constexpr int DT = HD / 16;
 
 SYN_EXPORT int syn_attention_head_dim() { return HD; }
 
+// Fragments of Q (or of a K row block) along the head dimension.  Head sizes that are a multiple of
+// 32 take k-steps of 32 (16x16x32); the others take k-steps of 16 throughout (16x16x16): one
+// accumulation chain never mixes the two shapes.
+constexpr int KSTEPS = TAIL16 ? HD / 16 : HD / 32;
+constexpr int KW = TAIL16 ? 4 : 8;  // elements a lane holds for one k-step
+typedef __attribute__((ext_vector_type(KW))) __bf16 kfrag_t;
+
 struct QFrag {
-  bf16x8 k32[KS32 > 0 ? KS32 : 1];
-  bf16x4 k16;
+  kfrag_t k[KSTEPS];
 };
 
 __device__ __forceinline__ f32x4 mfma16(bf16x4 a, bf16x4 b, f32x4 c) {
@@ -43,12 +49,26 @@ __device__ __forceinline__ f32x4 mfma16(bf16x4 a, bf16x4 b, f32x4 c) {
                                                    0, 0, 0);
 }
 
-__device__ __forceinline__ void load_q(QFrag& f, const bf16* qptr, int lane) {
-  const bf16x8 z8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  const bf16x4 z4 = {0, 0, 0, 0};
+__device__ __forceinline__ f32x4 mfma_qk(bf16x4 a, bf16x4 b, f32x4 c) { return mfma16(a, b, c); }
+__device__ __forceinline__ f32x4 mfma_qk(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// the fragments of one row of HD elements: in k-step ks, lane group g = lane / 16 holds elements ks*4*KW + KW*g .. + KW
+__device__ __forceinline__ void load_row(kfrag_t (&f)[KSTEPS], const bf16* row, int lane) {
 #pragma unroll
-  for (int ks = 0; ks < KS32; ++ks) f.k32[ks] = qptr ? *(const bf16x8*)(qptr + ks * 32 + 8 * (lane / 16)) : z8;
-  if (TAIL16) f.k16 = qptr ? *(const bf16x4*)(qptr + KS32 * 32 + 4 * (lane / 16)) : z4;
+  for (int ks = 0; ks < KSTEPS; ++ks) f[ks] = *(const kfrag_t*)(row + ks * (4 * KW) + KW * (lane / 16));
+}
+
+__device__ __forceinline__ void load_q(QFrag& f, const bf16* qptr, int lane) {
+  if (qptr) {
+    load_row(f.k, qptr, lane);
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+      for (int e = 0; e < KW; ++e) f.k[ks][e] = (bf16)0.f;
+  }
 }
 
 template <int QB>
@@ -82,18 +102,12 @@ __device__ __forceinline__ void attn_block(AttnState<QB>& st, const QFrag (&qf)[
   for (int t = 0; t < 4; ++t) {
 #pragma unroll
     for (int c = 0; c < QB; ++c) s[t][c] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    const bf16* krow = kpage + (size_t)(t * 16 + r16) * HD;
+    kfrag_t ka[KSTEPS];
+    load_row(ka, kpage + (size_t)(t * 16 + r16) * HD, lane);
 #pragma unroll
-    for (int ks = 0; ks < KS32; ++ks) {
-      const bf16x8 a = *(const bf16x8*)(krow + ks * 32 + 8 * g4);
+    for (int ks = 0; ks < KSTEPS; ++ks)
 #pragma unroll
-      for (int c = 0; c < QB; ++c) s[t][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[c].k32[ks], s[t][c], 0, 0, 0);
-    }
-    if (TAIL16) {
-      const bf16x4 a = *(const bf16x4*)(krow + KS32 * 32 + 4 * g4);
-#pragma unroll
-      for (int c = 0; c < QB; ++c) s[t][c] = mfma16(a, qf[c].k16, s[t][c]);
-    }
+      for (int c = 0; c < QB; ++c) s[t][c] = mfma_qk(ka[ks], qf[c].k[ks], s[t][c]);
   }
 #pragma unroll
   for (int c = 0; c < QB; ++c) {
@@ -231,79 +245,193 @@ SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, co
 }
 
 // ------------------------------------------------------------------ decode: split over keys, then merge
-// partial[(seq * nh + head) * n_splits + split] = { m, l, o[HD] } in float.
+// A workgroup of DEC_WAVES waves takes (sequence, kv head, up to 16 heads of its group, one split of
+// the key blocks); its waves take the split's blocks in turn and their states are combined in LDS.
+// With one split the workgroup writes the output itself; else it writes a partial
+//   partial[(seq * nh + head) * n_splits + split] = { m, l, o[HD] }   (float)
+// and a second kernel merges the splits.
 constexpr int PART = HD + 2;
+constexpr int DEC_WAVES = HD > 128 ? 2 : 4;
 
-__global__ void __launch_bounds__(SYN_WAVE)
+// Like attn_block for one column block, but every K and V fragment of the block is requested before
+// the first product needs one: a block costs one trip to memory instead of two.
+__device__ __forceinline__ void attn_block_decode(AttnState<1>& st, const QFrag& qf, const bf16* __restrict__ kpage,
+                                                  const bf16* __restrict__ vpage, int key0, int qpos, int lo,
+                                                  int kv_len, float scale, int lane) {
+  const int r16 = lane % 16, g4 = lane / 16;
+  kfrag_t ka[4][KSTEPS];
+  bf16x4 va[4][DT];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) load_row(ka[t], kpage + (size_t)(t * 16 + r16) * HD, lane);
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) va[t][dt] = *(const bf16x4*)(vpage + (size_t)(dt * 16 + r16) * SYN_PAGE + t * 16 + 4 * g4);
+
+  f32x4 s[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    s[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) s[t] = mfma_qk(ka[t][ks], qf.k[ks], s[t]);
+  }
+  float mloc = -INFINITY;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int key = key0 + t * 16 + 4 * g4 + e;
+      float v = s[t][e] * scale;
+      if (key > qpos || key < lo) v = -INFINITY;
+      s[t][e] = v;
+      mloc = fmaxf(mloc, v);
+    }
+  mloc = fmaxf(mloc, __shfl_xor(mloc, 16, SYN_WAVE));
+  mloc = fmaxf(mloc, __shfl_xor(mloc, 32, SYN_WAVE));
+  const float m_new = fmaxf(st.m[0], mloc);
+  const float m_use = m_new == -INFINITY ? 0.f : m_new;
+  const float alpha = __expf(st.m[0] - m_use);
+  st.m[0] = m_new;
+  float lsum = 0.f;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float p = __expf(s[t][e] - m_use);
+      s[t][e] = p;
+      lsum += p;
+    }
+  st.l[0] = st.l[0] * alpha + lsum;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) st.o[dt][0] *= alpha;
+  const bool ragged = key0 + SYN_PAGE > kv_len;
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    bf16x4 pb;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) pb[e] = (bf16)s[t][e];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      bf16x4 av = va[t][dt];
+      if (ragged) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (key0 + t * 16 + 4 * g4 + e >= kv_len) av[e] = (bf16)0.f;
+      }
+      st.o[dt][0] = mfma16(av, pb, st.o[dt][0]);
+    }
+  }
+}
+
+__global__ void __launch_bounds__(DEC_WAVES * SYN_WAVE)
 attn_decode_split_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages,
                          const bf16* __restrict__ v_pages, const int* __restrict__ page_table, int table_stride,
-                         const int* __restrict__ seq_len, float* __restrict__ partial, float scale, int window, int nh,
-                         int nkv, int n_splits) {
-  const int lane = threadIdx.x;
+                         const int* __restrict__ seq_len, float* __restrict__ partial, bf16* __restrict__ out,
+                         float scale, int window, int nh, int nkv, int n_splits) {
+  __shared__ float sm[DEC_WAVES][16];            // running maximum of each column
+  __shared__ float sl[DEC_WAVES][16];            // sum of each column
+  __shared__ float so[DEC_WAVES][16][HD + 4];    // unnormalised output of each column
+  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
   const int seq = blockIdx.x, split = blockIdx.z;
   const int g = nh / nkv, chunks = (g + 15) / 16;
   const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
   const int kv_len = seq_len[seq], pos = kv_len - 1;
-  const int hg = chunk * 16 + lane % 16;  // head inside the group
+  const int col = lane % 16;
+  const int hg = chunk * 16 + col;  // head inside the group
   const bool valid = hg < g;
-  const int head = kvh * g + hg;
+  const int n_cols = min(16, g - chunk * 16);
 
-  QFrag qf[1];
-  int qpos[1], lo[1];
-  qpos[0] = valid ? pos : -1;
-  lo[0] = window > 0 ? max(0, pos - window + 1) : 0;
-  load_q(qf[0], valid ? q + ((size_t)seq * nh + head) * HD : nullptr, lane);
+  QFrag qf;
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  load_q(qf, valid ? q + ((size_t)seq * nh + kvh * g + hg) * HD : nullptr, lane);
   AttnState<1> st;
   attn_init(st);
-  const int b_lo = lo[0] / SYN_PAGE, b_hi = pos / SYN_PAGE;
+  const int b_lo = lo / SYN_PAGE, b_hi = pos / SYN_PAGE;
   const int per = (b_hi - b_lo + n_splits) / n_splits;  // ceil((b_hi - b_lo + 1) / n_splits)
   const int b0 = b_lo + split * per, b1 = min(b_hi + 1, b0 + per);
-  for (int kb = b0; kb < b1; ++kb) {
+  for (int kb = b0 + wave; kb < b1; kb += DEC_WAVES) {
     const size_t base = ((size_t)page_table[(size_t)seq * table_stride + kb] * nkv + kvh) * SYN_PAGE * HD;
-    attn_block<1>(st, qf, k_pages + base, v_pages + base, kb * SYN_PAGE, qpos, lo, kv_len, scale, lane);
+    attn_block_decode(st, qf, k_pages + base, v_pages + base, kb * SYN_PAGE, valid ? pos : -1, lo, kv_len, scale, lane);
   }
   float l = st.l[0];
   l += __shfl_xor(l, 16, SYN_WAVE);
   l += __shfl_xor(l, 32, SYN_WAVE);
-  if (!valid) return;
-  float* p = partial + ((size_t)(seq * nh + head) * n_splits + split) * PART;
-  if (lane / 16 == 0) {
-    p[0] = st.m[0];
-    p[1] = l;
+  if (lane < 16) {
+    sm[wave][lane] = st.m[0];
+    sl[wave][lane] = l;
   }
+  if (valid) {
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) p[2 + dt * 16 + 4 * (lane / 16) + e] = st.o[dt][0][e];
+      for (int e = 0; e < 4; ++e) so[wave][col][dt * 16 + 4 * (lane / 16) + e] = st.o[dt][0][e];
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < n_cols * HD; idx += DEC_WAVES * SYN_WAVE) {
+    const int c = idx / HD, d = idx % HD;
+    float m = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) m = fmaxf(m, sm[w][c]);
+    float acc = 0.f, lsum = 0.f;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) {
+      if (sm[w][c] == -INFINITY) continue;  // a wave that had no block
+      const float f = __expf(sm[w][c] - m);
+      acc += f * so[w][c][d];
+      lsum += f * sl[w][c];
+    }
+    const int head = kvh * g + chunk * 16 + c;
+    if (n_splits == 1) {
+      out[((size_t)seq * nh + head) * HD + d] = (bf16)(acc / lsum);
+    } else {
+      float* p = partial + ((size_t)(seq * nh + head) * n_splits + split) * PART;
+      p[2 + d] = acc;
+      if (d == 0) {
+        p[0] = m;
+        p[1] = lsum;
+      }
+    }
+  }
 }
 
+// one wave a (sequence, head): lanes first share the splits' maxima and sums, then each takes output dims
 __global__ void __launch_bounds__(SYN_WAVE)
 attn_decode_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out, int n_splits) {
   const int row = blockIdx.x, lane = threadIdx.x;  // row = seq * nh + head
   const float* p = partial + (size_t)row * n_splits * PART;
-  float m = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) m = fmaxf(m, p[(size_t)s * PART]);
+  float wsum[(HD + SYN_WAVE - 1) / SYN_WAVE] = {};
   float l = 0.f;
-  float o[(HD + SYN_WAVE - 1) / SYN_WAVE] = {};
-  for (int s = 0; s < n_splits; ++s) {
-    const float ms = p[(size_t)s * PART];
-    if (ms == -INFINITY) continue;  // a split that had no keys
-    const float w = __expf(ms - m);
-    l += w * p[(size_t)s * PART + 1];
+  float m = -INFINITY;
+  for (int s0 = 0; s0 < n_splits; s0 += SYN_WAVE) {  // maximum over all splits
+    const int s = s0 + lane;
+    m = fmaxf(m, s < n_splits ? p[(size_t)s * PART] : -INFINITY);
+  }
+  m = wave_max(m);
+  for (int s0 = 0; s0 < n_splits; s0 += SYN_WAVE) {
+    const int s = s0 + lane;
+    const float ms = s < n_splits ? p[(size_t)s * PART] : -INFINITY;
+    const float w = ms == -INFINITY ? 0.f : __expf(ms - m);  // a split that had no keys weighs nothing
+    l += s < n_splits ? w * p[(size_t)s * PART + 1] : 0.f;
+    const int cnt = min(SYN_WAVE, n_splits - s0);
+    for (int j = 0; j < cnt; ++j) {
+      const float wj = __shfl(w, j, SYN_WAVE);
+      if (wj == 0.f) continue;
 #pragma unroll
-    for (int i = 0; i < (HD + SYN_WAVE - 1) / SYN_WAVE; ++i) {
-      const int d = lane + i * SYN_WAVE;
-      if (d < HD) o[i] += w * p[(size_t)s * PART + 2 + d];
+      for (int i = 0; i < (HD + SYN_WAVE - 1) / SYN_WAVE; ++i) {
+        const int d = lane + i * SYN_WAVE;
+        if (d < HD) wsum[i] += wj * p[(size_t)(s0 + j) * PART + 2 + d];
+      }
     }
   }
+  l = wave_sum(l);
 #pragma unroll
   for (int i = 0; i < (HD + SYN_WAVE - 1) / SYN_WAVE; ++i) {
     const int d = lane + i * SYN_WAVE;
-    if (d < HD) out[(size_t)row * HD + d] = (bf16)(o[i] / l);
+    if (d < HD) out[(size_t)row * HD + d] = (bf16)(wsum[i] / l);
   }
 }
 
-// workspace: n_seqs * nh * n_splits * (HD + 2) floats
+// workspace: n_seqs * nh * n_splits * (HD + 2) floats (unused with one split)
 SYN_EXPORT int syn_attention_decode_bf16(const void* q, const void* k_pages, const void* v_pages,
                                          const int* page_table, int table_stride, const int* seq_len, int n_seqs,
                                          void* out, float* workspace, int n_splits, float scale, int window, int nh,
@@ -313,11 +441,13 @@ SYN_EXPORT int syn_attention_decode_bf16(const void* q, const void* k_pages, con
   SYN_CHECK(nh % nkv == 0, "attention_decode: %d heads do not divide into %d kv heads", nh, nkv);
   const int chunks = (nh / nkv + 15) / 16;
   SYN_CHECK(nkv * chunks <= 65535 && n_splits <= 65535, "attention_decode: grid too large");
-  attn_decode_split_kernel<<<dim3(n_seqs, nkv * chunks, n_splits), SYN_WAVE, 0, stream>>>(
-      (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, page_table, table_stride, seq_len, workspace, scale,
-      window, nh, nkv, n_splits);
+  attn_decode_split_kernel<<<dim3(n_seqs, nkv * chunks, n_splits), DEC_WAVES * SYN_WAVE, 0, stream>>>(
+      (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, page_table, table_stride, seq_len, workspace,
+      (bf16*)out, scale, window, nh, nkv, n_splits);
   SYN_LAUNCH_CHECK("attention_decode_split");
-  attn_decode_merge_kernel<<<n_seqs * nh, SYN_WAVE, 0, stream>>>(workspace, (bf16*)out, n_splits);
-  SYN_LAUNCH_CHECK("attention_decode_merge");
+  if (n_splits > 1) {
+    attn_decode_merge_kernel<<<n_seqs * nh, SYN_WAVE, 0, stream>>>(workspace, (bf16*)out, n_splits);
+    SYN_LAUNCH_CHECK("attention_decode_merge");
+  }
   return 0;
 }

@@ -11,6 +11,7 @@
 // mma.sync m16n8k16), best_cu/gemv/mma_gemv.cu:19-133 (M == 1), best_cu/gemm/gemm_f32.cu (SIMT).
 // The tilings here are made for 64-lane waves and MFMA operand layouts, not translated.
 #include "common.h"
+#include <stdlib.h>
 
 // ------------------------------------------------------------------ SIMT, any type
 #define SIMT_BM 64
@@ -63,7 +64,7 @@ gemm_simt_kernel(const TIn* __restrict__ x, const TIn* __restrict__ w, TOut* __r
 // Both operands: lane holds row lane%16, k = 8*(lane/16) .. +8, one 16-byte load.
 // A workgroup owns RT*16 rows of W; its WAVES waves take k-chunks of 32 round-robin, so that at
 // any moment the workgroup reads WAVES*64 contiguous bytes of each row.
-template <int MB, int RT, int WAVES>
+template <int MB, int RT, int WAVES, int U>
 __global__ void __launch_bounds__(WAVES * SYN_WAVE)
 gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
                    int M, int N, int K) {
@@ -75,13 +76,13 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
 
   const bf16* wrow[RT];
 #pragma unroll
-  for (int r = 0; r < RT; ++r) wrow[r] = w + (size_t)min(n0 + r * 16 + r16, N - 1) * K;
+  for (int r = 0; r < RT; ++r) wrow[r] = w + (size_t)min(n0 + r * 16 + r16, N - 1) * K + kq;
   const bf16* xrow[MB];
   bool xok[MB];
 #pragma unroll
   for (int b = 0; b < MB; ++b) {
     xok[b] = b * 16 + r16 < M;
-    xrow[b] = x + (size_t)min(b * 16 + r16, M - 1) * K;
+    xrow[b] = x + (size_t)min(b * 16 + r16, M - 1) * K + kq;
   }
   f32x4 acc[MB][RT];
 #pragma unroll
@@ -89,18 +90,26 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
 #pragma unroll
     for (int r = 0; r < RT; ++r) acc[b][r] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  for (int k0 = wave * 32; k0 < K; k0 += WAVES * 32) {
-    const int k = k0 + kq;
-    const bool kin = k < K;  // K is a multiple of 8: a chunk of 8 lies inside or outside as a whole
-    bf16x8 bw[RT], ax[MB];
+  // U chunks of 32 at a time: all loads of a group are issued before the first product needs them,
+  // so that a wave keeps U * RT KiB of the weight stream in flight
+  for (int k0 = wave * (32 * U); k0 < K; k0 += WAVES * 32 * U) {
+    bf16x8 bw[U][RT], ax[U][MB];
 #pragma unroll
-    for (int r = 0; r < RT; ++r) bw[r] = kin ? *(const bf16x8*)(wrow[r] + k) : zero;
+    for (int u = 0; u < U; ++u) {
+      const int k = k0 + u * 32;
+      const bool kin = k + kq < K;  // K is a multiple of 8: a chunk of 8 lies inside or outside as a whole
 #pragma unroll
-    for (int b = 0; b < MB; ++b) ax[b] = (kin && xok[b]) ? *(const bf16x8*)(xrow[b] + k) : zero;
+      for (int r = 0; r < RT; ++r) bw[u][r] = kin ? __builtin_nontemporal_load((const bf16x8*)(wrow[r] + k)) : zero;
 #pragma unroll
-    for (int b = 0; b < MB; ++b)
+      for (int b = 0; b < MB; ++b) ax[u][b] = (kin && xok[b]) ? *(const bf16x8*)(xrow[b] + k) : zero;
+    }
 #pragma unroll
-      for (int r = 0; r < RT; ++r) acc[b][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[b], bw[r], acc[b][r], 0, 0, 0);
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int b = 0; b < MB; ++b)
+#pragma unroll
+        for (int r = 0; r < RT; ++r)
+          acc[b][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[u][b], bw[u][r], acc[b][r], 0, 0, 0);
   }
 
   // sum the waves' partial tiles in a fixed order
@@ -128,12 +137,18 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
   }
 }
 
-template <int MB, int RT, int WAVES>
+template <int MB, int RT, int WAVES, int U>
 static void launch_skinny(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
                           hipStream_t stream) {
   const int grid = (N + RT * 16 - 1) / (RT * 16);
   const size_t lds = (size_t)WAVES * MB * RT * 4 * 64 * sizeof(float);
-  gemm_skinny_kernel<MB, RT, WAVES><<<grid, WAVES * SYN_WAVE, lds, stream>>>(x, w, out, out_is_f32, M, N, K);
+  static bool raised = false;
+  if (lds > 65536 && !raised) {
+    hipFuncSetAttribute((const void*)gemm_skinny_kernel<MB, RT, WAVES, U>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                        (int)lds);
+    raised = true;
+  }
+  gemm_skinny_kernel<MB, RT, WAVES, U><<<grid, WAVES * SYN_WAVE, lds, stream>>>(x, w, out, out_is_f32, M, N, K);
 }
 
 // ------------------------------------------------------------------ tiled, bf16, large M
@@ -251,14 +266,32 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   }
   const bf16* xb = (const bf16*)x;
   const bf16* wb = (const bf16*)w;
+  // rows of W a workgroup owns: more rows amortise the loads of x, fewer rows give more workgroups
+  const int variant = getenv("SYN_SKINNY") ? atoi(getenv("SYN_SKINNY")) : -1;
   if (M <= 16) {
-    launch_skinny<1, 1, 8>(xb, wb, out, out_is_f32, M, N, K, stream);
+    const int v = variant >= 0 ? variant : (N <= 8192 ? 0 : (N <= 32768 ? 2 : 3));
+    if (v == 0) launch_skinny<1, 1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 1) launch_skinny<1, 1, 8, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 2) launch_skinny<1, 2, 8, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 3) launch_skinny<1, 4, 8, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 4) launch_skinny<1, 2, 16, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else launch_skinny<1, 4, 8, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
   } else if (M <= 32) {
-    launch_skinny<2, 2, 8>(xb, wb, out, out_is_f32, M, N, K, stream);
+    const int v = variant >= 0 ? variant : (N <= 8192 ? 0 : 2);
+    if (v == 0) launch_skinny<2, 1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 1) launch_skinny<2, 2, 8, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 2) launch_skinny<2, 4, 8, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 3) launch_skinny<2, 2, 16, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else launch_skinny<2, 4, 4, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
   } else if (M <= 48) {
-    launch_skinny<3, 2, 8>(xb, wb, out, out_is_f32, M, N, K, stream);
+    launch_skinny<3, 2, 8, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
   } else if (M <= 64) {
-    launch_skinny<4, 2, 8>(xb, wb, out, out_is_f32, M, N, K, stream);
+    const int v = variant >= 0 ? variant : (N <= 8192 ? 0 : 2);
+    if (v == 0) launch_skinny<4, 1, 16, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 1) launch_skinny<4, 2, 8, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 2) launch_skinny<4, 4, 8, 1>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 3) launch_skinny<4, 2, 16, 1>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else launch_skinny<4, 4, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
   } else {
     const dim3 grid((N + TG_BN - 1) / TG_BN, (M + TG_BM - 1) / TG_BM);
     gemm_tiled_kernel<<<grid, 256, 0, stream>>>(xb, wb, out, out_is_f32, M, N, K);

@@ -208,9 +208,10 @@ def attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, seq_past,
 
 
 def decode_splits(n_seqs, n_kv_heads, max_pages):
-    """How many ways the keys of a sequence are split in decode: enough waves to fill the chip."""
-    want = max(1, 2048 // max(1, n_seqs * n_kv_heads))
-    return int(max(1, min(want, max_pages, 64)))
+    """How many ways the key blocks of a sequence are split in decode: enough workgroups (of four
+    waves, a block a wave at a time) to fill the chip at small batches, one split at large ones."""
+    want = -(-512 // max(1, n_seqs * n_kv_heads))
+    return int(max(1, min(want, -(-max_pages // 4), 64)))
 
 
 def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,

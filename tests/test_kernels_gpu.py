@@ -283,6 +283,11 @@ def test_attention_prefill(ops, dtype, nh, nkv, hd, past, new, window):
     (8, 1, 16, [1000, 77], 0, 16),
     (4, 2, 96, [500, 30], 100, 5),
     (32, 8, 128, [2100] * 3, 0, 11),
+    (6, 2, 48, [35], 0, 1),                     # head sizes that are no multiple of 32, three heads a group
+    (6, 2, 48, [200, 35, 64], 0, 3),
+    (5, 1, 80, [100, 300], 0, 2),
+    (4, 4, 112, [70], 0, 1),
+    (8, 2, 256, [130, 700], 0, 4),
 ])
 def test_attention_decode_bf16(ops, nh, nkv, hd, lens, window, splits):
     B = len(lens)
