@@ -164,52 +164,199 @@ __device__ __forceinline__ void attn_block(AttnState<QB>& st, const QFrag (&qf)[
 }
 
 // ------------------------------------------------------------------ prefill
-constexpr int PF_QB = 2;                   // 16-column blocks a wave
+// A workgroup of 4 waves takes 128 query rows of one (sequence, head), a wave 32 of them (two column
+// blocks).  Blocks of 64 keys go through LDS, double-buffered: while the waves work on one block the
+// next one is on its way from memory into registers.  K lies in LDS as [64 keys][HD + 8], V^T as
+// [HD][64 + 8]; the paddings keep the 16-lane fragment reads free of bank conflicts.
+// Softmax runs in the exp2 domain (scores times scale * log2 e); masking is applied only to blocks
+// that reach beyond a row's causal limit, the window's start or the sequence's end.
+// PV takes k-steps of 32 keys: a lane's 8 probabilities come from two 16-key score tiles, and the
+// V^T fragment is read with the same pairing (keys 4g..4g+3 of either tile for lane group g).
+constexpr int PF_QB = 2;                        // 16-column blocks a wave
 constexpr int PF_WAVES = 4;
+constexpr int PF_THREADS = PF_WAVES * SYN_WAVE;
 constexpr int PF_ROWS = PF_WAVES * PF_QB * 16;  // query rows a workgroup
+constexpr int LDK = HD + 8;
+constexpr int LDV = SYN_PAGE + 8;
+constexpr int PF_TILE = SYN_PAGE * LDK + HD * LDV;          // bf16 elements of one buffer
+constexpr int PF_CHUNKS = (8 * HD + PF_THREADS - 1) / PF_THREADS;  // 16-byte chunks a thread moves for K (and for V)
 
-__global__ void __launch_bounds__(PF_WAVES * SYN_WAVE)
+__global__ void __launch_bounds__(PF_THREADS)
 attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
                     const int* __restrict__ page_table, int table_stride, const int* __restrict__ seq_start,
-                    const int* __restrict__ seq_past, int n_seqs, bf16* __restrict__ out, float scale, int window,
-                    int nh, int nkv) {
-  // which sequence and which rows: tiles are numbered sequence by sequence
-  int seq = -1, q0 = 0, t = 0;
+                    const int* __restrict__ seq_past, int n_seqs, int n_tiles, bf16* __restrict__ out, float scale,
+                    int window, int nh, int nkv) {
+  extern __shared__ __attribute__((aligned(16))) bf16 lds[];  // [2][PF_TILE]
+  // which sequence and which rows: tiles are numbered sequence by sequence; the grid runs through
+  // them backwards so that the tiles with the most key blocks start first
+  const int tile = n_tiles - 1 - (int)blockIdx.x;
+  int seq = -1, q0 = 0, t_acc = 0;
   for (int s = 0; s < n_seqs; ++s) {
     const int nt = (seq_start[s + 1] - seq_start[s] + PF_ROWS - 1) / PF_ROWS;
-    if ((int)blockIdx.x < t + nt) {
+    if (tile < t_acc + nt) {
       seq = s;
-      q0 = ((int)blockIdx.x - t) * PF_ROWS;
+      q0 = (tile - t_acc) * PF_ROWS;
       break;
     }
-    t += nt;
+    t_acc += nt;
   }
-  if (seq < 0) return;
-  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
+  if (seq < 0) return;  // the grid is an upper bound
+  const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE;
+  const int r16 = lane % 16, g4 = lane / 16;
   const int head = blockIdx.y, kvh = head / (nh / nkv);
   const int tok0 = seq_start[seq], n_new = seq_start[seq + 1] - tok0, past = seq_past[seq];
-  const int r0 = q0 + wave * PF_QB * 16;
-  if (r0 >= n_new) return;
   const int kv_len = past + n_new;
+  const int r0 = q0 + wave * PF_QB * 16;
+  const bool wave_on = r0 < n_new;
 
   QFrag qf[PF_QB];
   int qpos[PF_QB], lo[PF_QB];
 #pragma unroll
   for (int c = 0; c < PF_QB; ++c) {
-    const int row = r0 + c * 16 + lane % 16;
+    const int row = r0 + c * 16 + r16;
     const bool valid = row < n_new;
     qpos[c] = valid ? past + row : -1;
     lo[c] = (window > 0 && valid) ? max(0, qpos[c] - window + 1) : 0;
     load_q(qf[c], valid ? q + ((size_t)(tok0 + row) * nh + head) * HD : nullptr, lane);
   }
+  // visible keys of this wave, and of the whole workgroup
+  const int w_kmax = past + min(r0 + PF_QB * 16 - 1, n_new - 1);
+  const int w_qmin = past + r0;                                        // smallest position of the wave
+  const int w_kmin = window > 0 ? max(0, w_qmin - window + 1) : 0;
+  const int g_kmax = past + min(q0 + PF_ROWS - 1, n_new - 1);
+  const int g_kmin = window > 0 ? max(0, past + q0 - window + 1) : 0;
+  const int kb_lo = g_kmin / SYN_PAGE, kb_hi = g_kmax / SYN_PAGE;
+  const float scale2 = scale * 1.44269504088896340736f;
+
   AttnState<PF_QB> st;
   attn_init(st);
-  const int kmax = past + min(r0 + PF_QB * 16 - 1, n_new - 1);
-  const int kmin = window > 0 ? max(0, past + r0 - window + 1) : 0;
-  for (int kb = kmin / SYN_PAGE; kb <= kmax / SYN_PAGE; ++kb) {
+
+  bf16x8 rk[PF_CHUNKS], rv[PF_CHUNKS];
+  auto fetch = [&](int kb) {
     const size_t base = ((size_t)page_table[(size_t)seq * table_stride + kb] * nkv + kvh) * SYN_PAGE * HD;
-    attn_block<PF_QB>(st, qf, k_pages + base, v_pages + base, kb * SYN_PAGE, qpos, lo, kv_len, scale, lane);
+    const bf16* kp = k_pages + base;
+    const bf16* vp = v_pages + base;
+#pragma unroll
+    for (int i = 0; i < PF_CHUNKS; ++i) {
+      const int c = tid + i * PF_THREADS;
+      if (c < 8 * HD) {
+        rk[i] = *(const bf16x8*)(kp + (size_t)c * 8);   // K rows are contiguous: chunk c is elements 8c .. 8c+7
+        rv[i] = *(const bf16x8*)(vp + (size_t)c * 8);   // and so are the rows of V^T
+      }
+    }
+  };
+  auto stash = [&](int buf, int kb) {
+    bf16* ks = lds + buf * PF_TILE;
+    bf16* vs = ks + SYN_PAGE * LDK;
+    const bool ragged = (kb + 1) * SYN_PAGE > kv_len;
+#pragma unroll
+    for (int i = 0; i < PF_CHUNKS; ++i) {
+      const int c = tid + i * PF_THREADS;
+      if (c < 8 * HD) {
+        const int krow = c / (HD / 8), kcol = c % (HD / 8);
+        *(bf16x8*)(ks + krow * LDK + kcol * 8) = rk[i];
+        const int vrow = c / 8, vcol = c % 8;
+        bf16x8 v = rv[i];
+        if (ragged) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (kb * SYN_PAGE + vcol * 8 + e >= kv_len) v[e] = (bf16)0.f;  // 0 * (whatever lies there) must be 0
+        }
+        *(bf16x8*)(vs + vrow * LDV + vcol * 8) = v;
+      }
+    }
+  };
+
+  fetch(kb_lo);
+  stash(0, kb_lo);
+  __syncthreads();
+  for (int kb = kb_lo; kb <= kb_hi; ++kb) {
+    const int buf = (kb - kb_lo) & 1;
+    if (kb < kb_hi) fetch(kb + 1);
+    const int key0 = kb * SYN_PAGE;
+    if (wave_on && key0 <= w_kmax && key0 + SYN_PAGE > w_kmin) {
+      const bf16* ks = lds + buf * PF_TILE;
+      const bf16* vs = ks + SYN_PAGE * LDK;
+      f32x4 s[4][PF_QB];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+#pragma unroll
+        for (int c = 0; c < PF_QB; ++c) s[t][c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        kfrag_t ka[KSTEPS];
+        load_row(ka, ks + (t * 16 + r16) * LDK, lane);
+#pragma unroll
+        for (int kk = 0; kk < KSTEPS; ++kk)
+#pragma unroll
+          for (int c = 0; c < PF_QB; ++c) s[t][c] = mfma_qk(ka[kk], qf[c].k[kk], s[t][c]);
+      }
+      // a block needs masking if some row of the wave does not see all of it
+      const bool need_mask = key0 + SYN_PAGE - 1 > w_qmin ||                   // beyond some row's own position
+                             (window > 0 && key0 < w_kmax - window + 1) ||    // before some row's window
+                             r0 + PF_QB * 16 > n_new;                         // rows of padding
+#pragma unroll
+      for (int c = 0; c < PF_QB; ++c) {
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float v = s[t][c][e] * scale2;
+            if (need_mask) {
+              const int key = key0 + t * 16 + 4 * g4 + e;
+              if (key > qpos[c] || key < lo[c]) v = -INFINITY;
+            }
+            s[t][c][e] = v;
+            mloc = fmaxf(mloc, v);
+          }
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 16, SYN_WAVE));
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, SYN_WAVE));
+        const float m_new = fmaxf(st.m[c], mloc);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a column that has seen no key yet
+        const float alpha = __builtin_amdgcn_exp2f(st.m[c] - m_use);
+        st.m[c] = m_new;
+        float lsum = 0.f;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float p = __builtin_amdgcn_exp2f(s[t][c][e] - m_use);
+            s[t][c][e] = p;
+            lsum += p;
+          }
+        st.l[c] = st.l[c] * alpha + lsum;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) st.o[dt][c] *= alpha;
+      }
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        bf16x8 pb[PF_QB];
+#pragma unroll
+        for (int c = 0; c < PF_QB; ++c)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            pb[c][e] = (bf16)s[2 * tt][c][e];
+            pb[c][4 + e] = (bf16)s[2 * tt + 1][c][e];
+          }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const bf16* vrow = vs + (dt * 16 + r16) * LDV + tt * 32 + 4 * g4;
+          const bf16x4 v0 = *(const bf16x4*)(vrow);
+          const bf16x4 v1 = *(const bf16x4*)(vrow + 16);
+          bf16x8 av;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            av[e] = v0[e];
+            av[4 + e] = v1[e];
+          }
+#pragma unroll
+          for (int c = 0; c < PF_QB; ++c) st.o[dt][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, pb[c], st.o[dt][c], 0, 0, 0);
+        }
+      }
+    }
+    if (kb < kb_hi) stash(buf ^ 1, kb + 1);  // the other buffer was last read before the previous barrier
+    __syncthreads();
   }
+  if (!wave_on) return;
 #pragma unroll
   for (int c = 0; c < PF_QB; ++c) {
     float l = st.l[c];
@@ -217,7 +364,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages
     l += __shfl_xor(l, 32, SYN_WAVE);
     if (qpos[c] < 0) continue;
     const float inv = 1.f / l;
-    bf16* orow = out + ((size_t)(tok0 + r0 + c * 16 + lane % 16) * nh + head) * HD + 4 * (lane / 16);
+    bf16* orow = out + ((size_t)(tok0 + r0 + c * 16 + r16) * nh + head) * HD + 4 * g4;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       bf16x4 v;
@@ -237,9 +384,17 @@ SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, co
   SYN_CHECK(nh % nkv == 0, "attention_prefill: %d heads do not divide into %d kv heads", nh, nkv);
   SYN_CHECK(nh <= 65535, "attention_prefill: %d heads exceed the grid", nh);
   const int tiles = n_tokens / PF_ROWS + n_seqs;  // an upper bound; surplus workgroups leave at once
-  attn_prefill_kernel<<<dim3(tiles, nh), PF_WAVES * SYN_WAVE, 0, stream>>>(
+  const size_t lds = (size_t)2 * PF_TILE * sizeof(bf16);
+  static bool raised = false;
+  if (lds > 65536 && !raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)lds);
+    SYN_CHECK(e == hipSuccess, "attention_prefill: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
+    raised = true;
+  }
+  attn_prefill_kernel<<<dim3(tiles, nh), PF_THREADS, lds, stream>>>(
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, page_table, table_stride, seq_start, seq_past, n_seqs,
-      (bf16*)out, scale, window, nh, nkv);
+      tiles, (bf16*)out, scale, window, nh, nkv);
   SYN_LAUNCH_CHECK("attention_prefill");
   return 0;
 }
