@@ -4,7 +4,7 @@
 //                  the MFMA kernels refuse (K not a multiple of 8, unaligned rows).
 //   gemm_skinny    bf16, M <= 64: the weight matrix is streamed once from HBM through
 //                  v_mfma_f32_16x16x32_bf16; the waves of a workgroup split K and sum in LDS.
-//   gemm_tiled     bf16, M > 64: 128x128x32 tiles in LDS, 2x2 waves of 64x64,
+//   gemm_tiled     bf16, M > 64: 256x128x32 (or smaller) tiles in LDS, double-buffered, 2x2 waves,
 //                  v_mfma_f32_32x32x16_bf16.
 //
 // Reference counterparts: crates/synaptix-kernels-cuda/src/best_cu/gemm/gemm_bf16.cu (TN family,
@@ -74,6 +74,8 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
   const int n0 = blockIdx.x * (RT * 16);
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
+  // Rows of W beyond N are read from the last valid row (their results are never stored); rows of x
+  // beyond M are not loaded at all: the fewer lanes a load of x has, the less it costs.
   const bf16* wrow[RT];
 #pragma unroll
   for (int r = 0; r < RT; ++r) wrow[r] = w + (size_t)min(n0 + r * 16 + r16, N - 1) * K + kq;
@@ -92,16 +94,16 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
 
   // U chunks of 32 at a time: all loads of a group are issued before the first product needs them,
   // so that a wave keeps U * RT KiB of the weight stream in flight
-  for (int k0 = wave * (32 * U); k0 < K; k0 += WAVES * 32 * U) {
+  constexpr int GROUP = 32 * U;
+  const int k_full = K / (WAVES * GROUP) * (WAVES * GROUP);
+  for (int k0 = wave * GROUP; k0 < k_full; k0 += WAVES * GROUP) {
     bf16x8 bw[U][RT], ax[U][MB];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int k = k0 + u * 32;
-      const bool kin = k + kq < K;  // K is a multiple of 8: a chunk of 8 lies inside or outside as a whole
 #pragma unroll
-      for (int r = 0; r < RT; ++r) bw[u][r] = kin ? __builtin_nontemporal_load((const bf16x8*)(wrow[r] + k)) : zero;
+      for (int r = 0; r < RT; ++r) bw[u][r] = __builtin_nontemporal_load((const bf16x8*)(wrow[r] + k0 + u * 32));
 #pragma unroll
-      for (int b = 0; b < MB; ++b) ax[u][b] = (kin && xok[b]) ? *(const bf16x8*)(xrow[b] + k) : zero;
+      for (int b = 0; b < MB; ++b) ax[u][b] = xok[b] ? *(const bf16x8*)(xrow[b] + k0 + u * 32) : zero;
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -110,6 +112,20 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
 #pragma unroll
         for (int r = 0; r < RT; ++r)
           acc[b][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[u][b], bw[u][r], acc[b][r], 0, 0, 0);
+  }
+  // what is left of K, chunk by chunk; K is a multiple of 8, so a lane's 8 elements lie inside or
+  // outside as a whole
+  for (int k0 = k_full + wave * 32; k0 < K; k0 += WAVES * 32) {
+    const bool kin = k0 + kq < K;
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      const bf16x8 ax = (kin && xok[b]) ? *(const bf16x8*)(xrow[b] + k0) : zero;
+#pragma unroll
+      for (int r = 0; r < RT; ++r) {
+        const bf16x8 bw = kin ? *(const bf16x8*)(wrow[r] + k0) : zero;
+        acc[b][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, bw, acc[b][r], 0, 0, 0);
+      }
+    }
   }
 
   // sum the waves' partial tiles in a fixed order
@@ -152,54 +168,70 @@ static void launch_skinny(const bf16* x, const bf16* w, void* out, int out_is_f3
 }
 
 // ------------------------------------------------------------------ tiled, bf16, large M
-// Block tile 128 (m) x 128 (n) x 32 (k); 4 waves as 2x2, each 64x64 = 2x2 MFMA 32x32x16 tiles.
+// Block tile BM (m) x BN (n) x 32 (k); 4 waves as 2x2, each (BM/2) x (BN/2) of MFMA 32x32x16 tiles.
 // MFMA 32x32x16: A = x rows, B = W rows; lane holds row lane%32, k = 8*(lane/32) .. +8;
 // D[m = 8*(j/4) + 4*(lane/32) + j%4][n = lane%32], j = 0..15.
-#define TG_BM 128
-#define TG_BN 128
-#define TG_BK 32
-#define TG_LD (TG_BK + 8)  // padded row of the LDS tiles, in bf16 elements (80 bytes)
-
-__global__ void __launch_bounds__(256)
+// LDS tiles are double-buffered: while one k-tile is multiplied the next is on its way from memory
+// into registers, and is stored into the other buffer before the barrier.
+template <int BM, int BN, int BK, bool KTAIL>
+__global__ void __launch_bounds__(256, ((BM + BN) * (BK + 8) * 4 <= 80 * 1024 && BM * BN <= 256 * 128 ? 2 : 1))
 gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
                   int M, int N, int K) {
-  __shared__ __attribute__((aligned(16))) bf16 xs[2][TG_BM * TG_LD];
-  __shared__ __attribute__((aligned(16))) bf16 ws[2][TG_BN * TG_LD];
+  constexpr int LD = BK + 8;                         // padded row of the LDS tiles, in bf16 elements
+  constexpr int TM = BM / 64, TN = BN / 64;          // 32x32 tiles a wave holds in m and n
+  constexpr int CPR = BK / 8;                        // 16-byte chunks in a tile row
+  constexpr int RPP = 256 / CPR;                     // tile rows the workgroup moves in one pass
+  constexpr int XL = BM / RPP, WL = BN / RPP;        // passes for x and for W
+  extern __shared__ __attribute__((aligned(16))) bf16 smem[];  // [2][(BM + BN) * LD]
   const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE;
-  const int wm = (wave / 2) * 64, wn = (wave % 2) * 64;
-  const int m0 = blockIdx.y * TG_BM, n0 = blockIdx.x * TG_BN;
+  const int wm = (wave / 2) * (BM / 2), wn = (wave % 2) * (BN / 2);
+  // Which tile: workgroup b runs on XCD b % 8, and each XCD has an L2 of its own.  Tiles are grouped
+  // into panels of PM x PN (m fastest); a panel goes to one XCD, so the workgroups that run there at
+  // the same time share rows of x and of W in its L2.
+  const int tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM;
+  const int PM = min(8, tiles_m), PN = 4;
+  const int panels_m = (tiles_m + PM - 1) / PM;
+  const int xcd = (int)blockIdx.x % 8, local = (int)blockIdx.x / 8;
+  const int panel = (local / (PM * PN)) * 8 + xcd, in_panel = local % (PM * PN);
+  const int tm = (panel % panels_m) * PM + in_panel % PM, tn = (panel / panels_m) * PN + in_panel / PM;
+  if (tm >= tiles_m || tn >= tiles_n) return;
+  const int m0 = tm * BM, n0 = tn * BN;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  // global -> LDS: each tile is 128 rows x 4 chunks of 8; 512 chunks, 2 a thread
-  const int lrow = tid / 4, lchunk = (tid % 4) * 8;  // rows lrow and lrow + 64
-  const bf16* xg0 = x + (size_t)min(m0 + lrow, M - 1) * K + lchunk;
-  const bf16* xg1 = x + (size_t)min(m0 + lrow + 64, M - 1) * K + lchunk;
-  const bf16* wg0 = w + (size_t)min(n0 + lrow, N - 1) * K + lchunk;
-  const bf16* wg1 = w + (size_t)min(n0 + lrow + 64, N - 1) * K + lchunk;
+  // global -> LDS: thread t moves chunk t % CPR of rows t / CPR + RPP * i
+  const int lrow = tid / CPR, lchunk = (tid % CPR) * 8;
+  const bf16* xg[XL];
+  const bf16* wg[WL];
+#pragma unroll
+  for (int i = 0; i < XL; ++i) xg[i] = x + (size_t)min(m0 + lrow + RPP * i, M - 1) * K + lchunk;
+#pragma unroll
+  for (int i = 0; i < WL; ++i) wg[i] = w + (size_t)min(n0 + lrow + RPP * i, N - 1) * K + lchunk;
 
-  f32x16 acc[2][2];
+  f32x16 acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  const int nk = (K + TG_BK - 1) / TG_BK;
-  bf16x8 rx0, rx1, rw0, rw1;
+  const int nk = (K + BK - 1) / BK;
+  bf16x8 rx[XL], rw[WL];
   auto fetch = [&](int kt) {
-    const int k = kt * TG_BK + lchunk;
-    const bool kin = k < K;
-    rx0 = kin ? *(const bf16x8*)(xg0 + (size_t)kt * TG_BK) : zero;
-    rx1 = kin ? *(const bf16x8*)(xg1 + (size_t)kt * TG_BK) : zero;
-    rw0 = kin ? *(const bf16x8*)(wg0 + (size_t)kt * TG_BK) : zero;
-    rw1 = kin ? *(const bf16x8*)(wg1 + (size_t)kt * TG_BK) : zero;
+    // K is a multiple of 8: a chunk lies inside or outside as a whole
+    const bool kin = !KTAIL || kt * BK + lchunk < K;
+#pragma unroll
+    for (int i = 0; i < XL; ++i) rx[i] = kin ? *(const bf16x8*)(xg[i] + (size_t)kt * BK) : zero;
+#pragma unroll
+    for (int i = 0; i < WL; ++i) rw[i] = kin ? *(const bf16x8*)(wg[i] + (size_t)kt * BK) : zero;
   };
   auto stash = [&](int buf) {
-    *(bf16x8*)(&xs[buf][lrow * TG_LD + lchunk]) = rx0;
-    *(bf16x8*)(&xs[buf][(lrow + 64) * TG_LD + lchunk]) = rx1;
-    *(bf16x8*)(&ws[buf][lrow * TG_LD + lchunk]) = rw0;
-    *(bf16x8*)(&ws[buf][(lrow + 64) * TG_LD + lchunk]) = rw1;
+    bf16* xs = smem + buf * (BM + BN) * LD;
+    bf16* ws = xs + BM * LD;
+#pragma unroll
+    for (int i = 0; i < XL; ++i) *(bf16x8*)(xs + (lrow + RPP * i) * LD + lchunk) = rx[i];
+#pragma unroll
+    for (int i = 0; i < WL; ++i) *(bf16x8*)(ws + (lrow + RPP * i) * LD + lchunk) = rw[i];
   };
 
   fetch(0);
@@ -209,26 +241,28 @@ gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* 
   for (int kt = 0; kt < nk; ++kt) {
     const int buf = kt & 1;
     if (kt + 1 < nk) fetch(kt + 1);
+    const bf16* xs = smem + buf * (BM + BN) * LD;
+    const bf16* ws = xs + BM * LD;
 #pragma unroll
-    for (int ks = 0; ks < TG_BK; ks += 16) {
-      bf16x8 a[2], b[2];
+    for (int ks = 0; ks < BK; ks += 16) {
+      bf16x8 a[TM], b[TN];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) a[i] = *(const bf16x8*)(&xs[buf][(wm + i * 32 + fr) * TG_LD + ks + fk]);
+      for (int i = 0; i < TM; ++i) a[i] = *(const bf16x8*)(xs + (wm + i * 32 + fr) * LD + ks + fk);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) b[j] = *(const bf16x8*)(&ws[buf][(wn + j * 32 + fr) * TG_LD + ks + fk]);
+      for (int j = 0; j < TN; ++j) b[j] = *(const bf16x8*)(ws + (wn + j * 32 + fr) * LD + ks + fk);
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
     }
     if (kt + 1 < nk) stash(buf ^ 1);  // the other buffer was last read before the previous barrier
     __syncthreads();
   }
 
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int m = m0 + wm + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
@@ -240,6 +274,31 @@ gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* 
             ((bf16*)out)[(size_t)m * N + n] = (bf16)acc[i][j][e];
         }
       }
+}
+
+template <int BM, int BN, int BK>
+static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
+                        hipStream_t stream) {
+  const int tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM;
+  const int PM = tiles_m < 8 ? tiles_m : 8, PN = 4;
+  const int panels = ((tiles_m + PM - 1) / PM) * ((tiles_n + PN - 1) / PN);
+  const int grid = (panels + 7) / 8 * 8 * PM * PN;
+  const size_t lds = (size_t)2 * (BM + BN) * (BK + 8) * sizeof(bf16);
+  static bool raised = false;
+  if (lds > 65536 && !raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, false>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, true>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    SYN_CHECK(e == hipSuccess, "gemm: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
+    raised = true;
+  }
+  if (K % BK == 0)
+    gemm_tiled_kernel<BM, BN, BK, false><<<grid, 256, lds, stream>>>(x, w, out, out_is_f32, M, N, K);
+  else
+    gemm_tiled_kernel<BM, BN, BK, true><<<grid, 256, lds, stream>>>(x, w, out, out_is_f32, M, N, K);
+  return 0;
 }
 
 // ------------------------------------------------------------------ entry point
@@ -269,7 +328,7 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   // rows of W a workgroup owns: more rows amortise the loads of x, fewer rows give more workgroups
   const int variant = getenv("SYN_SKINNY") ? atoi(getenv("SYN_SKINNY")) : -1;
   if (M <= 16) {
-    const int v = variant >= 0 ? variant : (N <= 8192 ? 0 : (N <= 32768 ? 2 : 3));
+    const int v = variant >= 0 ? variant : (N <= 8192 ? 0 : 1);
     if (v == 0) launch_skinny<1, 1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
     else if (v == 1) launch_skinny<1, 1, 8, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
     else if (v == 2) launch_skinny<1, 2, 8, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
@@ -277,7 +336,7 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
     else if (v == 4) launch_skinny<1, 2, 16, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
     else launch_skinny<1, 4, 8, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
   } else if (M <= 32) {
-    const int v = variant >= 0 ? variant : (N <= 8192 ? 0 : 2);
+    const int v = variant >= 0 ? variant : (N <= 4096 ? 0 : (N <= 8192 ? 1 : 2));
     if (v == 0) launch_skinny<2, 1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
     else if (v == 1) launch_skinny<2, 2, 8, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
     else if (v == 2) launch_skinny<2, 4, 8, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
@@ -286,15 +345,26 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   } else if (M <= 48) {
     launch_skinny<3, 2, 8, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
   } else if (M <= 64) {
-    const int v = variant >= 0 ? variant : (N <= 8192 ? 0 : 2);
+    const int v = variant >= 0 ? variant : (N <= 4096 ? 0 : (N <= 8192 ? 3 : 4));
     if (v == 0) launch_skinny<4, 1, 16, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
     else if (v == 1) launch_skinny<4, 2, 8, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
     else if (v == 2) launch_skinny<4, 4, 8, 1>(xb, wb, out, out_is_f32, M, N, K, stream);
     else if (v == 3) launch_skinny<4, 2, 16, 1>(xb, wb, out, out_is_f32, M, N, K, stream);
     else launch_skinny<4, 4, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
   } else {
-    const dim3 grid((N + TG_BN - 1) / TG_BN, (M + TG_BM - 1) / TG_BM);
-    gemm_tiled_kernel<<<grid, 256, 0, stream>>>(xb, wb, out, out_is_f32, M, N, K);
+    // tile shapes: 256 x 128 where that leaves no compute unit idle, smaller tiles for small problems
+    const int tv = getenv("SYN_TILED") ? atoi(getenv("SYN_TILED")) : -1;
+    const long t256 = (long)((M + 255) / 256) * ((N + 127) / 128);
+    const int v = tv >= 0 ? tv : 1;
+    (void)t256;
+    int rc;
+    if (v == 0) rc = launch_tiled<256, 128, 32>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 1) rc = launch_tiled<128, 128, 64>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 2) rc = launch_tiled<128, 128, 32>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 3) rc = launch_tiled<256, 128, 64>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 4) rc = launch_tiled<128, 128, 128>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else rc = launch_tiled<128, 256, 64>(xb, wb, out, out_is_f32, M, N, K, stream);
+    if (rc) return rc;
   }
   SYN_LAUNCH_CHECK("gemm");
   return 0;
