@@ -63,14 +63,73 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const float* __res
   }
 }
 
+// The same for rows whose width is a multiple of 4 and at most 4 * VPT * blockDim: every thread
+// keeps its values (float4 loads) in registers between the sum of squares and the scaling.
+template <typename TOut, int VPT>
+__global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const float* __restrict__ delta,
+                                       const int* __restrict__ rows, const void* __restrict__ gain, int gain_is_f32,
+                                       float eps, TOut* __restrict__ out, int H) {
+  __shared__ float red[16];
+  const int r = rows ? rows[blockIdx.x] : blockIdx.x;
+  float4* x = (float4*)(resid + (size_t)r * H);
+  const float4* d = delta ? (const float4*)(delta + (size_t)r * H) : nullptr;
+  TOut* o = out + (size_t)blockIdx.x * H;
+  const bool write_back = (rows == nullptr) && (d != nullptr);
+  const int H4 = H / 4;
+  float4 v[VPT];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = threadIdx.x + j * blockDim.x;
+    if (i < H4) {
+      v[j] = x[i];
+      if (d) {
+        const float4 t = d[i];
+        v[j].x += t.x;
+        v[j].y += t.y;
+        v[j].z += t.z;
+        v[j].w += t.w;
+      }
+      if (write_back) x[i] = v[j];
+      ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+    }
+  }
+  ss = block_sum(ss, red);
+  const float inv = rsqrtf(ss / (float)H + eps);
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = threadIdx.x + j * blockDim.x;
+    if (i < H4) {
+      const float e[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+#pragma unroll
+      for (int c = 0; c < 4; ++c) o[4 * i + c] = from_f32<TOut>(load_gain(gain, gain_is_f32, 4 * i + c) * e[c] * inv);
+    }
+  }
+}
+
 SYN_EXPORT int syn_add_rmsnorm(float* resid, const float* delta, const int* rows, int n_out, const void* gain,
                                int gain_is_f32, float eps, void* out, int out_is_f32, int H, hipStream_t stream) {
   SYN_CHECK(n_out > 0 && H > 0, "add_rmsnorm: empty input (%d rows, width %d)", n_out, H);
-  int block = H >= 4096 ? 1024 : (H >= 1024 ? 512 : 256);
-  if (out_is_f32)
-    add_rmsnorm_kernel<float><<<n_out, block, 0, stream>>>(resid, delta, rows, gain, gain_is_f32, eps, (float*)out, H);
-  else
-    add_rmsnorm_kernel<bf16><<<n_out, block, 0, stream>>>(resid, delta, rows, gain, gain_is_f32, eps, (bf16*)out, H);
+  const bool vec = H % 4 == 0 && H <= 4 * 4 * 512 && ((uintptr_t)resid % 16 == 0) && ((uintptr_t)delta % 16 == 0);
+  if (vec) {
+    const int H4 = H / 4;
+    const int block = H4 <= 256 ? 256 : 512;
+    const int vpt = (H4 + block - 1) / block;  // 1 .. 4
+#define SYN_ARN(T, V)                                                                                         \
+  add_rmsnorm_vec_kernel<T, V><<<n_out, block, 0, stream>>>(resid, delta, rows, gain, gain_is_f32, eps, (T*)out, H)
+    if (out_is_f32) {
+      if (vpt == 1) SYN_ARN(float, 1); else if (vpt == 2) SYN_ARN(float, 2); else SYN_ARN(float, 4);
+    } else {
+      if (vpt == 1) SYN_ARN(bf16, 1); else if (vpt == 2) SYN_ARN(bf16, 2); else SYN_ARN(bf16, 4);
+    }
+#undef SYN_ARN
+  } else {
+    const int block = H >= 4096 ? 1024 : (H >= 1024 ? 512 : 256);
+    if (out_is_f32)
+      add_rmsnorm_kernel<float><<<n_out, block, 0, stream>>>(resid, delta, rows, gain, gain_is_f32, eps, (float*)out, H);
+    else
+      add_rmsnorm_kernel<bf16><<<n_out, block, 0, stream>>>(resid, delta, rows, gain, gain_is_f32, eps, (bf16*)out, H);
+  }
   SYN_LAUNCH_CHECK("add_rmsnorm");
   return 0;
 }
@@ -125,8 +184,35 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
   }
 }
 
+// 8 values a thread with 16-byte loads (bf16, width a multiple of 8)
+__global__ void swiglu_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int n_rows, int I) {
+  const int I8 = I / 8;
+  const size_t total = (size_t)n_rows * I8;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t n = idx / I8;
+    const int i = (int)(idx - n * I8) * 8;
+    const bf16x8 g = *(const bf16x8*)(gu + n * 2 * I + i);
+    const bf16x8 u = *(const bf16x8*)(gu + n * 2 * I + I + i);
+    bf16x8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float gf = (float)g[e];
+      o[e] = (bf16)(gf / (1.f + expf(-gf)) * (float)u[e]);
+    }
+    *(bf16x8*)(out + n * I + i) = o;
+  }
+}
+
 SYN_EXPORT int syn_swiglu(const void* gu, void* out, int is_f32, int n_rows, int I, hipStream_t stream) {
   SYN_CHECK(n_rows > 0 && I > 0, "swiglu: empty input (%d rows, width %d)", n_rows, I);
+  if (!is_f32 && I % 8 == 0 && (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    const size_t total = (size_t)n_rows * (I / 8);
+    int grid = (int)((total + 255) / 256);
+    if (grid > 65536) grid = 65536;
+    swiglu_vec8_kernel<<<grid, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, n_rows, I);
+    SYN_LAUNCH_CHECK("swiglu");
+    return 0;
+  }
   const size_t total = (size_t)n_rows * I;
   int grid = (int)((total + 255) / 256);
   if (grid > 65536) grid = 65536;
@@ -171,15 +257,19 @@ __global__ void qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, T* __res
   if (active) {
     const T* src = qkv + ((size_t)tok * heads + head) * hd;
     float ss = 0.f;
-    for (int d = lane; d < hd; d += SYN_WAVE) {
-      const float v = to_f32<T>(src[d]);
-      xs[d] = v;
-      ss += v * v;
+    for (int d = 2 * lane; d < hd; d += 2 * SYN_WAVE) {  // head sizes are even: two values a lane
+      const float v0 = to_f32<T>(src[d]), v1 = to_f32<T>(src[d + 1]);
+      xs[d] = v0;
+      xs[d + 1] = v1;
+      ss += v0 * v0 + v1 * v1;
     }
     if (gain) {
       ss = wave_sum(ss);
       const float inv = rsqrtf(ss / (float)hd + eps);
-      for (int d = lane; d < hd; d += SYN_WAVE) xs[d] = load_gain(gain, gain_is_f32, d) * xs[d] * inv;
+      for (int d = 2 * lane; d < hd; d += 2 * SYN_WAVE) {
+        xs[d] = load_gain(gain, gain_is_f32, d) * xs[d] * inv;
+        xs[d + 1] = load_gain(gain, gain_is_f32, d + 1) * xs[d + 1] * inv;
+      }
     }
   }
   __syncthreads();  // lanes read what other lanes of their wave wrote
@@ -202,7 +292,7 @@ __global__ void qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, T* __res
   }
   const bool rotate = (is_q || is_k) && cos_t != nullptr;
   const int half = rot / 2;
-  for (int d = lane; d < hd; d += SYN_WAVE) {
+  auto rotated = [&](int d) {
     float o = xs[d];
     if (rotate && d < rot) {
       if (d < half) {
@@ -213,7 +303,11 @@ __global__ void qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, T* __res
         o = xs[d] * c + xs[d - half] * s;
       }
     }
-    dst[(size_t)d * dst_stride] = from_f32<T>(o);
+    return o;
+  };
+  for (int d = 2 * lane; d < hd; d += 2 * SYN_WAVE) {
+    dst[(size_t)d * dst_stride] = from_f32<T>(rotated(d));
+    dst[(size_t)(d + 1) * dst_stride] = from_f32<T>(rotated(d + 1));
   }
 }
 
@@ -225,6 +319,7 @@ SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, void* q_out, void* k_p
   SYN_CHECK(n_tokens > 0 && nh > 0 && nkv > 0 && hd > 0, "qk_norm_rope_kv_write: empty input");
   SYN_CHECK(rot % 2 == 0 && rot >= 0 && rot <= hd, "qk_norm_rope_kv_write: rotary size %d does not fit head size %d",
             rot, hd);
+  SYN_CHECK(hd % 2 == 0, "qk_norm_rope_kv_write: head size %d is odd", hd);
   SYN_CHECK((cos_t == nullptr) == (sin_t == nullptr), "qk_norm_rope_kv_write: cos and sin come together");
   const int wpb = 4;
   const int heads = nh + 2 * nkv;
