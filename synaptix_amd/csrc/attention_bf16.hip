@@ -9,6 +9,11 @@
 //   v_mfma_f32_16x16x32_bf16 : A[i=lane%16][k=8*(lane/16)+e], B[k=8*(lane/16)+e][n=lane%16]
 //   v_mfma_f32_16x16x16_bf16 : A[i=lane%16][k=4*(lane/16)+e], B[k=4*(lane/16)+e][n=lane%16]
 //   both                     : D[i=4*(lane/16)+e][n=lane%16]
+// Which key a row of a 16-row score tile stands for is free, as long as the masks and the V^T
+// fragments follow: tile t = 2h + u of a block covers, for lane group g = lane / 16, the keys
+// 32h + 8g + 4u .. + 3.  The two tiles of a half h then give a lane the probabilities of the 8
+// consecutive keys 32h + 8g .. + 7: the B operand of one 16x16x32 step, whose V^T fragment is one
+// 16-byte load.
 // Scores, maxima, exponentials and sums are 32-bit; P is rounded to bf16 for the second product
 // (as crates/synaptix-kernels-cuda/src/cu/fused/attention/flash_splitq.cu:187-600 does); the output
 // is rounded once.
@@ -54,6 +59,14 @@ __device__ __forceinline__ f32x4 mfma_qk(bf16x8 a, bf16x8 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
+// key (inside its block of 64) that row r of score tile t stands for, and that element e of lane
+// group g's accumulator of tile t belongs to
+__device__ __forceinline__ int tile_row_key(int t, int r) { return (t / 2) * 32 + 8 * (r / 4) + 4 * (t % 2) + r % 4; }
+__device__ __forceinline__ int acc_key(int t, int g, int e) { return (t / 2) * 32 + 8 * g + 4 * (t % 2) + e; }
+
+// where the row of key k lies when a block's K rows are stored tile after tile (the inverse of tile_row_key)
+__device__ __forceinline__ int tile_slot(int k) { return 16 * (2 * (k / 32) + (k % 8) / 4) + 4 * ((k % 32) / 8) + k % 4; }
+
 // the fragments of one row of HD elements: in k-step ks, lane group g = lane / 16 holds elements ks*4*KW + KW*g .. + KW
 __device__ __forceinline__ void load_row(kfrag_t (&f)[KSTEPS], const bf16* row, int lane) {
 #pragma unroll
@@ -89,89 +102,14 @@ __device__ __forceinline__ void attn_init(AttnState<QB>& st) {
   }
 }
 
-// One block of 64 keys starting at key0.  qpos[c] / lo[c]: visible keys of this lane's column in
-// column block c are lo <= key <= qpos (qpos < 0: the column is padding).  kv_len: keys at and
-// beyond it hold no data of this sequence.
-template <int QB>
-__device__ __forceinline__ void attn_block(AttnState<QB>& st, const QFrag (&qf)[QB], const bf16* __restrict__ kpage,
-                                           const bf16* __restrict__ vpage, int key0, const int (&qpos)[QB],
-                                           const int (&lo)[QB], int kv_len, float scale, int lane) {
-  const int r16 = lane % 16, g4 = lane / 16;
-  f32x4 s[4][QB];
-#pragma unroll
-  for (int t = 0; t < 4; ++t) {
-#pragma unroll
-    for (int c = 0; c < QB; ++c) s[t][c] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    kfrag_t ka[KSTEPS];
-    load_row(ka, kpage + (size_t)(t * 16 + r16) * HD, lane);
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks)
-#pragma unroll
-      for (int c = 0; c < QB; ++c) s[t][c] = mfma_qk(ka[ks], qf[c].k[ks], s[t][c]);
-  }
-#pragma unroll
-  for (int c = 0; c < QB; ++c) {
-    float mloc = -INFINITY;
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int key = key0 + t * 16 + 4 * g4 + e;
-        float v = s[t][c][e] * scale;
-        if (key > qpos[c] || key < lo[c]) v = -INFINITY;
-        s[t][c][e] = v;
-        mloc = fmaxf(mloc, v);
-      }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, SYN_WAVE));
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, SYN_WAVE));
-    const float m_new = fmaxf(st.m[c], mloc);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a column that has seen no key yet
-    const float alpha = __expf(st.m[c] - m_use);
-    st.m[c] = m_new;
-    float lsum = 0.f;
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float p = __expf(s[t][c][e] - m_use);
-        s[t][c][e] = p;
-        lsum += p;
-      }
-    st.l[c] = st.l[c] * alpha + lsum;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) st.o[dt][c] *= alpha;
-  }
-  const bool ragged = key0 + SYN_PAGE > kv_len;  // only the sequence's last page
-#pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    bf16x4 pb[QB];
-#pragma unroll
-    for (int c = 0; c < QB; ++c)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) pb[c][e] = (bf16)s[t][c][e];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      bf16x4 av = *(const bf16x4*)(vpage + (size_t)(dt * 16 + r16) * SYN_PAGE + t * 16 + 4 * g4);
-      if (ragged) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (key0 + t * 16 + 4 * g4 + e >= kv_len) av[e] = (bf16)0.f;  // 0 * (whatever lies there) must be 0
-      }
-#pragma unroll
-      for (int c = 0; c < QB; ++c) st.o[dt][c] = mfma16(av, pb[c], st.o[dt][c]);
-    }
-  }
-}
-
 // ------------------------------------------------------------------ prefill
 // A workgroup of 4 waves takes 128 query rows of one (sequence, head), a wave 32 of them (two column
 // blocks).  Blocks of 64 keys go through LDS, double-buffered: while the waves work on one block the
-// next one is on its way from memory into registers.  K lies in LDS as [64 keys][HD + 8], V^T as
+// next one is on its way from memory into registers.  K lies in LDS as [64 keys, in tile order][HD + 8], V^T as
 // [HD][64 + 8]; the paddings keep the 16-lane fragment reads free of bank conflicts.
 // Softmax runs in the exp2 domain (scores times scale * log2 e); masking is applied only to blocks
 // that reach beyond a row's causal limit, the window's start or the sequence's end.
-// PV takes k-steps of 32 keys: a lane's 8 probabilities come from two 16-key score tiles, and the
-// V^T fragment is read with the same pairing (keys 4g..4g+3 of either tile for lane group g).
+// PV takes k-steps of 32 keys (see the key permutation above).
 constexpr int PF_QB = 2;                        // 16-column blocks a wave
 constexpr int PF_WAVES = 4;
 constexpr int PF_THREADS = PF_WAVES * SYN_WAVE;
@@ -253,8 +191,8 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages
     for (int i = 0; i < PF_CHUNKS; ++i) {
       const int c = tid + i * PF_THREADS;
       if (c < 8 * HD) {
-        const int krow = c / (HD / 8), kcol = c % (HD / 8);
-        *(bf16x8*)(ks + krow * LDK + kcol * 8) = rk[i];
+        const int key = c / (HD / 8), kcol = c % (HD / 8);
+        *(bf16x8*)(ks + tile_slot(key) * LDK + kcol * 8) = rk[i];
         const int vrow = c / 8, vcol = c % 8;
         bf16x8 v = rv[i];
         if (ragged) {
@@ -283,7 +221,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages
 #pragma unroll
         for (int c = 0; c < PF_QB; ++c) s[t][c] = (f32x4){0.f, 0.f, 0.f, 0.f};
         kfrag_t ka[KSTEPS];
-        load_row(ka, ks + (t * 16 + r16) * LDK, lane);
+        load_row(ka, ks + (t * 16 + r16) * LDK, lane);  // rows lie in LDS in tile order
 #pragma unroll
         for (int kk = 0; kk < KSTEPS; ++kk)
 #pragma unroll
@@ -302,7 +240,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages
           for (int e = 0; e < 4; ++e) {
             float v = s[t][c][e] * scale2;
             if (need_mask) {
-              const int key = key0 + t * 16 + 4 * g4 + e;
+              const int key = key0 + acc_key(t, g4, e);
               if (key > qpos[c] || key < lo[c]) v = -INFINITY;
             }
             s[t][c][e] = v;
@@ -339,15 +277,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages
           }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-          const bf16* vrow = vs + (dt * 16 + r16) * LDV + tt * 32 + 4 * g4;
-          const bf16x4 v0 = *(const bf16x4*)(vrow);
-          const bf16x4 v1 = *(const bf16x4*)(vrow + 16);
-          bf16x8 av;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            av[e] = v0[e];
-            av[4 + e] = v1[e];
-          }
+          const bf16x8 av = *(const bf16x8*)(vs + (dt * 16 + r16) * LDV + tt * 32 + 8 * g4);
 #pragma unroll
           for (int c = 0; c < PF_QB; ++c) st.o[dt][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, pb[c], st.o[dt][c], 0, 0, 0);
         }
@@ -415,13 +345,13 @@ __device__ __forceinline__ void attn_block_decode(AttnState<1>& st, const QFrag&
                                                   int kv_len, float scale, int lane) {
   const int r16 = lane % 16, g4 = lane / 16;
   kfrag_t ka[4][KSTEPS];
-  bf16x4 va[4][DT];
+  bf16x8 va[2][DT];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) load_row(ka[t], kpage + (size_t)(t * 16 + r16) * HD, lane);
+  for (int t = 0; t < 4; ++t) load_row(ka[t], kpage + (size_t)tile_row_key(t, r16) * HD, lane);
 #pragma unroll
-  for (int t = 0; t < 4; ++t)
+  for (int h = 0; h < 2; ++h)
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) va[t][dt] = *(const bf16x4*)(vpage + (size_t)(dt * 16 + r16) * SYN_PAGE + t * 16 + 4 * g4);
+    for (int dt = 0; dt < DT; ++dt) va[h][dt] = *(const bf16x8*)(vpage + (size_t)(dt * 16 + r16) * SYN_PAGE + h * 32 + 8 * g4);
 
   f32x4 s[4];
 #pragma unroll
@@ -435,7 +365,7 @@ __device__ __forceinline__ void attn_block_decode(AttnState<1>& st, const QFrag&
   for (int t = 0; t < 4; ++t)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const int key = key0 + t * 16 + 4 * g4 + e;
+      const int key = key0 + acc_key(t, g4, e);
       float v = s[t][e] * scale;
       if (key > qpos || key < lo) v = -INFINITY;
       s[t][e] = v;
@@ -461,19 +391,22 @@ __device__ __forceinline__ void attn_block_decode(AttnState<1>& st, const QFrag&
   for (int dt = 0; dt < DT; ++dt) st.o[dt][0] *= alpha;
   const bool ragged = key0 + SYN_PAGE > kv_len;
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    bf16x4 pb;
+  for (int h = 0; h < 2; ++h) {
+    bf16x8 pb;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) pb[e] = (bf16)s[t][e];
+    for (int e = 0; e < 4; ++e) {
+      pb[e] = (bf16)s[2 * h][e];
+      pb[4 + e] = (bf16)s[2 * h + 1][e];
+    }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      bf16x4 av = va[t][dt];
+      bf16x8 av = va[h][dt];
       if (ragged) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (key0 + t * 16 + 4 * g4 + e >= kv_len) av[e] = (bf16)0.f;
+        for (int e = 0; e < 8; ++e)
+          if (key0 + h * 32 + 8 * g4 + e >= kv_len) av[e] = (bf16)0.f;  // 0 * (whatever lies there) must be 0
       }
-      st.o[dt][0] = mfma16(av, pb, st.o[dt][0]);
+      st.o[dt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, pb, st.o[dt][0], 0, 0, 0);
     }
   }
 }
