@@ -18,7 +18,7 @@
 // (as crates/synaptix-kernels-cuda/src/cu/fused/attention/flash_splitq.cu:187-600 does); the output
 // is rounded once.
 //
-//   prefill: a workgroup of 4 waves takes 128 query rows of one (sequence, head); a wave 32 of them.
+//   prefill: a workgroup of 8 waves takes 128 query rows of one (sequence, head); a wave 16 of them.
 //   decode : a workgroup takes (sequence, kv head, up to 16 heads of its group, one split of the keys);
 //            the heads of a group share every K/V load and the waves share the split's blocks.
 //            A second kernel merges the splits when there is more than one.
@@ -103,15 +103,16 @@ __device__ __forceinline__ void attn_init(AttnState<QB>& st) {
 }
 
 // ------------------------------------------------------------------ prefill
-// A workgroup of 4 waves takes 128 query rows of one (sequence, head), a wave 32 of them (two column
-// blocks).  Blocks of 64 keys go through LDS, double-buffered: while the waves work on one block the
+// A workgroup of 8 waves takes 128 query rows of one (sequence, head), a wave 16 of them; two waves
+// share a SIMD, so that one multiplies while the other waits for LDS or memory.  Blocks of 64 keys go through LDS, double-buffered: while the waves work on one block the
 // next one is on its way from memory into registers.  K lies in LDS as [64 keys, in tile order][HD + 8], V^T as
 // [HD][64 + 8]; the paddings keep the 16-lane fragment reads free of bank conflicts.
 // Softmax runs in the exp2 domain (scores times scale * log2 e); masking is applied only to blocks
 // that reach beyond a row's causal limit, the window's start or the sequence's end.
 // PV takes k-steps of 32 keys (see the key permutation above).
-constexpr int PF_QB = 2;                        // 16-column blocks a wave
-constexpr int PF_WAVES = 4;
+constexpr float RESCALE_AT = 8.f;
+constexpr int PF_QB = 1;                        // 16-column blocks a wave
+constexpr int PF_WAVES = 8;
 constexpr int PF_THREADS = PF_WAVES * SYN_WAVE;
 constexpr int PF_ROWS = PF_WAVES * PF_QB * 16;  // query rows a workgroup
 constexpr int LDK = HD + 8;
@@ -248,10 +249,20 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages
           }
         mloc = fmaxf(mloc, __shfl_xor(mloc, 16, SYN_WAVE));
         mloc = fmaxf(mloc, __shfl_xor(mloc, 32, SYN_WAVE));
-        const float m_new = fmaxf(st.m[c], mloc);
-        const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a column that has seen no key yet
-        const float alpha = __builtin_amdgcn_exp2f(st.m[c] - m_use);
-        st.m[c] = m_new;
+        // st.m is the reference of the exponents, not the exact maximum: it is only raised when a
+        // block exceeds it by more than RESCALE_AT (in log2 units), so that the accumulators are
+        // rescaled in few blocks.  Probabilities then reach at most 2^RESCALE_AT, well inside
+        // float and bf16 range; the final division by the sum removes the common factor.
+        const bool raise = mloc > st.m[c] + RESCALE_AT || (st.m[c] == -INFINITY && mloc > -INFINITY);
+        if (__any(raise)) {  // same decision for the whole wave: columns that stay get alpha = 1
+          const float m_new = raise ? mloc : st.m[c];
+          const float alpha = raise ? __builtin_amdgcn_exp2f(st.m[c] - m_new) : 1.f;  // from -inf: 0
+          st.m[c] = m_new;
+          st.l[c] *= alpha;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) st.o[dt][c] *= alpha;
+        }
+        const float m_use = st.m[c] == -INFINITY ? 0.f : st.m[c];  // a column that has seen no key yet
         float lsum = 0.f;
 #pragma unroll
         for (int t = 0; t < 4; ++t)
@@ -261,9 +272,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages
             s[t][c][e] = p;
             lsum += p;
           }
-        st.l[c] = st.l[c] * alpha + lsum;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) st.o[dt][c] *= alpha;
+        st.l[c] += lsum;
       }
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt) {
