@@ -4,8 +4,8 @@
 //                  the MFMA kernels refuse (K not a multiple of 8, unaligned rows).
 //   gemm_skinny    bf16, M <= 64: the weight matrix is streamed once from HBM through
 //                  v_mfma_f32_16x16x32_bf16; the waves of a workgroup split K and sum in LDS.
-//   gemm_tiled     bf16, M > 64: 256x128x32 (or smaller) tiles in LDS, double-buffered, 2x2 waves,
-//                  v_mfma_f32_32x32x16_bf16.
+//   gemm_tiled     bf16, M > 64: 256x256x64 tiles with 8 waves (or 128x128x64 with 4) in LDS,
+//                  double-buffered, v_mfma_f32_32x32x16_bf16.
 //
 // Reference counterparts: crates/synaptix-kernels-cuda/src/best_cu/gemm/gemm_bf16.cu (TN family,
 // mma.sync m16n8k16), best_cu/gemv/mma_gemv.cu:19-133 (M == 1), best_cu/gemm/gemm_f32.cu (SIMT).
@@ -168,23 +168,25 @@ static void launch_skinny(const bf16* x, const bf16* w, void* out, int out_is_f3
 }
 
 // ------------------------------------------------------------------ tiled, bf16, large M
-// Block tile BM (m) x BN (n) x 32 (k); 4 waves as 2x2, each (BM/2) x (BN/2) of MFMA 32x32x16 tiles.
+// Block tile BM (m) x BN (n) x BK (k); WM x WN waves, each (BM/WM) x (BN/WN) of MFMA 32x32x16 tiles.
 // MFMA 32x32x16: A = x rows, B = W rows; lane holds row lane%32, k = 8*(lane/32) .. +8;
 // D[m = 8*(j/4) + 4*(lane/32) + j%4][n = lane%32], j = 0..15.
 // LDS tiles are double-buffered: while one k-tile is multiplied the next is on its way from memory
 // into registers, and is stored into the other buffer before the barrier.
-template <int BM, int BN, int BK, bool KTAIL>
-__global__ void __launch_bounds__(256, ((BM + BN) * (BK + 8) * 4 <= 80 * 1024 && BM * BN <= 256 * 128 ? 2 : 1))
+template <int BM, int BN, int BK, int WM, int WN, bool KTAIL>
+__global__ void __launch_bounds__(64 * WM * WN)
 gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
                   int M, int N, int K) {
+  constexpr int THREADS = 64 * WM * WN;              // WM x WN waves
   constexpr int LD = BK + 8;                         // padded row of the LDS tiles, in bf16 elements
-  constexpr int TM = BM / 64, TN = BN / 64;          // 32x32 tiles a wave holds in m and n
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;  // 32x32 tiles a wave holds in m and n
   constexpr int CPR = BK / 8;                        // 16-byte chunks in a tile row
-  constexpr int RPP = 256 / CPR;                     // tile rows the workgroup moves in one pass
+  constexpr int RPP = THREADS / CPR;                 // tile rows the workgroup moves in one pass
   constexpr int XL = BM / RPP, WL = BN / RPP;        // passes for x and for W
+  static_assert(BM % RPP == 0 && BN % RPP == 0 && TM >= 1 && TN >= 1, "tile shape");
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];  // [2][(BM + BN) * LD]
   const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE;
-  const int wm = (wave / 2) * (BM / 2), wn = (wave % 2) * (BN / 2);
+  const int wm = (wave / WN) * (BM / WM), wn = (wave % WN) * (BN / WN);
   // Which tile: workgroup b runs on XCD b % 8, and each XCD has an L2 of its own.  Tiles are grouped
   // into panels of PM x PN (m fastest); a panel goes to one XCD, so the workgroups that run there at
   // the same time share rows of x and of W in its L2.
@@ -276,7 +278,7 @@ gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* 
       }
 }
 
-template <int BM, int BN, int BK>
+template <int BM, int BN, int BK, int WM, int WN>
 static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
                         hipStream_t stream) {
   const int tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM;
@@ -286,18 +288,18 @@ static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32,
   const size_t lds = (size_t)2 * (BM + BN) * (BK + 8) * sizeof(bf16);
   static bool raised = false;
   if (lds > 65536 && !raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, false>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, WM, WN, false>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, true>,
+      e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, WM, WN, true>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     SYN_CHECK(e == hipSuccess, "gemm: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
     raised = true;
   }
   if (K % BK == 0)
-    gemm_tiled_kernel<BM, BN, BK, false><<<grid, 256, lds, stream>>>(x, w, out, out_is_f32, M, N, K);
+    gemm_tiled_kernel<BM, BN, BK, WM, WN, false><<<grid, 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K);
   else
-    gemm_tiled_kernel<BM, BN, BK, true><<<grid, 256, lds, stream>>>(x, w, out, out_is_f32, M, N, K);
+    gemm_tiled_kernel<BM, BN, BK, WM, WN, true><<<grid, 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K);
   return 0;
 }
 
@@ -352,18 +354,18 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
     else if (v == 3) launch_skinny<4, 2, 16, 1>(xb, wb, out, out_is_f32, M, N, K, stream);
     else launch_skinny<4, 4, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
   } else {
-    // tile shapes: 256 x 128 where that leaves no compute unit idle, smaller tiles for small problems
+    // 256 x 256 tiles (8 waves) where they keep at least three quarters of the compute units busy,
+    // 128 x 128 tiles (4 waves) for smaller problems
     const int tv = getenv("SYN_TILED") ? atoi(getenv("SYN_TILED")) : -1;
-    const long t256 = (long)((M + 255) / 256) * ((N + 127) / 128);
-    const int v = tv >= 0 ? tv : 1;
-    (void)t256;
+    const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+    const int v = tv >= 0 ? tv : (t256 >= 192 ? 0 : 1);
     int rc;
-    if (v == 0) rc = launch_tiled<256, 128, 32>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 1) rc = launch_tiled<128, 128, 64>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 2) rc = launch_tiled<128, 128, 32>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 3) rc = launch_tiled<256, 128, 64>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 4) rc = launch_tiled<128, 128, 128>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else rc = launch_tiled<128, 256, 64>(xb, wb, out, out_is_f32, M, N, K, stream);
+    if (v == 0) rc = launch_tiled<256, 256, 64, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 1) rc = launch_tiled<128, 128, 64, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 2) rc = launch_tiled<256, 256, 32, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 3) rc = launch_tiled<256, 128, 64, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (v == 4) rc = launch_tiled<256, 256, 64, 2, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else rc = launch_tiled<128, 256, 64, 2, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
     if (rc) return rc;
   }
   SYN_LAUNCH_CHECK("gemm");
