@@ -36,29 +36,34 @@ SYN_EXPORT int syn_embed(const void* table, int table_is_f32, const int* ids, fl
 // ------------------------------------------------------------------ residual sum + RMSNorm
 // rows == nullptr: for every row r: resid[r] += delta[r] (if delta), out[r] = norm(resid[r]).
 // rows != nullptr: out[i] = norm(resid[rows[i]] + delta[rows[i]]); resid stays as it is.
-// The sum, the mean of squares and the scaling are 32-bit; one rounding at the store.
+// delta may come as n_parts partial sums [n_parts][n_rows][H] (a product cut along K); they are
+// added in order.  The sum, the mean of squares and the scaling are 32-bit; one rounding at the store.
 template <typename TOut>
-__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const float* __restrict__ delta,
-                                   const int* __restrict__ rows, const void* __restrict__ gain, int gain_is_f32,
-                                   float eps, TOut* __restrict__ out, int H) {
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const float* __restrict__ delta, int n_parts,
+                                   size_t part_stride, const int* __restrict__ rows, const void* __restrict__ gain,
+                                   int gain_is_f32, float eps, TOut* __restrict__ out, int H) {
   __shared__ float red[16];
   const int r = rows ? rows[blockIdx.x] : blockIdx.x;
   float* x = resid + (size_t)r * H;
   const float* d = delta ? delta + (size_t)r * H : nullptr;
   TOut* o = out + (size_t)blockIdx.x * H;
   const bool write_back = (rows == nullptr) && (d != nullptr);
+  auto summed = [&](int i) {
+    float v = x[i];
+    if (d)
+      for (int p = 0; p < n_parts; ++p) v += d[p * part_stride + i];
+    return v;
+  };
   float ss = 0.f;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    float v = x[i];
-    if (d) v += d[i];
+    const float v = summed(i);
     if (write_back) x[i] = v;
     ss += v * v;
   }
   ss = block_sum(ss, red);
   const float inv = rsqrtf(ss / (float)H + eps);
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    float v = x[i];
-    if (d && !write_back) v += d[i];
+    const float v = write_back ? x[i] : summed(i);
     o[i] = from_f32<TOut>(load_gain(gain, gain_is_f32, i) * v * inv);
   }
 }
@@ -66,9 +71,10 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const float* __res
 // The same for rows whose width is a multiple of 4 and at most 4 * VPT * blockDim: every thread
 // keeps its values (float4 loads) in registers between the sum of squares and the scaling.
 template <typename TOut, int VPT>
-__global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const float* __restrict__ delta,
-                                       const int* __restrict__ rows, const void* __restrict__ gain, int gain_is_f32,
-                                       float eps, TOut* __restrict__ out, int H) {
+__global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const float* __restrict__ delta, int n_parts,
+                                       size_t part_stride, const int* __restrict__ rows,
+                                       const void* __restrict__ gain, int gain_is_f32, float eps,
+                                       TOut* __restrict__ out, int H) {
   __shared__ float red[16];
   const int r = rows ? rows[blockIdx.x] : blockIdx.x;
   float4* x = (float4*)(resid + (size_t)r * H);
@@ -76,6 +82,7 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const float* _
   TOut* o = out + (size_t)blockIdx.x * H;
   const bool write_back = (rows == nullptr) && (d != nullptr);
   const int H4 = H / 4;
+  const size_t stride4 = part_stride / 4;
   float4 v[VPT];
   float ss = 0.f;
 #pragma unroll
@@ -84,11 +91,13 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const float* _
     if (i < H4) {
       v[j] = x[i];
       if (d) {
-        const float4 t = d[i];
-        v[j].x += t.x;
-        v[j].y += t.y;
-        v[j].z += t.z;
-        v[j].w += t.w;
+        for (int p = 0; p < n_parts; ++p) {
+          const float4 t = d[p * stride4 + i];
+          v[j].x += t.x;
+          v[j].y += t.y;
+          v[j].z += t.z;
+          v[j].w += t.w;
+        }
       }
       if (write_back) x[i] = v[j];
       ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
@@ -107,16 +116,20 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const float* _
   }
 }
 
-SYN_EXPORT int syn_add_rmsnorm(float* resid, const float* delta, const int* rows, int n_out, const void* gain,
-                               int gain_is_f32, float eps, void* out, int out_is_f32, int H, hipStream_t stream) {
-  SYN_CHECK(n_out > 0 && H > 0, "add_rmsnorm: empty input (%d rows, width %d)", n_out, H);
+SYN_EXPORT int syn_add_rmsnorm(float* resid, const float* delta, int n_parts, int n_rows, const int* rows, int n_out,
+                               const void* gain, int gain_is_f32, float eps, void* out, int out_is_f32, int H,
+                               hipStream_t stream) {
+  SYN_CHECK(n_out > 0 && H > 0 && n_rows > 0, "add_rmsnorm: empty input (%d rows, width %d)", n_out, H);
+  SYN_CHECK(n_parts >= 1 && n_parts <= 64, "add_rmsnorm: %d partial sums", n_parts);
+  const size_t stride = (size_t)n_rows * H;
   const bool vec = H % 4 == 0 && H <= 4 * 4 * 512 && ((uintptr_t)resid % 16 == 0) && ((uintptr_t)delta % 16 == 0);
   if (vec) {
     const int H4 = H / 4;
     const int block = H4 <= 256 ? 256 : 512;
     const int vpt = (H4 + block - 1) / block;  // 1 .. 4
-#define SYN_ARN(T, V)                                                                                         \
-  add_rmsnorm_vec_kernel<T, V><<<n_out, block, 0, stream>>>(resid, delta, rows, gain, gain_is_f32, eps, (T*)out, H)
+#define SYN_ARN(T, V)                                                                                          \
+  add_rmsnorm_vec_kernel<T, V><<<n_out, block, 0, stream>>>(resid, delta, n_parts, stride, rows, gain, gain_is_f32, \
+                                                            eps, (T*)out, H)
     if (out_is_f32) {
       if (vpt == 1) SYN_ARN(float, 1); else if (vpt == 2) SYN_ARN(float, 2); else SYN_ARN(float, 4);
     } else {
@@ -126,9 +139,11 @@ SYN_EXPORT int syn_add_rmsnorm(float* resid, const float* delta, const int* rows
   } else {
     const int block = H >= 4096 ? 1024 : (H >= 1024 ? 512 : 256);
     if (out_is_f32)
-      add_rmsnorm_kernel<float><<<n_out, block, 0, stream>>>(resid, delta, rows, gain, gain_is_f32, eps, (float*)out, H);
+      add_rmsnorm_kernel<float><<<n_out, block, 0, stream>>>(resid, delta, n_parts, stride, rows, gain, gain_is_f32,
+                                                            eps, (float*)out, H);
     else
-      add_rmsnorm_kernel<bf16><<<n_out, block, 0, stream>>>(resid, delta, rows, gain, gain_is_f32, eps, (bf16*)out, H);
+      add_rmsnorm_kernel<bf16><<<n_out, block, 0, stream>>>(resid, delta, n_parts, stride, rows, gain, gain_is_f32,
+                                                           eps, (bf16*)out, H);
   }
   SYN_LAUNCH_CHECK("add_rmsnorm");
   return 0;

@@ -67,7 +67,9 @@ gemm_simt_kernel(const TIn* __restrict__ x, const TIn* __restrict__ w, TOut* __r
 template <int MB, int RT, int WAVES, int U>
 __global__ void __launch_bounds__(WAVES * SYN_WAVE)
 gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
-                   int M, int N, int K) {
+                   int M, int N, int K, int k_slice) {
+  // blockIdx.y = which slice of K this workgroup sums (k_slice elements, a multiple of 32); with
+  // more than one slice the output is float [slices, M, N] and whoever reads it adds the slices
   extern __shared__ float part[];  // [WAVES][MB*RT*4][64]
   const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
   const int r16 = lane % 16, kq = (lane / 16) * 8;
@@ -95,8 +97,9 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
   // U chunks of 32 at a time: all loads of a group are issued before the first product needs them,
   // so that a wave keeps U * RT KiB of the weight stream in flight
   constexpr int GROUP = 32 * U;
-  const int k_full = K / (WAVES * GROUP) * (WAVES * GROUP);
-  for (int k0 = wave * GROUP; k0 < k_full; k0 += WAVES * GROUP) {
+  const int k_begin = (int)blockIdx.y * k_slice, k_end = min(K, k_begin + k_slice);
+  const int k_full = k_begin + (k_end - k_begin) / (WAVES * GROUP) * (WAVES * GROUP);
+  for (int k0 = k_begin + wave * GROUP; k0 < k_full; k0 += WAVES * GROUP) {
     bf16x8 bw[U][RT], ax[U][MB];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -115,8 +118,8 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
   }
   // what is left of K, chunk by chunk; K is a multiple of 8, so a lane's 8 elements lie inside or
   // outside as a whole
-  for (int k0 = k_full + wave * 32; k0 < K; k0 += WAVES * 32) {
-    const bool kin = k0 + kq < K;
+  for (int k0 = k_full + wave * 32; k0 < k_end; k0 += WAVES * 32) {
+    const bool kin = k0 + kq < k_end;
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
       const bf16x8 ax = (kin && xok[b]) ? *(const bf16x8*)(xrow[b] + k0) : zero;
@@ -146,7 +149,7 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
     const int m = b * 16 + 4 * (ln / 16) + j, n = n0 + r * 16 + ln % 16;
     if (m < M && n < N) {
       if (out_is_f32)
-        ((float*)out)[(size_t)m * N + n] = s;
+        ((float*)out)[((size_t)blockIdx.y * M + m) * N + n] = s;
       else
         ((bf16*)out)[(size_t)m * N + n] = (bf16)s;
     }
@@ -155,8 +158,9 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
 
 template <int MB, int RT, int WAVES, int U>
 static void launch_skinny(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
-                          hipStream_t stream) {
-  const int grid = (N + RT * 16 - 1) / (RT * 16);
+                          int slices, hipStream_t stream) {
+  const int k_slice = ((K + slices - 1) / slices + 31) / 32 * 32;
+  const dim3 grid((N + RT * 16 - 1) / (RT * 16), slices);
   const size_t lds = (size_t)WAVES * MB * RT * 4 * 64 * sizeof(float);
   static bool raised = false;
   if (lds > 65536 && !raised) {
@@ -164,7 +168,7 @@ static void launch_skinny(const bf16* x, const bf16* w, void* out, int out_is_f3
                         (int)lds);
     raised = true;
   }
-  gemm_skinny_kernel<MB, RT, WAVES, U><<<grid, WAVES * SYN_WAVE, lds, stream>>>(x, w, out, out_is_f32, M, N, K);
+  gemm_skinny_kernel<MB, RT, WAVES, U><<<grid, WAVES * SYN_WAVE, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
 }
 
 // ------------------------------------------------------------------ tiled, bf16, large M
@@ -305,10 +309,14 @@ static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32,
 
 // ------------------------------------------------------------------ entry point
 // dtype: 0 = float in, float out; 1 = bf16 in, bf16 out; 2 = bf16 in, float out.
+// slices > 1 (bf16 in, float out, M <= 64 only): out is [slices, M, N], slice s holds the sum over its
+// part of K; the reader adds the slices.
 SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int M, int N, int K, int force_simt,
-                        hipStream_t stream) {
+                        int slices, hipStream_t stream) {
   SYN_CHECK(M > 0 && N > 0 && K > 0, "gemm: empty shape M=%d N=%d K=%d", M, N, K);
   SYN_CHECK(dtype >= 0 && dtype <= 2, "gemm: unknown dtype code %d", dtype);
+  SYN_CHECK(slices >= 1 && (slices == 1 || (dtype == 2 && M <= 64 && !force_simt && K % 8 == 0 && slices <= 64)),
+            "gemm: %d slices of K need bf16 operands, a float output and M <= 64 (M = %d)", slices, M);
   const dim3 simt_grid((N + SIMT_BN - 1) / SIMT_BN, (M + SIMT_BM - 1) / SIMT_BM);
   if (dtype == 0) {
     gemm_simt_kernel<float, float><<<simt_grid, 256, 0, stream>>>((const float*)x, (const float*)w, (float*)out, M, N, K);
@@ -317,6 +325,7 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   }
   const int out_is_f32 = dtype == 2;
   const bool aligned = (K % 8 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
+  SYN_CHECK(slices == 1 || aligned, "gemm: slices of K need 16-byte aligned operands");
   if (force_simt || !aligned) {
     if (out_is_f32)
       gemm_simt_kernel<bf16, float><<<simt_grid, 256, 0, stream>>>((const bf16*)x, (const bf16*)w, (float*)out, M, N, K);
@@ -330,29 +339,29 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   // rows of W a workgroup owns: more rows amortise the loads of x, fewer rows give more workgroups
   const int variant = getenv("SYN_SKINNY") ? atoi(getenv("SYN_SKINNY")) : -1;
   if (M <= 16) {
-    const int v = variant >= 0 ? variant : (N <= 8192 ? 0 : 1);
-    if (v == 0) launch_skinny<1, 1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 1) launch_skinny<1, 1, 8, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 2) launch_skinny<1, 2, 8, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 3) launch_skinny<1, 4, 8, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 4) launch_skinny<1, 2, 16, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else launch_skinny<1, 4, 8, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
+    const int v = variant >= 0 ? variant : ((N <= 8192 && slices == 1) ? 0 : 1);
+    if (v == 0) launch_skinny<1, 1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else if (v == 1) launch_skinny<1, 1, 8, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else if (v == 2) launch_skinny<1, 2, 8, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else if (v == 3) launch_skinny<1, 4, 8, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else if (v == 4) launch_skinny<1, 2, 16, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else launch_skinny<1, 4, 8, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
   } else if (M <= 32) {
     const int v = variant >= 0 ? variant : (N <= 4096 ? 0 : (N <= 8192 ? 1 : 2));
-    if (v == 0) launch_skinny<2, 1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 1) launch_skinny<2, 2, 8, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 2) launch_skinny<2, 4, 8, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 3) launch_skinny<2, 2, 16, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else launch_skinny<2, 4, 4, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
+    if (v == 0) launch_skinny<2, 1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else if (v == 1) launch_skinny<2, 2, 8, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else if (v == 2) launch_skinny<2, 4, 8, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else if (v == 3) launch_skinny<2, 2, 16, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else launch_skinny<2, 4, 4, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
   } else if (M <= 48) {
-    launch_skinny<3, 2, 8, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
+    launch_skinny<3, 2, 8, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
   } else if (M <= 64) {
     const int v = variant >= 0 ? variant : (N <= 4096 ? 0 : (N <= 8192 ? 3 : 4));
-    if (v == 0) launch_skinny<4, 1, 16, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 1) launch_skinny<4, 2, 8, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 2) launch_skinny<4, 4, 8, 1>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 3) launch_skinny<4, 2, 16, 1>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else launch_skinny<4, 4, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
+    if (v == 0) launch_skinny<4, 1, 16, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else if (v == 1) launch_skinny<4, 2, 8, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else if (v == 2) launch_skinny<4, 4, 8, 1>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else if (v == 3) launch_skinny<4, 2, 16, 1>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else launch_skinny<4, 4, 4, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
   } else {
     // 256 x 256 tiles (8 waves) where they keep at least three quarters of the compute units busy,
     // 128 x 128 tiles (4 waves) for smaller problems

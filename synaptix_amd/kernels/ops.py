@@ -69,18 +69,24 @@ def embed(table, ids, resid):
 
 def add_rmsnorm(resid, delta, gain, eps, out, rows=None):
     """rows is None:  resid += delta (when given), out = RMSNorm(resid) * gain, for every row.
-    rows [n] int32: out[i] = RMSNorm(resid[rows[i]] + delta[rows[i]]) * gain; resid is not written."""
+    rows [n] int32: out[i] = RMSNorm(resid[rows[i]] + delta[rows[i]]) * gain; resid is not written.
+    delta may be [S, N, H]: partial sums that are added up on the way."""
     _need(resid, "add_rmsnorm.resid", _F32, (None, None))
     N, H = resid.shape
+    n_parts = 1
     if delta is not None:
-        _need(delta, "add_rmsnorm.delta", _F32, (N, H))
+        if delta.dim() == 3:
+            n_parts = delta.shape[0]
+            _need(delta, "add_rmsnorm.delta", _F32, (n_parts, N, H))
+        else:
+            _need(delta, "add_rmsnorm.delta", _F32, (N, H))
     _need(gain, "add_rmsnorm.gain", (_BF16, _F32), (H,))
     n_out = N
     if rows is not None:
         _need(rows, "add_rmsnorm.rows", _I32, (None,))
         n_out = rows.shape[0]
     _need(out, "add_rmsnorm.out", (_BF16, _F32), (n_out, H))
-    _call(load_library("core"), "syn_add_rmsnorm", _ptr(resid), _ptr(delta), _ptr(rows), n_out, _ptr(gain),
+    _call(load_library("core"), "syn_add_rmsnorm", _ptr(resid), _ptr(delta), n_parts, N, _ptr(rows), n_out, _ptr(gain),
           _is_f32(gain), ctypes.c_float(eps), _ptr(out), _is_f32(out), H, _stream())
 
 
@@ -108,19 +114,37 @@ def swiglu(gate_up, out):
 
 def gemm(x, w, out, force_simt=False):
     """out[M, N] = x[M, K] . w[N, K]^T with 32-bit accumulation.
-    float x float -> float (plain FMA); bf16 x bf16 -> bf16 or float (MFMA)."""
+    float x float -> float (plain FMA); bf16 x bf16 -> bf16 or float (MFMA).
+    A float out of shape [S, M, N] (bf16 operands, M <= 64) receives S partial sums over slices
+    of K instead; their sum over S is the product."""
     _need(x, "gemm.x", (_BF16, _F32), (None, None))
     M, K = x.shape
     _need(w, "gemm.w", x.dtype, (None, K))
     N = w.shape[0]
-    if x.dtype == _F32:
+    slices = 1
+    if out.dim() == 3:
+        slices = out.shape[0]
+        if x.dtype != _BF16 or M > 64 or force_simt:
+            raise KernelError("gemm: partial sums over slices of K need bf16 operands and M <= 64")
+        _need(out, "gemm.out", _F32, (slices, M, N))
+        code = 2
+    elif x.dtype == _F32:
         _need(out, "gemm.out", _F32, (M, N))
         code = 0
     else:
         _need(out, "gemm.out", (_BF16, _F32), (M, N))
         code = 2 if out.dtype == _F32 else 1
     _call(load_library("core"), "syn_gemm", _ptr(x), _ptr(w), _ptr(out), code, M, N, K, 1 if force_simt else 0,
-          _stream())
+          slices, _stream())
+
+
+def gemm_slices(M, N, K, dtype):
+    """Into how many slices of K a product whose output feeds a sum is cut.  Measured at M = 1 and 8:
+    a product with few rows of W and a long K (4096 x 12288) gains 7 % from two slices; shorter ones
+    gain nothing (their time is launch and first-byte latency, not the number of workgroups)."""
+    if dtype != _BF16 or M > 16 or K % 8 != 0 or N > 8192 or K < 8192:
+        return 1
+    return 2
 
 
 # ----------------------------------------------------------------------------- attention

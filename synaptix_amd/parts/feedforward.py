@@ -10,7 +10,7 @@ import torch
 from ..kernels import ops
 from ..weights.source import TensorSpec
 from .base import Part
-from .linear import linear
+from .linear import linear, linear_for_sum
 
 
 class FeedForward(Part):
@@ -44,4 +44,4 @@ class GatedMlp(FeedForward):
         gu = linear(h, self.w_gate_up, h.dtype)
         m = torch.empty((h.shape[0], self.intermediate), dtype=h.dtype, device=h.device)
         ops.swiglu(gu, m)
-        return linear(m, self.w_down, torch.float32)
+        return linear_for_sum(m, self.w_down)

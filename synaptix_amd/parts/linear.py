@@ -21,3 +21,17 @@ def linear(x, w, out_dtype):
                       device=x.device)
     ops.gemm(x, w, out)
     return out if out.dtype == out_dtype else out.to(out_dtype)
+
+
+def linear_for_sum(x, w):
+    """The product as float partial sums for a consumer that adds them up (the residual sum fused
+    into the next norm): [S, M, N] when cutting K into S slices gives a small product more
+    workgroups, else [M, N]."""
+    M, K = x.shape
+    N = w.shape[0]
+    slices = ops.gemm_slices(M, N, K, x.dtype) if w.dtype == x.dtype else 1
+    if slices <= 1:
+        return linear(x, w, torch.float32)
+    out = torch.empty((slices, M, N), dtype=torch.float32, device=x.device)
+    ops.gemm(x, w, out)
+    return out

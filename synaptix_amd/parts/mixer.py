@@ -15,7 +15,7 @@ import torch
 from ..kernels import ops
 from ..weights.source import TensorSpec
 from .base import Part, KvNeed
-from .linear import linear
+from .linear import linear, linear_for_sum
 from .position import Position, NoPosition
 
 
@@ -25,7 +25,8 @@ class Mixer(Part):
     cache_need(): KvNeed, StateNeed or None: what it keeps for each sequence.
     forward(h, ctx, cache, owner): h [N, hidden] in the activation type, ctx the step's
     StepContext, cache the view of its cache layer (None without a need); owner is False when the
-    layer reads a cache that another layer writes.  Returns the residual delta [N, hidden] float.
+    layer reads a cache that another layer writes.  Returns the residual delta as float [N, hidden],
+    or as partial sums [S, N, hidden] that the following norm adds up.
     """
 
     def cache_need(self):
@@ -100,4 +101,4 @@ class GqaAttention(Mixer):
         else:
             ops.attention_prefill_bf16(q, cache.k_pages, cache.v_pages, table, ctx.seq_start, ctx.seq_past, o,
                                        self.scale, window, nh, nkv, hd)
-        return linear(o, self.w_o, torch.float32)
+        return linear_for_sum(o, self.w_o)

@@ -24,6 +24,8 @@ def embed(table, ids, resid):
 
 
 def add_rmsnorm(resid, delta, gain, eps, out, rows=None):
+    if delta is not None and delta.dim() == 3:
+        delta = delta.sum(0)
     if rows is None:
         if delta is not None:
             resid.add_(delta)
@@ -49,7 +51,17 @@ def swiglu(gate_up, out):
 
 
 def gemm(x, w, out, force_simt=False):
+    if out.dim() == 3:                      # partial sums over slices of K
+        S, K = out.shape[0], x.shape[1]
+        step = ((K + S - 1) // S + 31) // 32 * 32
+        for s in range(S):
+            out[s] = x[:, s * step:(s + 1) * step].to(F32) @ w[:, s * step:(s + 1) * step].to(F32).T
+        return
     out.copy_((x.to(F32) @ w.to(F32).T).to(out.dtype))
+
+
+def gemm_slices(M, N, K, dtype):
+    return 2 if (dtype == torch.bfloat16 and M <= 16 and K >= 64 and K % 8 == 0) else 1
 
 
 def qk_norm_rope_kv_write(qkv, q_out, k_pages, v_pages, page_table, tok_seq, tok_pos, q_gain, k_gain, eps,
@@ -148,7 +160,7 @@ def sample_rows(logits, temperature, uniform, out):
         out[r] = int(hit[0]) if hit.numel() else x.numel() - 1
 
 
-ALL = ["embed", "add_rmsnorm", "rmsnorm_rows", "swiglu", "gemm", "qk_norm_rope_kv_write", "attention_f32",
+ALL = ["embed", "add_rmsnorm", "rmsnorm_rows", "swiglu", "gemm", "gemm_slices", "qk_norm_rope_kv_write", "attention_f32",
        "attention_prefill_bf16", "decode_splits", "attention_decode_bf16", "sample_rows"]
 
 

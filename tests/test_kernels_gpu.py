@@ -151,6 +151,39 @@ def test_gemm_bf16(ops, out_dtype, M, N, K):
     close(out, want, atol if out_dtype == F32 else atol + 0.02, 0 if out_dtype == F32 else 1e-2, f"gemm bf16 {M}x{N}x{K}")
 
 
+@pytest.mark.parametrize("M,N,K,S", [(1, 48, 4096, 4), (8, 4096, 4096, 4), (8, 100, 1000, 3), (16, 64, 12288, 8),
+                                     (40, 70, 2048, 2), (64, 130, 520, 5)])
+def test_gemm_bf16_partial_sums_over_slices_of_k(ops, M, N, K, S):
+    """[S, M, N]: slice s holds the sum over its part of K; the slices add up to the product, also
+    when K is no multiple of the slice and the last slices are short or empty."""
+    x, w = rnd((M, K), 14, BF16), rnd((N, K), 15, BF16)
+    out = torch.full((S, M, N), float("nan"), dtype=F32, device=DEV)
+    ops.gemm(x.to(DEV), w.to(DEV), out)
+    want = (x.double() @ w.double().T).float()
+    close(out.sum(0), want, 1e-3 * math.sqrt(K), what=f"sum of {S} slices")
+    step = ((K + S - 1) // S + 31) // 32 * 32
+    first = (x[:, :step].double() @ w[:, :step].double().T).float()
+    close(out[0], first, 1e-3 * math.sqrt(step), what="first slice")
+    # the consumer adds the slices: resid + sum(delta) normed
+    H = N
+    resid = rnd((M, H), 16)
+    gain = (1 + 0.1 * rnd((H,), 17)).to(BF16)
+    r = resid.to(DEV)
+    normed = torch.empty((M, H), dtype=BF16, device=DEV)
+    ops.add_rmsnorm(r, out, gain.to(DEV), 1e-6, normed)
+    want_resid = resid + out.sum(0).cpu()
+    close(r, want_resid, 1e-4, 1e-5, "residual + slices")
+    want_n = torch.empty((M, H), dtype=BF16)
+    ref.add_rmsnorm(want_resid.clone(), None, gain, 1e-6, want_n)
+    close(normed, want_n, 2e-2, 1e-2, "norm of residual + slices")
+    rows = torch.tensor([M - 1, 0], dtype=I32)
+    got2 = torch.empty((2, H), dtype=F32, device=DEV)
+    ops.add_rmsnorm(resid.to(DEV), out, gain.to(DEV), 1e-6, got2, rows.to(DEV))
+    want2 = torch.empty((2, H), dtype=F32)
+    ref.add_rmsnorm(resid.clone(), out.cpu(), gain, 1e-6, want2, rows)
+    close(got2, want2, 1e-4, 1e-4, "gathered rows of residual + slices")
+
+
 def test_gemm_bf16_paths_agree(ops):
     """The MFMA kernels and the plain kernel compute the same sums."""
     for M in (4, 40, 300):

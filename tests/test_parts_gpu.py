@@ -116,14 +116,25 @@ def test_attention_part_alone(dtype, nh, nkv, hd, rot, qk_norm, window):
     assert err <= (2e-4 if dtype == F32 else 4e-2) * max(1.0, float(want.abs().max())), float(err)
 
 
-@pytest.mark.parametrize("dtype", [F32, BF16])
-def test_gated_mlp_part_alone(dtype):
-    from synaptix_amd.parts import GatedMlp
-    ff = GatedMlp("m.", 56, 200)
+@pytest.mark.parametrize("dtype,inter", [(F32, 200), (BF16, 200), (BF16, 2048)])
+def test_gated_mlp_part_alone(dtype, inter):
+    """With 2048 intermediate values and few rows the last product comes as partial sums over
+    slices of K, which the norm that follows adds up."""
+    from synaptix_amd.parts import GatedMlp, RmsNorm
+    ff = GatedMlp("m.", 56, inter)
     w = {n: rnd(s.shape, 40 + i, 0.2).to(dtype) for i, (n, s) in enumerate(ff.tensor_specs().items())}
     ff.load(lambda name: w[name].to(DEV))
     x = rnd((9, 56), 50).to(dtype)
-    got = ff.forward(x.to(DEV), None).cpu()
+    got = ff.forward(x.to(DEV), None)
+    if inter >= 2048 and dtype == BF16:
+        assert got.dim() == 3 and got.shape[0] > 1
+    if got.dim() == 3:
+        norm = RmsNorm("g", 56, 1e-6)
+        norm.load(lambda name: torch.ones(56, device=DEV))
+        resid = torch.zeros((9, 56), device=DEV)
+        norm.add_apply(resid, got, torch.float32)           # resid = 0 + sum of the slices
+        got = resid
+    got = got.cpu()
     want = P.swiglu_mlp(x.float(), w["m.gate_proj.weight"].float(), w["m.up_proj.weight"].float(),
                         w["m.down_proj.weight"].float())
     # bf16: the activations silu(g) * u are rounded once (2^-9 relative) before the last product
