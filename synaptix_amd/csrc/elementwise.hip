@@ -248,8 +248,10 @@ SYN_EXPORT int syn_swiglu(const void* gu, void* out, int is_f32, int n_rows, int
 //   d < rot/2:        o[d] = x[d] cos[p, d]         - x[d + rot/2] sin[p, d]
 //   rot/2 <= d < rot: o[d] = x[d] cos[p, d - rot/2] + x[d - rot/2] sin[p, d - rot/2]
 // All arithmetic is 32-bit; each value is rounded once when stored.
-template <typename T>
-__global__ void qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_pages,
+// TIn = T, or float with n_parts >= 1 partial sums [n_parts][tokens][heads * hd] that are added first.
+template <typename T, typename TIn>
+__global__ void qk_norm_rope_kv_write_kernel(const TIn* __restrict__ qkv, int n_parts, size_t part_stride,
+                                             T* __restrict__ q_out, T* __restrict__ k_pages,
                                              T* __restrict__ v_pages, const int* __restrict__ page_table,
                                              int table_stride, const int* __restrict__ tok_seq,
                                              const int* __restrict__ tok_pos, const void* __restrict__ q_gain,
@@ -270,10 +272,14 @@ __global__ void qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, T* __res
   const void* gain = is_q ? q_gain : (is_k ? k_gain : nullptr);
 
   if (active) {
-    const T* src = qkv + ((size_t)tok * heads + head) * hd;
+    const TIn* src = qkv + ((size_t)tok * heads + head) * hd;
     float ss = 0.f;
     for (int d = 2 * lane; d < hd; d += 2 * SYN_WAVE) {  // head sizes are even: two values a lane
-      const float v0 = to_f32<T>(src[d]), v1 = to_f32<T>(src[d + 1]);
+      float v0 = to_f32<TIn>(src[d]), v1 = to_f32<TIn>(src[d + 1]);
+      for (int p = 1; p < n_parts; ++p) {
+        v0 += to_f32<TIn>(src[p * part_stride + d]);
+        v1 += to_f32<TIn>(src[p * part_stride + d + 1]);
+      }
       xs[d] = v0;
       xs[d + 1] = v1;
       ss += v0 * v0 + v1 * v1;
@@ -326,8 +332,8 @@ __global__ void qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, T* __res
   }
 }
 
-SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, void* q_out, void* k_pages, void* v_pages, int is_f32,
-                                         const int* page_table, int table_stride, const int* tok_seq,
+SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, int n_parts, void* q_out, void* k_pages, void* v_pages,
+                                         int is_f32, const int* page_table, int table_stride, const int* tok_seq,
                                          const int* tok_pos, const void* q_gain, const void* k_gain, int gain_is_f32,
                                          float eps, const float* cos_t, const float* sin_t, int rot, int n_tokens,
                                          int nh, int nkv, int hd, int write_kv, hipStream_t stream) {
@@ -336,18 +342,23 @@ SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, void* q_out, void* k_p
             rot, hd);
   SYN_CHECK(hd % 2 == 0, "qk_norm_rope_kv_write: head size %d is odd", hd);
   SYN_CHECK((cos_t == nullptr) == (sin_t == nullptr), "qk_norm_rope_kv_write: cos and sin come together");
+  SYN_CHECK(n_parts >= 0 && n_parts <= 64, "qk_norm_rope_kv_write: %d partial sums", n_parts);
   const int wpb = 4;
   const int heads = nh + 2 * nkv;
   dim3 grid(n_tokens, (heads + wpb - 1) / wpb);
   const size_t lds = (size_t)wpb * hd * sizeof(float);
+  const size_t stride = (size_t)n_tokens * heads * hd;
+#define SYN_QK(T, TIn)                                                                                             \
+  qk_norm_rope_kv_write_kernel<T, TIn><<<grid, wpb * SYN_WAVE, lds, stream>>>(                                     \
+      (const TIn*)qkv, n_parts > 0 ? n_parts : 1, stride, (T*)q_out, (T*)k_pages, (T*)v_pages, page_table,          \
+      table_stride, tok_seq, tok_pos, q_gain, k_gain, gain_is_f32, eps, cos_t, sin_t, rot, nh, nkv, hd, write_kv)
   if (is_f32)
-    qk_norm_rope_kv_write_kernel<float><<<grid, wpb * SYN_WAVE, lds, stream>>>(
-        (const float*)qkv, (float*)q_out, (float*)k_pages, (float*)v_pages, page_table, table_stride, tok_seq,
-        tok_pos, q_gain, k_gain, gain_is_f32, eps, cos_t, sin_t, rot, nh, nkv, hd, write_kv);
+    SYN_QK(float, float);
+  else if (n_parts > 0)
+    SYN_QK(bf16, float);
   else
-    qk_norm_rope_kv_write_kernel<bf16><<<grid, wpb * SYN_WAVE, lds, stream>>>(
-        (const bf16*)qkv, (bf16*)q_out, (bf16*)k_pages, (bf16*)v_pages, page_table, table_stride, tok_seq, tok_pos,
-        q_gain, k_gain, gain_is_f32, eps, cos_t, sin_t, rot, nh, nkv, hd, write_kv);
+    SYN_QK(bf16, bf16);
+#undef SYN_QK
   SYN_LAUNCH_CHECK("qk_norm_rope_kv_write");
   return 0;
 }

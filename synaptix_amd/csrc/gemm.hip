@@ -4,6 +4,8 @@
 //                  the MFMA kernels refuse (K not a multiple of 8, unaligned rows).
 //   gemm_skinny    bf16, M <= 64: the weight matrix is streamed once from HBM through
 //                  v_mfma_f32_16x16x32_bf16; the waves of a workgroup split K and sum in LDS.
+//   gemm_xlds      bf16, M <= 64: the waves of a workgroup own different rows of W and share the rows
+//                  of x through LDS; K may be cut into slices whose partial sums the reader adds.
 //   gemm_tiled     bf16, M > 64: 256x256x64 tiles with 8 waves (or 128x128x64 with 4) in LDS,
 //                  double-buffered, v_mfma_f32_32x32x16_bf16.
 //
@@ -171,6 +173,118 @@ static void launch_skinny(const bf16* x, const bf16* w, void* out, int out_is_f3
   gemm_skinny_kernel<MB, RT, WAVES, U><<<grid, WAVES * SYN_WAVE, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
 }
 
+// ------------------------------------------------------------------ skinny with x in LDS, bf16, M <= 64
+// The waves of a workgroup own different rows of W (16 * RT each) and run over the same K range; the
+// rows of x for a k-tile go through LDS once and serve all waves, so x costs M / (16 * RT * WAVES)
+// of the weight traffic instead of M / (16 * RT).  W fragments come straight from memory (each is
+// used by one wave only), two k-tiles ahead.  blockIdx.y cuts K into slices as in gemm_skinny.
+template <int MB, int RT, int WAVES, int BK>
+__global__ void __launch_bounds__(WAVES * SYN_WAVE)
+gemm_xlds_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
+                 int M, int N, int K, int k_slice) {
+  constexpr int LD = BK + 8;
+  constexpr int KS = BK / 32;                              // k-steps of 32 in a k-tile
+  constexpr int XCH = MB * 16 * (BK / 8);                  // 16-byte chunks of an x tile
+  constexpr int XL = (XCH + WAVES * 64 - 1) / (WAVES * 64);  // chunks a thread moves
+  __shared__ __attribute__((aligned(16))) bf16 xs[2][MB * 16 * LD];
+  const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE;
+  const int r16 = lane % 16, kq = (lane / 16) * 8;
+  const int n0 = (blockIdx.x * WAVES + wave) * (RT * 16);
+  const int k_begin = (int)blockIdx.y * k_slice, k_end = min(K, k_begin + k_slice);
+  const int nk = (k_end - k_begin + BK - 1) / BK;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  const bf16* wrow[RT];
+#pragma unroll
+  for (int r = 0; r < RT; ++r) wrow[r] = w + (size_t)min(n0 + r * 16 + r16, N - 1) * K + kq;
+
+  bf16x8 rx[XL];
+  auto fetch_x = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < XL; ++i) {
+      const int c = tid + i * WAVES * 64;
+      const int row = c / (BK / 8), k = k_begin + kt * BK + (c % (BK / 8)) * 8;
+      rx[i] = (c < XCH && row < M && k < k_end) ? *(const bf16x8*)(x + (size_t)row * K + k) : zero;
+    }
+  };
+  auto stash_x = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < XL; ++i) {
+      const int c = tid + i * WAVES * 64;
+      if (c < XCH) *(bf16x8*)(&xs[buf][(c / (BK / 8)) * LD + (c % (BK / 8)) * 8]) = rx[i];
+    }
+  };
+  bf16x8 bw0[KS][RT], bw1[KS][RT];  // W fragments of even and of odd k-tiles (indices known at compile time)
+  auto fetch_w = [&](int kt, bf16x8 (&bw)[KS][RT]) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int k = k_begin + kt * BK + ks * 32;
+#pragma unroll
+      for (int r = 0; r < RT; ++r)
+        bw[ks][r] = (k + kq < k_end) ? __builtin_nontemporal_load((const bf16x8*)(wrow[r] + k)) : zero;
+    }
+  };
+
+  f32x4 acc[MB][RT];
+#pragma unroll
+  for (int b = 0; b < MB; ++b)
+#pragma unroll
+    for (int r = 0; r < RT; ++r) acc[b][r] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  // one k-tile: x fragments from LDS buffer `buf`, W fragments from `bw`, which is refilled for the
+  // tile after next as soon as it is used up
+  auto tile = [&](int kt, int buf, bf16x8 (&bw)[KS][RT]) {
+    if (kt + 1 < nk) fetch_x(kt + 1);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      bf16x8 ax[MB];
+#pragma unroll
+      for (int b = 0; b < MB; ++b) ax[b] = *(const bf16x8*)(&xs[buf][(b * 16 + r16) * LD + ks * 32 + kq]);
+#pragma unroll
+      for (int b = 0; b < MB; ++b)
+#pragma unroll
+        for (int r = 0; r < RT; ++r)
+          acc[b][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[b], bw[ks][r], acc[b][r], 0, 0, 0);
+    }
+    if (kt + 2 < nk) fetch_w(kt + 2, bw);
+    if (kt + 1 < nk) stash_x(buf ^ 1);  // the other buffer was last read before the previous barrier
+    __syncthreads();
+  };
+
+  fetch_x(0);
+  fetch_w(0, bw0);
+  stash_x(0);
+  if (nk > 1) fetch_w(1, bw1);
+  __syncthreads();
+  for (int kt = 0; kt < nk; kt += 2) {
+    tile(kt, 0, bw0);
+    if (kt + 1 < nk) tile(kt + 1, 1, bw1);
+  }
+#pragma unroll
+  for (int b = 0; b < MB; ++b)
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int m = b * 16 + 4 * (lane / 16) + j, n = n0 + r * 16 + lane % 16;
+        if (m < M && n < N) {
+          if (out_is_f32)
+            ((float*)out)[((size_t)blockIdx.y * M + m) * N + n] = acc[b][r][j];
+          else
+            ((bf16*)out)[(size_t)m * N + n] = (bf16)acc[b][r][j];
+        }
+      }
+}
+
+template <int MB, int RT, int WAVES, int BK>
+static void launch_xlds(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K, int slices,
+                        hipStream_t stream) {
+  const int k_slice = ((K + slices - 1) / slices + 31) / 32 * 32;
+  const int rows = WAVES * RT * 16;
+  gemm_xlds_kernel<MB, RT, WAVES, BK><<<dim3((N + rows - 1) / rows, slices), WAVES * SYN_WAVE, 0, stream>>>(
+      x, w, out, out_is_f32, M, N, K, k_slice);
+}
+
 // ------------------------------------------------------------------ tiled, bf16, large M
 // Block tile BM (m) x BN (n) x BK (k); WM x WN waves, each (BM/WM) x (BN/WN) of MFMA 32x32x16 tiles.
 // MFMA 32x32x16: A = x rows, B = W rows; lane holds row lane%32, k = 8*(lane/32) .. +8;
@@ -336,6 +450,17 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   }
   const bf16* xb = (const bf16*)x;
   const bf16* wb = (const bf16*)w;
+  // x through LDS (waves on different rows of W) for the widest products and for every product
+  // that is cut along K; measured against gemm_skinny at M = 8, 16 and 64 for the shapes of an 8B model
+  if (M <= 64 && (slices > 1 || N > 32768)) {
+    const int mb = (M + 15) / 16;
+    if (mb == 1) launch_xlds<1, 1, 4, 128>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else if (mb == 2) launch_xlds<2, 1, 4, 128>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else if (mb == 3) launch_xlds<3, 1, 4, 128>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else launch_xlds<4, 1, 4, 128>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    SYN_LAUNCH_CHECK("gemm_xlds");
+    return 0;
+  }
   // rows of W a workgroup owns: more rows amortise the loads of x, fewer rows give more workgroups
   const int variant = getenv("SYN_SKINNY") ? atoi(getenv("SYN_SKINNY")) : -1;
   if (M <= 16) {

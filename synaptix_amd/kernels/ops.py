@@ -139,12 +139,13 @@ def gemm(x, w, out, force_simt=False):
 
 
 def gemm_slices(M, N, K, dtype):
-    """Into how many slices of K a product whose output feeds a sum is cut.  Measured at M = 1 and 8:
-    a product with few rows of W and a long K (4096 x 12288) gains 7 % from two slices; shorter ones
-    gain nothing (their time is launch and first-byte latency, not the number of workgroups)."""
-    if dtype != _BF16 or M > 16 or K % 8 != 0 or N > 8192 or K < 8192:
+    """Into how many slices of K a product is cut when its reader can add partial sums.  Products
+    with few rows of W have too few workgroups to pull the weights at speed; measured at the
+    shapes of an 8B model (N = 4096 or 6144, K = 4096 or 12288), eight slices are best for M = 8
+    and M = 64 alike and cost nothing at N = K = 4096."""
+    if dtype != _BF16 or M > 64 or K % 8 != 0 or N > 8192 or K < 2048:
         return 1
-    return 2
+    return 8
 
 
 # ----------------------------------------------------------------------------- attention
@@ -156,15 +157,23 @@ def _check_pages(k_pages, v_pages, dtype, nkv, hd, name):
 
 def qk_norm_rope_kv_write(qkv, q_out, k_pages, v_pages, page_table, tok_seq, tok_pos, q_gain, k_gain, eps,
                           cos, sin, n_heads, n_kv_heads, head_dim, write_kv=True):
-    """Split a fused [q | k | v] projection row into heads; RMSNorm q and k heads (if gains are
+    """qkv [N, width] in the activation type, or float partial sums [S, N, width] that are added first.
+    Split a fused [q | k | v] projection row into heads; RMSNorm q and k heads (if gains are
     given), rotate them at tok_pos (if tables are given; their width is rotary_dim / 2), write q to
     q_out [N, nh*hd], k and v into the cache pages of sequence tok_seq[n] at position tok_pos[n]
     (not with write_kv False: a layer that reads a cache which another layer writes)."""
     nh, nkv, hd = n_heads, n_kv_heads, head_dim
-    _need(qkv, "qk_norm_rope_kv_write.qkv", (_BF16, _F32), (None, (nh + 2 * nkv) * hd))
-    N = qkv.shape[0]
-    _need(q_out, "qk_norm_rope_kv_write.q_out", qkv.dtype, (N, nh * hd))
-    _check_pages(k_pages, v_pages, qkv.dtype, nkv, hd, "qk_norm_rope_kv_write")
+    n_parts = 0
+    if qkv.dim() == 3:          # float partial sums [S, N, width] of a product cut along K
+        n_parts = qkv.shape[0]
+        _need(qkv, "qk_norm_rope_kv_write.qkv", _F32, (n_parts, None, (nh + 2 * nkv) * hd))
+        N = qkv.shape[1]
+        _need(q_out, "qk_norm_rope_kv_write.q_out", (_BF16, _F32), (N, nh * hd))
+    else:
+        _need(qkv, "qk_norm_rope_kv_write.qkv", (_BF16, _F32), (None, (nh + 2 * nkv) * hd))
+        N = qkv.shape[0]
+        _need(q_out, "qk_norm_rope_kv_write.q_out", qkv.dtype, (N, nh * hd))
+    _check_pages(k_pages, v_pages, q_out.dtype, nkv, hd, "qk_norm_rope_kv_write")
     _need(page_table, "qk_norm_rope_kv_write.page_table", _I32, (None, None))
     _need(tok_seq, "qk_norm_rope_kv_write.tok_seq", _I32, (N,))
     _need(tok_pos, "qk_norm_rope_kv_write.tok_pos", _I32, (N,))
@@ -184,8 +193,8 @@ def qk_norm_rope_kv_write(qkv, q_out, k_pages, v_pages, page_table, tok_seq, tok
         rot = 2 * cos.shape[1]
         if rot > hd:
             raise KernelError(f"qk_norm_rope_kv_write: rotary size {rot} exceeds head size {hd}")
-    _call(load_library("core"), "syn_qk_norm_rope_kv_write", _ptr(qkv), _ptr(q_out), _ptr(k_pages), _ptr(v_pages),
-          _is_f32(qkv), _ptr(page_table), page_table.shape[1], _ptr(tok_seq), _ptr(tok_pos), _ptr(q_gain), _ptr(k_gain),
+    _call(load_library("core"), "syn_qk_norm_rope_kv_write", _ptr(qkv), n_parts, _ptr(q_out), _ptr(k_pages), _ptr(v_pages),
+          _is_f32(q_out), _ptr(page_table), page_table.shape[1], _ptr(tok_seq), _ptr(tok_pos), _ptr(q_gain), _ptr(k_gain),
           gain_f32, ctypes.c_float(eps), _ptr(cos), _ptr(sin), rot, N, nh, nkv, hd, 1 if write_kv else 0, _stream())
 
 

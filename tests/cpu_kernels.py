@@ -67,6 +67,8 @@ def gemm_slices(M, N, K, dtype):
 def qk_norm_rope_kv_write(qkv, q_out, k_pages, v_pages, page_table, tok_seq, tok_pos, q_gain, k_gain, eps,
                           cos, sin, n_heads, n_kv_heads, head_dim, write_kv=True):
     nh, nkv, hd = n_heads, n_kv_heads, head_dim
+    if qkv.dim() == 3:                      # partial sums over slices of K
+        qkv = qkv.sum(0)
     N = qkv.shape[0]
     x = qkv.to(F32).view(N, nh + 2 * nkv, hd)
     q, k, v = x[:, :nh], x[:, nh:nh + nkv], x[:, nh + nkv:]

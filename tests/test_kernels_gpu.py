@@ -252,6 +252,16 @@ def test_qk_norm_rope_kv_write(ops, dtype, nh, nkv, hd, rot, norm):
     # untouched places of the pages stay as they were
     untouched = (kw == k0)
     assert torch.equal(kd.cpu()[untouched], k0[untouched])
+    # the same from float partial sums [S, N, width] (a product cut along K): they are added first
+    if dtype == BF16:
+        parts = rnd((3, N, (nh + 2 * nkv) * hd), 24)
+        parts[2] = qkv.float() - parts[0] - parts[1]
+        kd3, vd3, qd3 = k0.to(DEV), v0.to(DEV), torch.empty((N, nh * hd), dtype=dtype, device=DEV)
+        ops.qk_norm_rope_kv_write(d(parts), qd3, kd3, vd3, d(table), d(tok_seq), d(tok_pos), d(qg), d(kg), 1e-5, d(cos),
+                                  d(sin), nh, nkv, hd)
+        close(qd3, qw, what="q from partial sums", **tol)
+        close(kd3, kw, what="k pages from partial sums", **tol)
+        close(vd3, vw, 2e-2, 1e-2, what="v pages from partial sums")
     # a reader of another layer's cache writes nothing
     kd2, vd2 = k0.to(DEV), v0.to(DEV)
     ops.qk_norm_rope_kv_write(d(qkv), qd, kd2, vd2, d(table), d(tok_seq), d(tok_pos), d(qg), d(kg), 1e-5, d(cos), d(sin),
