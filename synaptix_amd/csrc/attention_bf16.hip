@@ -339,13 +339,13 @@ SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, co
 }
 
 // ------------------------------------------------------------------ decode: split over keys, then merge
-// A workgroup of DEC_WAVES waves takes (sequence, kv head, up to 16 heads of its group, one split of
+// A workgroup of up to 8 waves takes (sequence, kv head, up to 16 heads of its group, one split of
 // the key blocks); its waves take the split's blocks in turn and their states are combined in LDS.
 // With one split the workgroup writes the output itself; else it writes a partial
 //   partial[(seq * nh + head) * n_splits + split] = { m, l, o[HD] }   (float)
 // and a second kernel merges the splits.
 constexpr int PART = HD + 2;
-constexpr int DEC_WAVES = HD > 128 ? 2 : 4;
+constexpr int DEC_MAX_WAVES = HD > 128 ? 4 : 8;  // as many as keep their ~190 registers each without spilling
 
 // Like attn_block for one column block, but every K and V fragment of the block is requested before
 // the first product needs one: a block costs one trip to memory instead of two.
@@ -420,14 +420,18 @@ __device__ __forceinline__ void attn_block_decode(AttnState<1>& st, const QFrag&
   }
 }
 
-__global__ void __launch_bounds__(DEC_WAVES * SYN_WAVE)
+__global__ void __launch_bounds__(DEC_MAX_WAVES * SYN_WAVE)
 attn_decode_split_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages,
                          const bf16* __restrict__ v_pages, const int* __restrict__ page_table, int table_stride,
                          const int* __restrict__ seq_len, float* __restrict__ partial, bf16* __restrict__ out,
-                         float scale, int window, int nh, int nkv, int n_splits) {
-  __shared__ float sm[DEC_WAVES][16];            // running maximum of each column
-  __shared__ float sl[DEC_WAVES][16];            // sum of each column
-  __shared__ float so[DEC_WAVES][16][HD + 4];    // unnormalised output of each column
+                         float scale, int window, int nh, int nkv, int n_splits, int cols_alloc) {
+  // LDS: sm[waves][16] running maxima, sl[waves][16] sums, so[waves][cols_alloc][HD + 4] outputs
+  extern __shared__ float dec_lds[];
+  const int n_waves = blockDim.x / SYN_WAVE;
+  float* sm = dec_lds;
+  float* sl = sm + n_waves * 16;
+  float* so = sl + n_waves * 16;
+  constexpr int SO_LD = HD + 4;
   const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
   const int seq = blockIdx.x, split = blockIdx.z;
   const int g = nh / nkv, chunks = (g + 15) / 16;
@@ -446,7 +450,7 @@ attn_decode_split_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
   const int b_lo = lo / SYN_PAGE, b_hi = pos / SYN_PAGE;
   const int per = (b_hi - b_lo + n_splits) / n_splits;  // ceil((b_hi - b_lo + 1) / n_splits)
   const int b0 = b_lo + split * per, b1 = min(b_hi + 1, b0 + per);
-  for (int kb = b0 + wave; kb < b1; kb += DEC_WAVES) {
+  for (int kb = b0 + wave; kb < b1; kb += n_waves) {
     const size_t base = ((size_t)page_table[(size_t)seq * table_stride + kb] * nkv + kvh) * SYN_PAGE * HD;
     attn_block_decode(st, qf, k_pages + base, v_pages + base, kb * SYN_PAGE, valid ? pos : -1, lo, kv_len, scale, lane);
   }
@@ -454,28 +458,27 @@ attn_decode_split_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
   l += __shfl_xor(l, 16, SYN_WAVE);
   l += __shfl_xor(l, 32, SYN_WAVE);
   if (lane < 16) {
-    sm[wave][lane] = st.m[0];
-    sl[wave][lane] = l;
+    sm[wave * 16 + lane] = st.m[0];
+    sl[wave * 16 + lane] = l;
   }
   if (valid) {
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) so[wave][col][dt * 16 + 4 * (lane / 16) + e] = st.o[dt][0][e];
+      for (int e = 0; e < 4; ++e) so[((size_t)wave * cols_alloc + col) * SO_LD + dt * 16 + 4 * (lane / 16) + e] = st.o[dt][0][e];
   }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < n_cols * HD; idx += DEC_WAVES * SYN_WAVE) {
+  for (int idx = threadIdx.x; idx < n_cols * HD; idx += blockDim.x) {
     const int c = idx / HD, d = idx % HD;
     float m = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < DEC_WAVES; ++w) m = fmaxf(m, sm[w][c]);
+    for (int w = 0; w < n_waves; ++w) m = fmaxf(m, sm[w * 16 + c]);
     float acc = 0.f, lsum = 0.f;
-#pragma unroll
-    for (int w = 0; w < DEC_WAVES; ++w) {
-      if (sm[w][c] == -INFINITY) continue;  // a wave that had no block
-      const float f = __expf(sm[w][c] - m);
-      acc += f * so[w][c][d];
-      lsum += f * sl[w][c];
+    for (int w = 0; w < n_waves; ++w) {
+      const float mw = sm[w * 16 + c];
+      if (mw == -INFINITY) continue;  // a wave that had no block
+      const float f = __expf(mw - m);
+      acc += f * so[((size_t)w * cols_alloc + c) * SO_LD + d];
+      lsum += f * sl[w * 16 + c];
     }
     const int head = kvh * g + chunk * 16 + c;
     if (n_splits == 1) {
@@ -538,9 +541,18 @@ SYN_EXPORT int syn_attention_decode_bf16(const void* q, const void* k_pages, con
   SYN_CHECK(nh % nkv == 0, "attention_decode: %d heads do not divide into %d kv heads", nh, nkv);
   const int chunks = (nh / nkv + 15) / 16;
   SYN_CHECK(nkv * chunks <= 65535 && n_splits <= 65535, "attention_decode: grid too large");
-  attn_decode_split_kernel<<<dim3(n_seqs, nkv * chunks, n_splits), DEC_WAVES * SYN_WAVE, 0, stream>>>(
+  // waves a workgroup: as many as the LDS for their states allows (up to 8), but no more than make
+  // about 2,048 waves in all: at large batches four waves a workgroup are plenty
+  const int cols_alloc = nh / nkv < 16 ? nh / nkv : 16;
+  int waves = DEC_MAX_WAVES;
+  while (waves > 2 && ((size_t)waves * (32 + (size_t)cols_alloc * (HD + 4)) * sizeof(float) > 64 * 1024 ||
+                       (long)n_seqs * nkv * chunks * n_splits * waves > 2048))
+    waves /= 2;
+  if (waves < 4 && (size_t)4 * (32 + (size_t)cols_alloc * (HD + 4)) * sizeof(float) <= 64 * 1024) waves = 4;
+  const size_t lds = (size_t)waves * (32 + (size_t)cols_alloc * (HD + 4)) * sizeof(float);
+  attn_decode_split_kernel<<<dim3(n_seqs, nkv * chunks, n_splits), waves * SYN_WAVE, lds, stream>>>(
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, page_table, table_stride, seq_len, workspace,
-      (bf16*)out, scale, window, nh, nkv, n_splits);
+      (bf16*)out, scale, window, nh, nkv, n_splits, cols_alloc);
   SYN_LAUNCH_CHECK("attention_decode_split");
   if (n_splits > 1) {
     attn_decode_merge_kernel<<<n_seqs * nh, SYN_WAVE, 0, stream>>>(workspace, (bf16*)out, n_splits);

@@ -13,7 +13,6 @@
 // mma.sync m16n8k16), best_cu/gemv/mma_gemv.cu:19-133 (M == 1), best_cu/gemm/gemm_f32.cu (SIMT).
 // The tilings here are made for 64-lane waves and MFMA operand layouts, not translated.
 #include "common.h"
-#include <stdlib.h>
 
 // ------------------------------------------------------------------ SIMT, any type
 #define SIMT_BM 64
@@ -452,6 +451,8 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   const bf16* wb = (const bf16*)w;
   // x through LDS (waves on different rows of W) for the widest products and for every product
   // that is cut along K; measured against gemm_skinny at M = 8, 16 and 64 for the shapes of an 8B model
+  // x through LDS (waves on different rows of W) for the widest products and for every product
+  // that is cut along K; measured against gemm_skinny at M = 8, 16 and 64 for the shapes of an 8B model
   if (M <= 64 && (slices > 1 || N > 32768)) {
     const int mb = (M + 15) / 16;
     if (mb == 1) launch_xlds<1, 1, 4, 128>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
@@ -461,45 +462,28 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
     SYN_LAUNCH_CHECK("gemm_xlds");
     return 0;
   }
-  // rows of W a workgroup owns: more rows amortise the loads of x, fewer rows give more workgroups
-  const int variant = getenv("SYN_SKINNY") ? atoi(getenv("SYN_SKINNY")) : -1;
+  // gemm_skinny: rows of W a workgroup owns, waves and unroll by (M, N), from sweeps at the shapes of
+  // an 8B model: few rows (many workgroups) win up to M = 16; more rows amortise x beyond that
   if (M <= 16) {
-    const int v = variant >= 0 ? variant : ((N <= 8192 && slices == 1) ? 0 : 1);
-    if (v == 0) launch_skinny<1, 1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else if (v == 1) launch_skinny<1, 1, 8, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else if (v == 2) launch_skinny<1, 2, 8, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else if (v == 3) launch_skinny<1, 4, 8, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else if (v == 4) launch_skinny<1, 2, 16, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else launch_skinny<1, 4, 8, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    if (N <= 8192) launch_skinny<1, 1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else launch_skinny<1, 1, 8, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
   } else if (M <= 32) {
-    const int v = variant >= 0 ? variant : (N <= 4096 ? 0 : (N <= 8192 ? 1 : 2));
-    if (v == 0) launch_skinny<2, 1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else if (v == 1) launch_skinny<2, 2, 8, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else if (v == 2) launch_skinny<2, 4, 8, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else if (v == 3) launch_skinny<2, 2, 16, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else launch_skinny<2, 4, 4, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    if (N <= 4096) launch_skinny<2, 1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else if (N <= 8192) launch_skinny<2, 2, 8, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else launch_skinny<2, 4, 8, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
   } else if (M <= 48) {
     launch_skinny<3, 2, 8, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
   } else if (M <= 64) {
-    const int v = variant >= 0 ? variant : (N <= 4096 ? 0 : (N <= 8192 ? 3 : 4));
-    if (v == 0) launch_skinny<4, 1, 16, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else if (v == 1) launch_skinny<4, 2, 8, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else if (v == 2) launch_skinny<4, 4, 8, 1>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else if (v == 3) launch_skinny<4, 2, 16, 1>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    if (N <= 4096) launch_skinny<4, 1, 16, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    else if (N <= 8192) launch_skinny<4, 2, 16, 1>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
     else launch_skinny<4, 4, 4, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
   } else {
     // 256 x 256 tiles (8 waves) where they keep at least three quarters of the compute units busy,
     // 128 x 128 tiles (4 waves) for smaller problems
-    const int tv = getenv("SYN_TILED") ? atoi(getenv("SYN_TILED")) : -1;
     const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-    const int v = tv >= 0 ? tv : (t256 >= 192 ? 0 : 1);
     int rc;
-    if (v == 0) rc = launch_tiled<256, 256, 64, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 1) rc = launch_tiled<128, 128, 64, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 2) rc = launch_tiled<256, 256, 32, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 3) rc = launch_tiled<256, 128, 64, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (v == 4) rc = launch_tiled<256, 256, 64, 2, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else rc = launch_tiled<128, 256, 64, 2, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
+    if (t256 >= 192) rc = launch_tiled<256, 256, 64, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else rc = launch_tiled<128, 128, 64, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
     if (rc) return rc;
   }
   SYN_LAUNCH_CHECK("gemm");

@@ -27,8 +27,13 @@ TINY_B = dict(num_hidden_layers=3, hidden_size=128, num_attention_heads=8, num_k
 TINY_C = dict(num_hidden_layers=2, hidden_size=120, num_attention_heads=6, num_key_value_heads=2, head_dim=48,
               intermediate_size=200, vocab_size=777, rope_theta=5e5, rms_norm_eps=3e-6, max_position_embeddings=1024,
               tie_word_embeddings=False, eos_token_id=None, bos_token_id=None)
-SEEDS = {"A": 0, "B": 1, "C": 2}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+# A middle-sized one: wide enough that the engine takes the kernels which the tiny ones never reach
+# (partial sums over slices of K, x through LDS, the large GEMM tiles), still seconds on the CPU.
+MID_D = dict(num_hidden_layers=2, hidden_size=2048, num_attention_heads=16, num_key_value_heads=4, head_dim=128,
+             intermediate_size=2560, vocab_size=33024, rope_theta=1e6, rms_norm_eps=1e-6, max_position_embeddings=2048,
+             tie_word_embeddings=True, eos_token_id=None, bos_token_id=None)
+SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": MID_D}
 
 _made = {}
 _tmp = None

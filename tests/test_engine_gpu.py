@@ -94,6 +94,32 @@ def test_batch_rows_do_not_depend_on_their_neighbours():
         assert float((lg - alone).abs().max()) <= (1e-5 if dtype == "float32" else 2e-2)
 
 
+def test_middle_sized_model_reaches_the_large_kernels():
+    """Hidden 2048, head size 128, vocabulary 33024: prompts of hundreds of tokens take the tiled GEMM,
+    single tokens the products cut along K and the wide output product with x through LDS."""
+    name, dtype = "D", "bfloat16"
+    V = CONFIGS[name]["vocab_size"]
+    reqs = [random_tokens(V, n, 700 + n) for n in (300, 130, 65)]
+    eng = make_engine(name, dtype, 2048)
+    slots = [eng.acquire() for _ in reqs]
+    head = [len(r) - 6 for r in reqs]
+    got = [[] for _ in reqs]
+    lg = eng.step([(s, r[:h]) for s, r, h in zip(slots, reqs, head)], want=[[h - 2, h - 1] for h in head])
+    for i in range(3):
+        got[i].append(lg[2 * i:2 * i + 2])
+    for j in range(6):
+        lg = eng.step([(s, [r[h + j]]) for s, r, h in zip(slots, reqs, head)], want="last")
+        for i in range(3):
+            got[i].append(lg[i:i + 1])
+    for i, r in enumerate(reqs):
+        want = plain_logits(name, r)[head[i] - 2:]
+        assert_logits_close(torch.cat(got[i]), want, dtype, f"middle-sized model, request {i}")
+    # and the 32-bit path of the same model on one short request
+    e32 = make_engine(name, "float32", 256)
+    s = e32.acquire()
+    assert_logits_close(e32.step([(s, reqs[2])], want="last"), plain_logits(name, reqs[2])[-1:], "float32", "middle-sized, 32-bit")
+
+
 # ----------------------------------------------------------------------------- the replay program
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_trace_run_whole_one_by_one_and_batched(tmp_path, dtype):

@@ -140,6 +140,8 @@ def test_gemm_f32(ops, M, N, K):
     (1, 48, 64), (3, 1000, 176), (16, 100, 320), (17, 40, 72), (33, 1000, 128), (48, 70, 2048), (64, 4096, 512),
     (65, 130, 104), (128, 128, 32), (200, 300, 1000), (513, 257, 4096),
     (5, 30, 20), (70, 50, 36),          # K no multiple of 8: the plain kernel takes them
+    (2048, 6144, 512), (1000, 12300, 136),   # large enough for the 256 x 256 tiles with 8 waves, ragged edges
+    (8, 40000, 256), (40, 33000, 72), (64, 50000, 1000),   # wide enough for x through LDS
 ])
 def test_gemm_bf16(ops, out_dtype, M, N, K):
     x, w = rnd((M, K), 10, BF16), rnd((N, K), 11, BF16)
