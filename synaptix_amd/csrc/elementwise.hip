@@ -69,7 +69,26 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const float* __res
 }
 
 // The same for rows whose width is a multiple of 4 and at most 4 * VPT * blockDim: every thread
-// keeps its values (float4 loads) in registers between the sum of squares and the scaling.
+// keeps its values (float4 loads) in registers between the sum of squares and the scaling.  The
+// partial sums are fetched eight at a time, so that their loads are in flight together, and
+// added in their order.
+__device__ inline float4 load_gain4(const void* gain, int gain_is_f32, int i4) {
+  if (gain_is_f32) return ((const float4*)gain)[i4];
+  struct alignas(8) bf16x4s { bf16 e[4]; };
+  const bf16x4s g = ((const bf16x4s*)gain)[i4];
+  return make_float4((float)g.e[0], (float)g.e[1], (float)g.e[2], (float)g.e[3]);
+}
+
+__device__ inline void store4(float* o, int i4, const float4 r) { ((float4*)o)[i4] = r; }
+__device__ inline void store4(bf16* o, int i4, const float4 r) {
+  struct alignas(8) bf16x4s { bf16 e[4]; } t;
+  t.e[0] = (bf16)r.x;
+  t.e[1] = (bf16)r.y;
+  t.e[2] = (bf16)r.z;
+  t.e[3] = (bf16)r.w;
+  ((bf16x4s*)o)[i4] = t;
+}
+
 template <typename TOut, int VPT>
 __global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const float* __restrict__ delta, int n_parts,
                                        size_t part_stride, const int* __restrict__ rows,
@@ -83,20 +102,27 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const float* _
   const bool write_back = (rows == nullptr) && (d != nullptr);
   const int H4 = H / 4;
   const size_t stride4 = part_stride / 4;
-  float4 v[VPT];
+  float4 v[VPT], g[VPT];
   float ss = 0.f;
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
     const int i = threadIdx.x + j * blockDim.x;
     if (i < H4) {
       v[j] = x[i];
+      g[j] = load_gain4(gain, gain_is_f32, i);  // fetched here, beside the values, not after the sum
       if (d) {
-        for (int p = 0; p < n_parts; ++p) {
-          const float4 t = d[p * stride4 + i];
-          v[j].x += t.x;
-          v[j].y += t.y;
-          v[j].z += t.z;
-          v[j].w += t.w;
+        for (int p0 = 0; p0 < n_parts; p0 += 8) {
+          float4 t[8];
+#pragma unroll
+          for (int q = 0; q < 8; ++q)
+            t[q] = p0 + q < n_parts ? d[(size_t)(p0 + q) * stride4 + i] : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+          for (int q = 0; q < 8; ++q) {
+            v[j].x += t[q].x;
+            v[j].y += t[q].y;
+            v[j].z += t[q].z;
+            v[j].w += t[q].w;
+          }
         }
       }
       if (write_back) x[i] = v[j];
@@ -108,11 +134,9 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const float* _
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
     const int i = threadIdx.x + j * blockDim.x;
-    if (i < H4) {
-      const float e[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
-#pragma unroll
-      for (int c = 0; c < 4; ++c) o[4 * i + c] = from_f32<TOut>(load_gain(gain, gain_is_f32, 4 * i + c) * e[c] * inv);
-    }
+    if (i < H4)
+      store4(o, i, make_float4(g[j].x * v[j].x * inv, g[j].y * v[j].y * inv, g[j].z * v[j].z * inv,
+                               g[j].w * v[j].w * inv));
   }
 }
 
@@ -122,10 +146,11 @@ SYN_EXPORT int syn_add_rmsnorm(float* resid, const float* delta, int n_parts, in
   SYN_CHECK(n_out > 0 && H > 0 && n_rows > 0, "add_rmsnorm: empty input (%d rows, width %d)", n_out, H);
   SYN_CHECK(n_parts >= 1 && n_parts <= 64, "add_rmsnorm: %d partial sums", n_parts);
   const size_t stride = (size_t)n_rows * H;
-  const bool vec = H % 4 == 0 && H <= 4 * 4 * 512 && ((uintptr_t)resid % 16 == 0) && ((uintptr_t)delta % 16 == 0);
+  const bool vec = H % 4 == 0 && H <= 4 * 4 * 1024 && ((uintptr_t)resid % 16 == 0) && ((uintptr_t)delta % 16 == 0) &&
+                   ((uintptr_t)out % 16 == 0) && ((uintptr_t)gain % 16 == 0);
   if (vec) {
     const int H4 = H / 4;
-    const int block = H4 <= 256 ? 256 : 512;
+    const int block = H4 <= 256 ? 256 : (H4 <= 512 ? 512 : 1024);
     const int vpt = (H4 + block - 1) / block;  // 1 .. 4
 #define SYN_ARN(T, V)                                                                                          \
   add_rmsnorm_vec_kernel<T, V><<<n_out, block, 0, stream>>>(resid, delta, n_parts, stride, rows, gain, gain_is_f32, \

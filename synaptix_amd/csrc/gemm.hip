@@ -177,7 +177,9 @@ static void launch_skinny(const bf16* x, const bf16* w, void* out, int out_is_f3
 // rows of x for a k-tile go through LDS once and serve all waves, so x costs M / (16 * RT * WAVES)
 // of the weight traffic instead of M / (16 * RT).  W fragments come straight from memory (each is
 // used by one wave only), two k-tiles ahead.  blockIdx.y cuts K into slices as in gemm_skinny.
-template <int MB, int RT, int WAVES, int BK>
+// GATED: x is not stored anywhere; row m of it is silu(g) * u of the row [g (K values) | u (K values)]
+// of a fused gate/up product, computed in 32-bit and rounded once on its way into LDS.
+template <int MB, int RT, int WAVES, int BK, bool GATED>
 __global__ void __launch_bounds__(WAVES * SYN_WAVE)
 gemm_xlds_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
                  int M, int N, int K, int k_slice) {
@@ -197,20 +199,34 @@ gemm_xlds_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* _
 #pragma unroll
   for (int r = 0; r < RT; ++r) wrow[r] = w + (size_t)min(n0 + r * 16 + r16, N - 1) * K + kq;
 
-  bf16x8 rx[XL];
+  bf16x8 rx[XL], ru[GATED ? XL : 1];
   auto fetch_x = [&](int kt) {
 #pragma unroll
     for (int i = 0; i < XL; ++i) {
       const int c = tid + i * WAVES * 64;
       const int row = c / (BK / 8), k = k_begin + kt * BK + (c % (BK / 8)) * 8;
-      rx[i] = (c < XCH && row < M && k < k_end) ? *(const bf16x8*)(x + (size_t)row * K + k) : zero;
+      const bool ok = c < XCH && row < M && k < k_end;
+      if constexpr (GATED) {
+        rx[i] = ok ? *(const bf16x8*)(x + (size_t)row * 2 * K + k) : zero;
+        ru[i] = ok ? *(const bf16x8*)(x + (size_t)row * 2 * K + K + k) : zero;
+      } else {
+        rx[i] = ok ? *(const bf16x8*)(x + (size_t)row * K + k) : zero;
+      }
     }
   };
   auto stash_x = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < XL; ++i) {
       const int c = tid + i * WAVES * 64;
-      if (c < XCH) *(bf16x8*)(&xs[buf][(c / (BK / 8)) * LD + (c % (BK / 8)) * 8]) = rx[i];
+      bf16x8 v = rx[i];
+      if constexpr (GATED) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float g = (float)rx[i][e];
+          v[e] = (bf16)(g / (1.f + expf(-g)) * (float)ru[i][e]);
+        }
+      }
+      if (c < XCH) *(bf16x8*)(&xs[buf][(c / (BK / 8)) * LD + (c % (BK / 8)) * 8]) = v;
     }
   };
   bf16x8 bw0[KS][RT], bw1[KS][RT];  // W fragments of even and of odd k-tiles (indices known at compile time)
@@ -275,12 +291,12 @@ gemm_xlds_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* _
       }
 }
 
-template <int MB, int RT, int WAVES, int BK>
+template <int MB, int RT, int WAVES, int BK, bool GATED = false>
 static void launch_xlds(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K, int slices,
                         hipStream_t stream) {
   const int k_slice = ((K + slices - 1) / slices + 31) / 32 * 32;
   const int rows = WAVES * RT * 16;
-  gemm_xlds_kernel<MB, RT, WAVES, BK><<<dim3((N + rows - 1) / rows, slices), WAVES * SYN_WAVE, 0, stream>>>(
+  gemm_xlds_kernel<MB, RT, WAVES, BK, GATED><<<dim3((N + rows - 1) / rows, slices), WAVES * SYN_WAVE, 0, stream>>>(
       x, w, out, out_is_f32, M, N, K, k_slice);
 }
 
@@ -451,8 +467,6 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   const bf16* wb = (const bf16*)w;
   // x through LDS (waves on different rows of W) for the widest products and for every product
   // that is cut along K; measured against gemm_skinny at M = 8, 16 and 64 for the shapes of an 8B model
-  // x through LDS (waves on different rows of W) for the widest products and for every product
-  // that is cut along K; measured against gemm_skinny at M = 8, 16 and 64 for the shapes of an 8B model
   if (M <= 64 && (slices > 1 || N > 32768)) {
     const int mb = (M + 15) / 16;
     if (mb == 1) launch_xlds<1, 1, 4, 128>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
@@ -487,5 +501,29 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
     if (rc) return rc;
   }
   SYN_LAUNCH_CHECK("gemm");
+  return 0;
+}
+
+// out = (silu(g) * u) . w^T for rows [g | u] of gate_up [M, 2K] (bf16, M <= 64), w [N, K]: the
+// activation is applied while x is on its way into LDS and is never stored.  dtype and slices as in
+// syn_gemm (1 = bf16 out, 2 = float out, slices of K only with float out).
+SYN_EXPORT int syn_gemm_gated(const void* gate_up, const void* w, void* out, int dtype, int M, int N, int K,
+                              int slices, hipStream_t stream) {
+  SYN_CHECK(M > 0 && N > 0 && K > 0, "gemm_gated: empty shape M=%d N=%d K=%d", M, N, K);
+  SYN_CHECK(dtype == 1 || dtype == 2, "gemm_gated: bf16 operands only (dtype code %d)", dtype);
+  SYN_CHECK(M <= 64, "gemm_gated: at most 64 rows (M = %d)", M);
+  SYN_CHECK(slices >= 1 && slices <= 64 && (slices == 1 || dtype == 2), "gemm_gated: %d slices of K need a float output",
+            slices);
+  SYN_CHECK(K % 8 == 0 && (uintptr_t)gate_up % 16 == 0 && (uintptr_t)w % 16 == 0,
+            "gemm_gated: K = %d must be a multiple of 8 and the operands 16-byte aligned", K);
+  const bf16* xb = (const bf16*)gate_up;
+  const bf16* wb = (const bf16*)w;
+  const int out_is_f32 = dtype == 2;
+  const int mb = (M + 15) / 16;
+  if (mb == 1) launch_xlds<1, 1, 4, 128, true>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+  else if (mb == 2) launch_xlds<2, 1, 4, 128, true>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+  else if (mb == 3) launch_xlds<3, 1, 4, 128, true>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+  else launch_xlds<4, 1, 4, 128, true>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+  SYN_LAUNCH_CHECK("gemm_gated");
   return 0;
 }

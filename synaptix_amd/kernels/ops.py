@@ -138,6 +138,28 @@ def gemm(x, w, out, force_simt=False):
           slices, _stream())
 
 
+def gemm_gated(gate_up, w, out):
+    """out = (silu(g) * u) . w^T for rows [g | u] of gate_up [M, 2K] (bf16, M <= 64) and w [N, K]:
+    the gated activation inside the product, so that it is never stored.  out is [M, N] in bf16
+    or float, or float partial sums [S, M, N] over slices of K."""
+    _need(gate_up, "gemm_gated.gate_up", _BF16, (None, None))
+    M, K2 = gate_up.shape
+    if K2 % 2 or M > 64:
+        raise KernelError(f"gemm_gated: gate_up {tuple(gate_up.shape)} needs an even width and at most 64 rows")
+    K = K2 // 2
+    _need(w, "gemm_gated.w", _BF16, (None, K))
+    N = w.shape[0]
+    slices = 1
+    if out.dim() == 3:
+        slices = out.shape[0]
+        _need(out, "gemm_gated.out", _F32, (slices, M, N))
+        code = 2
+    else:
+        _need(out, "gemm_gated.out", (_BF16, _F32), (M, N))
+        code = 2 if out.dtype == _F32 else 1
+    _call(load_library("core"), "syn_gemm_gated", _ptr(gate_up), _ptr(w), _ptr(out), code, M, N, K, slices, _stream())
+
+
 def gemm_slices(M, N, K, dtype):
     """Into how many slices of K a product is cut when its reader can add partial sums.  Products
     with few rows of W have too few workgroups to pull the weights at speed; measured at the

@@ -10,7 +10,7 @@ import torch
 from ..kernels import ops
 from ..weights.source import TensorSpec
 from .base import Part
-from .linear import linear, linear_for_sum
+from .linear import gated_linear_for_sum, linear, linear_for_sum
 
 
 class FeedForward(Part):
@@ -42,6 +42,9 @@ class GatedMlp(FeedForward):
 
     def forward(self, h, ctx):
         gu = linear(h, self.w_gate_up, h.dtype)
+        fused = gated_linear_for_sum(gu, self.w_down)
+        if fused is not None:
+            return fused
         m = torch.empty((h.shape[0], self.intermediate), dtype=h.dtype, device=h.device)
         ops.swiglu(gu, m)
         return linear_for_sum(m, self.w_down)

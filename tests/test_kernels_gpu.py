@@ -186,6 +186,30 @@ def test_gemm_bf16_partial_sums_over_slices_of_k(ops, M, N, K, S):
     close(got2, want2, 1e-4, 1e-4, "gathered rows of residual + slices")
 
 
+@pytest.mark.parametrize("M,N,K,S", [(1, 48, 64, 1), (8, 4096, 12288, 8), (7, 100, 1000, 3), (33, 70, 136, 1),
+                                     (64, 130, 2048, 4)])
+def test_gemm_with_gated_activation_inside(ops, M, N, K, S):
+    """(silu(g) * u) . W^T from the fused [g | u] rows equals the activation kernel followed by the
+    product, value for value: the activation is rounded to bf16 once in both."""
+    gu, w = rnd((M, 2 * K), 18, BF16).to(DEV), rnd((N, K), 19, BF16).to(DEV)
+    act = torch.empty((M, K), dtype=BF16, device=DEV)
+    ops.swiglu(gu, act)
+    g, u = gu[:, :K].cpu().float(), gu[:, K:].cpu().float()
+    close(act, (g / (1 + torch.exp(-g)) * u).to(BF16), 2e-2, 1e-2, "activation kernel")
+    want = (act.cpu().double() @ w.cpu().double().T).float()
+    shape = (S, M, N) if S > 1 else (M, N)
+    out = torch.full(shape, float("nan"), dtype=F32, device=DEV)
+    ops.gemm_gated(gu, w, out)
+    got = out.sum(0) if S > 1 else out
+    close(got, want, 1e-3 * math.sqrt(K), what=f"gated product {M}x{N}x{K}, {S} slice(s)")
+    if S == 1:
+        out16 = torch.empty((M, N), dtype=BF16, device=DEV)
+        ops.gemm_gated(gu, w, out16)
+        close(out16, want, 1e-3 * math.sqrt(K) + 0.02, 1e-2, "gated product, bf16 out")
+    with pytest.raises(Exception, match="64 rows"):
+        ops.gemm_gated(torch.zeros((65, 2 * K), dtype=BF16, device=DEV), w, torch.empty((65, N), dtype=F32, device=DEV))
+
+
 def test_gemm_bf16_paths_agree(ops):
     """The MFMA kernels and the plain kernel compute the same sums."""
     for M in (4, 40, 300):
