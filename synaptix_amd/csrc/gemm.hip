@@ -2,12 +2,15 @@
 //
 //   gemm_simt      any shape and type; plain FMA.  The whole 32-bit path, and bf16 shapes that
 //                  the MFMA kernels refuse (K not a multiple of 8, unaligned rows).
-//   gemm_skinny    bf16, M <= 64: the weight matrix is streamed once from HBM through
+//   gemm_skinny    bf16, M == 1: the weight matrix is streamed once from HBM through
 //                  v_mfma_f32_16x16x32_bf16; the waves of a workgroup split K and sum in LDS.
-//   gemm_xlds      bf16, M <= 64: the waves of a workgroup own different rows of W and share the rows
-//                  of x through LDS; K may be cut into slices whose partial sums the reader adds.
-//   gemm_tiled     bf16, M > 64: 256x256x64 tiles with 8 waves (or 128x128x64 with 4) in LDS,
-//                  double-buffered, v_mfma_f32_32x32x16_bf16.
+//   gemm_tiled     bf16: tiles of x and W in LDS, double-buffered, v_mfma_f32_32x32x16_bf16.
+//                  M > 64: 256x256x64 tiles with 8 waves (or 128x128x64 with 4).
+//                  M <= 64: 32 or 64 rows of x, 64 (or 32) rows of W, 128 (or 256) deep: the rows of
+//                  W arrive as whole 256-byte pieces, which streams them faster than loading MFMA
+//                  fragments (64 bytes a row) straight from memory.  K may be cut into slices
+//                  whose partial sums the reader adds; x may be the gated activation of a fused
+//                  [gate | up] row, computed on its way into LDS.
 //
 // Reference counterparts: crates/synaptix-kernels-cuda/src/best_cu/gemm/gemm_bf16.cu (TN family,
 // mma.sync m16n8k16), best_cu/gemv/mma_gemv.cu:19-133 (M == 1), best_cu/gemm/gemm_f32.cu (SIMT).
@@ -60,7 +63,7 @@ gemm_simt_kernel(const TIn* __restrict__ x, const TIn* __restrict__ w, TOut* __r
     }
 }
 
-// ------------------------------------------------------------------ skinny, bf16, M <= 64
+// ------------------------------------------------------------------ skinny, bf16, one row of x (or a few)
 // MFMA 16x16x32: A = x rows (m), B = W rows (n), D[m = 4*(lane/16)+j][n = lane%16].
 // Both operands: lane holds row lane%16, k = 8*(lane/16) .. +8, one 16-byte load.
 // A workgroup owns RT*16 rows of W; its WAVES waves take k-chunks of 32 round-robin, so that at
@@ -165,151 +168,25 @@ static void launch_skinny(const bf16* x, const bf16* w, void* out, int out_is_f3
   const size_t lds = (size_t)WAVES * MB * RT * 4 * 64 * sizeof(float);
   static bool raised = false;
   if (lds > 65536 && !raised) {
-    hipFuncSetAttribute((const void*)gemm_skinny_kernel<MB, RT, WAVES, U>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                        (int)lds);
+    if (hipFuncSetAttribute((const void*)gemm_skinny_kernel<MB, RT, WAVES, U>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return;  // the launch reports the refusal
     raised = true;
   }
   gemm_skinny_kernel<MB, RT, WAVES, U><<<grid, WAVES * SYN_WAVE, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
 }
 
-// ------------------------------------------------------------------ skinny with x in LDS, bf16, M <= 64
-// The waves of a workgroup own different rows of W (16 * RT each) and run over the same K range; the
-// rows of x for a k-tile go through LDS once and serve all waves, so x costs M / (16 * RT * WAVES)
-// of the weight traffic instead of M / (16 * RT).  W fragments come straight from memory (each is
-// used by one wave only), two k-tiles ahead.  blockIdx.y cuts K into slices as in gemm_skinny.
-// GATED: x is not stored anywhere; row m of it is silu(g) * u of the row [g (K values) | u (K values)]
-// of a fused gate/up product, computed in 32-bit and rounded once on its way into LDS.
-template <int MB, int RT, int WAVES, int BK, bool GATED>
-__global__ void __launch_bounds__(WAVES * SYN_WAVE)
-gemm_xlds_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
-                 int M, int N, int K, int k_slice) {
-  constexpr int LD = BK + 8;
-  constexpr int KS = BK / 32;                              // k-steps of 32 in a k-tile
-  constexpr int XCH = MB * 16 * (BK / 8);                  // 16-byte chunks of an x tile
-  constexpr int XL = (XCH + WAVES * 64 - 1) / (WAVES * 64);  // chunks a thread moves
-  __shared__ __attribute__((aligned(16))) bf16 xs[2][MB * 16 * LD];
-  const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE;
-  const int r16 = lane % 16, kq = (lane / 16) * 8;
-  const int n0 = (blockIdx.x * WAVES + wave) * (RT * 16);
-  const int k_begin = (int)blockIdx.y * k_slice, k_end = min(K, k_begin + k_slice);
-  const int nk = (k_end - k_begin + BK - 1) / BK;
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-
-  const bf16* wrow[RT];
-#pragma unroll
-  for (int r = 0; r < RT; ++r) wrow[r] = w + (size_t)min(n0 + r * 16 + r16, N - 1) * K + kq;
-
-  bf16x8 rx[XL], ru[GATED ? XL : 1];
-  auto fetch_x = [&](int kt) {
-#pragma unroll
-    for (int i = 0; i < XL; ++i) {
-      const int c = tid + i * WAVES * 64;
-      const int row = c / (BK / 8), k = k_begin + kt * BK + (c % (BK / 8)) * 8;
-      const bool ok = c < XCH && row < M && k < k_end;
-      if constexpr (GATED) {
-        rx[i] = ok ? *(const bf16x8*)(x + (size_t)row * 2 * K + k) : zero;
-        ru[i] = ok ? *(const bf16x8*)(x + (size_t)row * 2 * K + K + k) : zero;
-      } else {
-        rx[i] = ok ? *(const bf16x8*)(x + (size_t)row * K + k) : zero;
-      }
-    }
-  };
-  auto stash_x = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < XL; ++i) {
-      const int c = tid + i * WAVES * 64;
-      bf16x8 v = rx[i];
-      if constexpr (GATED) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float g = (float)rx[i][e];
-          v[e] = (bf16)(g / (1.f + expf(-g)) * (float)ru[i][e]);
-        }
-      }
-      if (c < XCH) *(bf16x8*)(&xs[buf][(c / (BK / 8)) * LD + (c % (BK / 8)) * 8]) = v;
-    }
-  };
-  bf16x8 bw0[KS][RT], bw1[KS][RT];  // W fragments of even and of odd k-tiles (indices known at compile time)
-  auto fetch_w = [&](int kt, bf16x8 (&bw)[KS][RT]) {
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int k = k_begin + kt * BK + ks * 32;
-#pragma unroll
-      for (int r = 0; r < RT; ++r)
-        bw[ks][r] = (k + kq < k_end) ? __builtin_nontemporal_load((const bf16x8*)(wrow[r] + k)) : zero;
-    }
-  };
-
-  f32x4 acc[MB][RT];
-#pragma unroll
-  for (int b = 0; b < MB; ++b)
-#pragma unroll
-    for (int r = 0; r < RT; ++r) acc[b][r] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
-  // one k-tile: x fragments from LDS buffer `buf`, W fragments from `bw`, which is refilled for the
-  // tile after next as soon as it is used up
-  auto tile = [&](int kt, int buf, bf16x8 (&bw)[KS][RT]) {
-    if (kt + 1 < nk) fetch_x(kt + 1);
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      bf16x8 ax[MB];
-#pragma unroll
-      for (int b = 0; b < MB; ++b) ax[b] = *(const bf16x8*)(&xs[buf][(b * 16 + r16) * LD + ks * 32 + kq]);
-#pragma unroll
-      for (int b = 0; b < MB; ++b)
-#pragma unroll
-        for (int r = 0; r < RT; ++r)
-          acc[b][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[b], bw[ks][r], acc[b][r], 0, 0, 0);
-    }
-    if (kt + 2 < nk) fetch_w(kt + 2, bw);
-    if (kt + 1 < nk) stash_x(buf ^ 1);  // the other buffer was last read before the previous barrier
-    __syncthreads();
-  };
-
-  fetch_x(0);
-  fetch_w(0, bw0);
-  stash_x(0);
-  if (nk > 1) fetch_w(1, bw1);
-  __syncthreads();
-  for (int kt = 0; kt < nk; kt += 2) {
-    tile(kt, 0, bw0);
-    if (kt + 1 < nk) tile(kt + 1, 1, bw1);
-  }
-#pragma unroll
-  for (int b = 0; b < MB; ++b)
-#pragma unroll
-    for (int r = 0; r < RT; ++r)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int m = b * 16 + 4 * (lane / 16) + j, n = n0 + r * 16 + lane % 16;
-        if (m < M && n < N) {
-          if (out_is_f32)
-            ((float*)out)[((size_t)blockIdx.y * M + m) * N + n] = acc[b][r][j];
-          else
-            ((bf16*)out)[(size_t)m * N + n] = (bf16)acc[b][r][j];
-        }
-      }
-}
-
-template <int MB, int RT, int WAVES, int BK, bool GATED = false>
-static void launch_xlds(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K, int slices,
-                        hipStream_t stream) {
-  const int k_slice = ((K + slices - 1) / slices + 31) / 32 * 32;
-  const int rows = WAVES * RT * 16;
-  gemm_xlds_kernel<MB, RT, WAVES, BK, GATED><<<dim3((N + rows - 1) / rows, slices), WAVES * SYN_WAVE, 0, stream>>>(
-      x, w, out, out_is_f32, M, N, K, k_slice);
-}
-
-// ------------------------------------------------------------------ tiled, bf16, large M
+// ------------------------------------------------------------------ tiled, bf16
 // Block tile BM (m) x BN (n) x BK (k); WM x WN waves, each (BM/WM) x (BN/WN) of MFMA 32x32x16 tiles.
 // MFMA 32x32x16: A = x rows, B = W rows; lane holds row lane%32, k = 8*(lane/32) .. +8;
 // D[m = 8*(j/4) + 4*(lane/32) + j%4][n = lane%32], j = 0..15.
 // LDS tiles are double-buffered: while one k-tile is multiplied the next is on its way from memory
 // into registers, and is stored into the other buffer before the barrier.
-template <int BM, int BN, int BK, int WM, int WN, bool KTAIL>
+template <int BM, int BN, int BK, int WM, int WN, bool KTAIL, bool GATED>
 __global__ void __launch_bounds__(64 * WM * WN)
 gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
-                  int M, int N, int K) {
+                  int M, int N, int K, int k_slice) {
+  constexpr bool FEW = BM <= 64;                     // the variants for few rows of x: slices of K, absent rows
   constexpr int THREADS = 64 * WM * WN;              // WM x WN waves
   constexpr int LD = BK + 8;                         // padded row of the LDS tiles, in bf16 elements
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;  // 32x32 tiles a wave holds in m and n
@@ -335,10 +212,16 @@ gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* 
 
   // global -> LDS: thread t moves chunk t % CPR of rows t / CPR + RPP * i
   const int lrow = tid / CPR, lchunk = (tid % CPR) * 8;
+  // rows of x beyond M are not fetched (their LDS rows hold zeros and their results are never
+  // stored): with few rows this spares most of the traffic for x
   const bf16* xg[XL];
   const bf16* wg[WL];
+  bool xin[XL];
 #pragma unroll
-  for (int i = 0; i < XL; ++i) xg[i] = x + (size_t)min(m0 + lrow + RPP * i, M - 1) * K + lchunk;
+  for (int i = 0; i < XL; ++i) {
+    xin[i] = !FEW || m0 + lrow + RPP * i < M;
+    xg[i] = x + (size_t)min(m0 + lrow + RPP * i, M - 1) * (GATED ? 2 * K : K) + lchunk;
+  }
 #pragma unroll
   for (int i = 0; i < WL; ++i) wg[i] = w + (size_t)min(n0 + lrow + RPP * i, N - 1) * K + lchunk;
 
@@ -350,19 +233,37 @@ gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* 
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  const int nk = (K + BK - 1) / BK;
-  bf16x8 rx[XL], rw[WL];
+  // blockIdx.y = which slice of K (k_slice elements, a multiple of 32) this workgroup sums, as in gemm_skinny
+  const int k_begin = FEW ? (int)blockIdx.y * k_slice : 0, k_end = FEW ? min(K, k_begin + k_slice) : K;
+  const int nk = (k_end - k_begin + BK - 1) / BK;
+  bf16x8 rx[XL], ru[GATED ? XL : 1], rw[WL];
   auto fetch = [&](int kt) {
     // K is a multiple of 8: a chunk lies inside or outside as a whole
-    const bool kin = !KTAIL || kt * BK + lchunk < K;
+    const int k = k_begin + kt * BK;
+    const bool kin = !KTAIL || k + lchunk < k_end;
 #pragma unroll
-    for (int i = 0; i < XL; ++i) rx[i] = kin ? *(const bf16x8*)(xg[i] + (size_t)kt * BK) : zero;
+    for (int i = 0; i < XL; ++i) {
+      rx[i] = (kin && xin[i]) ? *(const bf16x8*)(xg[i] + k) : zero;
+      if constexpr (GATED) ru[i] = (kin && xin[i]) ? *(const bf16x8*)(xg[i] + K + k) : zero;
+    }
 #pragma unroll
-    for (int i = 0; i < WL; ++i) rw[i] = kin ? *(const bf16x8*)(wg[i] + (size_t)kt * BK) : zero;
+    for (int i = 0; i < WL; ++i) rw[i] = kin ? *(const bf16x8*)(wg[i] + k) : zero;
   };
   auto stash = [&](int buf) {
     bf16* xs = smem + buf * (BM + BN) * LD;
     bf16* ws = xs + BM * LD;
+    if constexpr (GATED) {
+      // x = silu(g) * u of the fused [g | u] row, in 32-bit, rounded once
+#pragma unroll
+      for (int i = 0; i < XL; ++i)
+        if (xin[i]) {  // rows beyond M stay zero and cost no exponentials
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float g = (float)rx[i][e];
+            rx[i][e] = (bf16)(g / (1.f + expf(-g)) * (float)ru[i][e]);
+          }
+        }
+    }
 #pragma unroll
     for (int i = 0; i < XL; ++i) *(bf16x8*)(xs + (lrow + RPP * i) * LD + lchunk) = rx[i];
 #pragma unroll
@@ -404,16 +305,18 @@ gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* 
         const int n = n0 + wn + j * 32 + lane % 32;
         if (m < M && n < N) {
           if (out_is_f32)
-            ((float*)out)[(size_t)m * N + n] = acc[i][j][e];
+            ((float*)out)[((size_t)(FEW ? blockIdx.y : 0) * M + m) * N + n] = acc[i][j][e];
           else
             ((bf16*)out)[(size_t)m * N + n] = (bf16)acc[i][j][e];
         }
       }
 }
 
-template <int BM, int BN, int BK, int WM, int WN>
+template <int BM, int BN, int BK, int WM, int WN, bool GATED = false>
 static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
-                        hipStream_t stream) {
+                        hipStream_t stream, int slices = 1) {
+  SYN_CHECK(slices == 1 || BM <= 64, "gemm: slices of K only with the tiles for few rows");
+  const int k_slice = ((K + slices - 1) / slices + 31) / 32 * 32;
   const int tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM;
   const int PM = tiles_m < 8 ? tiles_m : 8, PN = 4;
   const int panels = ((tiles_m + PM - 1) / PM) * ((tiles_n + PN - 1) / PN);
@@ -421,18 +324,20 @@ static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32,
   const size_t lds = (size_t)2 * (BM + BN) * (BK + 8) * sizeof(bf16);
   static bool raised = false;
   if (lds > 65536 && !raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, WM, WN, false>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, WM, WN, false, GATED>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, WM, WN, true>,
+      e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, WM, WN, true, GATED>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     SYN_CHECK(e == hipSuccess, "gemm: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
     raised = true;
   }
-  if (K % BK == 0)
-    gemm_tiled_kernel<BM, BN, BK, WM, WN, false><<<grid, 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K);
+  if (K % BK == 0 && k_slice % BK == 0)
+    gemm_tiled_kernel<BM, BN, BK, WM, WN, false, GATED>
+        <<<dim3(grid, slices), 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
   else
-    gemm_tiled_kernel<BM, BN, BK, WM, WN, true><<<grid, 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K);
+    gemm_tiled_kernel<BM, BN, BK, WM, WN, true, GATED>
+        <<<dim3(grid, slices), 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
   return 0;
 }
 
@@ -465,41 +370,26 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   }
   const bf16* xb = (const bf16*)x;
   const bf16* wb = (const bf16*)w;
-  // x through LDS (waves on different rows of W) for the widest products and for every product
-  // that is cut along K; measured against gemm_skinny at M = 8, 16 and 64 for the shapes of an 8B model
-  if (M <= 64 && (slices > 1 || N > 32768)) {
-    const int mb = (M + 15) / 16;
-    if (mb == 1) launch_xlds<1, 1, 4, 128>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else if (mb == 2) launch_xlds<2, 1, 4, 128>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else if (mb == 3) launch_xlds<3, 1, 4, 128>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else launch_xlds<4, 1, 4, 128>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    SYN_LAUNCH_CHECK("gemm_xlds");
-    return 0;
-  }
-  // gemm_skinny: rows of W a workgroup owns, waves and unroll by (M, N), from sweeps at the shapes of
-  // an 8B model: few rows (many workgroups) win up to M = 16; more rows amortise x beyond that
-  if (M <= 16) {
+  // From sweeps at the shapes of an 8B model (N = 4096 .. 151936, K = 4096 and 12288).
+  int rc = 0;
+  if (M == 1 && slices == 1) {
+    // one row: fragments of W straight from memory, K split over the waves
     if (N <= 8192) launch_skinny<1, 1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
     else launch_skinny<1, 1, 8, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
   } else if (M <= 32) {
-    if (N <= 4096) launch_skinny<2, 1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else if (N <= 8192) launch_skinny<2, 2, 8, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else launch_skinny<2, 4, 8, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-  } else if (M <= 48) {
-    launch_skinny<3, 2, 8, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    // few rows: memory-bound; small tiles (many workgroups), deep in K (long pieces of each row)
+    if (N >= 65536) rc = launch_tiled<32, 32, 256, 1, 1>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
+    else rc = launch_tiled<32, 64, 128, 1, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
   } else if (M <= 64) {
-    if (N <= 4096) launch_skinny<4, 1, 16, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else if (N <= 8192) launch_skinny<4, 2, 16, 1>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else launch_skinny<4, 4, 4, 2>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    rc = launch_tiled<64, 64, 128, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
   } else {
     // 256 x 256 tiles (8 waves) where they keep at least three quarters of the compute units busy,
     // 128 x 128 tiles (4 waves) for smaller problems
     const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-    int rc;
     if (t256 >= 192) rc = launch_tiled<256, 256, 64, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
     else rc = launch_tiled<128, 128, 64, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
-    if (rc) return rc;
   }
+  if (rc) return rc;
   SYN_LAUNCH_CHECK("gemm");
   return 0;
 }
@@ -519,11 +409,10 @@ SYN_EXPORT int syn_gemm_gated(const void* gate_up, const void* w, void* out, int
   const bf16* xb = (const bf16*)gate_up;
   const bf16* wb = (const bf16*)w;
   const int out_is_f32 = dtype == 2;
-  const int mb = (M + 15) / 16;
-  if (mb == 1) launch_xlds<1, 1, 4, 128, true>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-  else if (mb == 2) launch_xlds<2, 1, 4, 128, true>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-  else if (mb == 3) launch_xlds<3, 1, 4, 128, true>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-  else launch_xlds<4, 1, 4, 128, true>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+  int rc;
+  if (M <= 32) rc = launch_tiled<32, 64, 128, 1, 2, true>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
+  else rc = launch_tiled<64, 64, 128, 2, 2, true>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
+  if (rc) return rc;
   SYN_LAUNCH_CHECK("gemm_gated");
   return 0;
 }

@@ -141,7 +141,9 @@ def test_gemm_f32(ops, M, N, K):
     (65, 130, 104), (128, 128, 32), (200, 300, 1000), (513, 257, 4096),
     (5, 30, 20), (70, 50, 36),          # K no multiple of 8: the plain kernel takes them
     (2048, 6144, 512), (1000, 12300, 136),   # large enough for the 256 x 256 tiles with 8 waves, ragged edges
-    (8, 40000, 256), (40, 33000, 72), (64, 50000, 1000),   # wide enough for x through LDS
+    (8, 40000, 256), (40, 33000, 72), (64, 50000, 1000),   # wide
+    (1, 9000, 520), (1, 70000, 136),                       # one row: W straight from memory, K over the waves
+    (8, 70000, 264), (20, 66000, 72),                      # few rows, very wide: 32-row tiles, 256 deep
 ])
 def test_gemm_bf16(ops, out_dtype, M, N, K):
     x, w = rnd((M, K), 10, BF16), rnd((N, K), 11, BF16)
