@@ -51,9 +51,31 @@ sample_rows_kernel(const float* __restrict__ logits, const float* __restrict__ t
   const float T = temperature ? temperature[row] : 0.f;
 
   ArgBest best = {-INFINITY, -1};
-  for (int i = tid; i < V; i += blockDim.x) {
-    ArgBest c = {x[i], i};
-    best = arg_better(best, c);
+  if (V % 4 == 0 && (uintptr_t)logits % 16 == 0) {
+    // 16-byte loads, four of them in flight: the row is read once, at memory speed
+    const float4* x4 = (const float4*)x;
+    const int V4 = V / 4, step = blockDim.x;
+    for (int i0 = tid; i0 < V4; i0 += 4 * step) {
+      float4 v[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        v[q] = i0 + q * step < V4 ? x4[i0 + q * step] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int i = 4 * (i0 + q * step);
+        if (i0 + q * step < V4) {
+          best = arg_better(best, ArgBest{v[q].x, i});
+          best = arg_better(best, ArgBest{v[q].y, i + 1});
+          best = arg_better(best, ArgBest{v[q].z, i + 2});
+          best = arg_better(best, ArgBest{v[q].w, i + 3});
+        }
+      }
+    }
+  } else {
+    for (int i = tid; i < V; i += blockDim.x) {
+      ArgBest c = {x[i], i};
+      best = arg_better(best, c);
+    }
   }
   best = block_argmax(best, red_arg);
   if (!(T > 0.f)) {

@@ -452,8 +452,8 @@ def test_attention_window_edge(ops):
 
 # ----------------------------------------------------------------------------- sampling
 
-def test_sample_rows_greedy_and_ties(ops):
-    V = 1000
+@pytest.mark.parametrize("V", [1000, 999, 40004])
+def test_sample_rows_greedy_and_ties(ops, V):
     x = rnd((5, V), 70)
     x[1, 17] = x[1, 900] = 9.0           # the last of equal maxima wins
     x[2, :] = 0.0                        # all equal: the last index
