@@ -16,13 +16,15 @@ attention reads positions below the sequence's length only.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+import ctypes as C
+from dataclasses import dataclass
 
 import numpy as np
 import torch
 
+from ..kernels import runtime as rt
 from ..parts.base import KvNeed, StateNeed
-from .pages import PAGE_TOKENS, PagePool, CacheFull, CacheError, pages_for
+from .pages import PAGE_TOKENS, CacheFull, CacheError, pages_for
 
 
 @dataclass
@@ -39,22 +41,25 @@ class StateLayerView:
     state: torch.Tensor
 
 
+class _GroupPool:
+    """The page pool of one group, as the native cache keeps it."""
+
+    def __init__(self, cache, group: int, n_pages: int):
+        self._cache, self._group, self.n_pages = cache, group, n_pages
+
+    @property
+    def free_pages(self) -> int:
+        return rt.lib().syn_cache_free_pages(self._cache._h, self._group)
+
+
 @dataclass
 class _Group:
     need: KvNeed
     layers: list                      # cache-layer indices
-    pool: PagePool
+    pool: _GroupPool = None
     k: torch.Tensor = None
     v: torch.Tensor = None
     spare_page: int = 0               # a page beyond the pool that no sequence owns (padding rows write there)
-
-
-@dataclass
-class _Slot:
-    live: bool = False
-    length: int = 0
-    reserved: int = 0                 # tokens for which pages are held (>= length)
-    pages: dict = field(default_factory=dict)     # group -> list of page ids by logical page (-1: given back)
 
 
 class SequenceCache:
@@ -74,6 +79,7 @@ class SequenceCache:
         self._layer_group = {}
         self._layer_index = {}
         self._state = {}
+        self._h = None
         for i, need in enumerate(needs):
             if isinstance(need, KvNeed):
                 for gi, g in enumerate(self.groups):
@@ -81,7 +87,7 @@ class SequenceCache:
                         break
                 else:
                     gi = len(self.groups)
-                    self.groups.append(_Group(need, [], PagePool(self.n_pages)))
+                    self.groups.append(_Group(need, []))
                 self._layer_group[i] = gi
                 self._layer_index[i] = len(self.groups[gi].layers)
                 self.groups[gi].layers.append(i)
@@ -90,104 +96,96 @@ class SequenceCache:
                                              device=self.device)
             elif need is not None:
                 raise CacheError(f"cache layer {i}: unknown need {need!r}")
-        for g in self.groups:
+        if rt.lib().syn_rt_page_tokens() != PAGE_TOKENS:
+            raise RuntimeError("the runtime library was built for another page size")
+        windows = [-1 if g.need.window is None else int(g.need.window) for g in self.groups]
+        self._h = rt.lib().syn_cache_new(len(self.groups), rt.longs(windows), self.n_pages, self.max_slots,
+                                         -1 if max_positions is None else int(max_positions))
+        if not self._h:
+            raise CacheError(rt.last_error())
+        for gi, g in enumerate(self.groups):
             n, nd = len(g.layers), g.need
+            g.pool = _GroupPool(self, gi, self.n_pages)
             # zeros: what a kernel may touch beyond a sequence's end is at least a number
             g.spare_page = self.n_pages
             g.k = torch.zeros((n, self.n_pages + 1, nd.kv_heads, PAGE_TOKENS, nd.head_dim), dtype=dtype, device=self.device)
             g.v = torch.zeros((n, self.n_pages + 1, nd.kv_heads, nd.head_dim, PAGE_TOKENS), dtype=dtype, device=self.device)
-        self._slots = [_Slot() for _ in range(self.max_slots)]
-        self._free_slots = list(range(self.max_slots - 1, -1, -1))
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            rt.lib().syn_cache_delete(self._h)
+            self._h = None
+
+    @staticmethod
+    def _sid(sid) -> int:
+        if not isinstance(sid, (int, np.integer)) or isinstance(sid, bool):
+            raise CacheError(f"slot {sid!r} is not live")
+        return int(sid)
 
     # ------------------------------------------------------------------ slots
     @property
     def free_slots(self) -> int:
-        return len(self._free_slots)
+        return rt.lib().syn_cache_free_slots(self._h)
 
     @property
     def live_slots(self) -> list:
-        return [i for i, s in enumerate(self._slots) if s.live]
+        out = (C.c_int * self.max_slots)()
+        n = rt.lib().syn_cache_live_slots(self._h, out)
+        return list(out[:n])
 
     def acquire(self) -> int:
-        if not self._free_slots:
-            raise CacheFull(f"all {self.max_slots} slots are taken")
-        sid = self._free_slots.pop()
-        s = self._slots[sid]
-        s.live, s.length, s.reserved = True, 0, 0
-        s.pages = {gi: [] for gi in range(len(self.groups))}
+        sid = C.c_int()
+        rt.check(rt.lib().syn_cache_acquire(self._h, C.byref(sid)))
         for st in self._state.values():
-            st[sid].zero_()
-        return sid
+            st[sid.value].zero_()
+        return sid.value
 
     def release(self, sid: int) -> None:
-        s = self._slot(sid)
-        for gi, pages in s.pages.items():
-            self.groups[gi].pool.give_back([p for p in pages if p >= 0])
-        s.live, s.length, s.reserved, s.pages = False, 0, 0, {}
-        self._free_slots.append(sid)
-
-    def _slot(self, sid: int) -> _Slot:
-        if not isinstance(sid, (int, np.integer)) or not (0 <= sid < self.max_slots) or not self._slots[sid].live:
-            raise CacheError(f"slot {sid!r} is not live")
-        return self._slots[sid]
+        rt.check(rt.lib().syn_cache_release(self._h, self._sid(sid)))
 
     def length(self, sid: int) -> int:
-        return self._slot(sid).length
+        out = C.c_long()
+        rt.check(rt.lib().syn_cache_length(self._h, self._sid(sid), C.byref(out)))
+        return out.value
 
     # ------------------------------------------------------------------ growth
     def pages_needed(self, sid: int, n_new: int) -> int:
         """Pages of the fullest-keeping group that `reserve(sid, n_new)` would take."""
-        s = self._slot(sid)
-        return max(0, pages_for(s.length + n_new) - pages_for(s.reserved))
+        out = C.c_long()
+        rt.check(rt.lib().syn_cache_pages_needed(self._h, self._sid(sid), int(n_new), C.byref(out)))
+        return out.value
 
     def reserve(self, sid: int, n_new: int) -> None:
         """Hold pages for n_new more tokens in every group, or raise CacheFull and change nothing."""
-        s = self._slot(sid)
-        if n_new <= 0:
-            raise CacheError("a step brings at least one token for each of its sequences")
-        total = s.length + n_new
-        if self.max_positions is not None and total > self.max_positions:
-            raise CacheError(f"KV overflow: {s.length} + {n_new} tokens exceed the position range {self.max_positions}")
-        want = pages_for(total) - pages_for(s.reserved)
-        if want > 0:
-            for g in self.groups:
-                if g.pool.free_pages < want:
-                    raise CacheFull(f"{want} pages wanted, {g.pool.free_pages} of {g.pool.n_pages} free")
-            for gi, g in enumerate(self.groups):
-                s.pages[gi].extend(g.pool.take(want))
-        s.reserved = max(s.reserved, total)
+        rt.check(rt.lib().syn_cache_reserve(self._h, self._sid(sid), int(n_new)))
+
+    def reserve_step(self, sids: list, counts: list) -> None:
+        """All pages that a step's sequences need, or CacheFull and nothing changed."""
+        sids = [self._sid(s) for s in sids]
+        rt.check(rt.lib().syn_cache_reserve_step(self._h, len(sids), rt.ints(sids), rt.longs([int(c) for c in counts])))
 
     def commit(self, sid: int, n_new: int) -> None:
         """The step has written n_new tokens; windows give back the pages that fell out of reach."""
-        s = self._slot(sid)
-        if s.length + n_new > s.reserved:
-            raise CacheError("commit without reserve")
-        s.length += n_new
-        for gi, g in enumerate(self.groups):
-            w = g.need.window
-            if w is None:
-                continue
-            # the next query sits at position `length`; it sees keys > length - w
-            first_needed = max(0, s.length - w + 1) // PAGE_TOKENS
-            pages = s.pages[gi]
-            gone = [p for p in pages[:first_needed] if p >= 0]
-            if gone:
-                g.pool.give_back(gone)
-                for i in range(first_needed):
-                    pages[i] = -1
+        rt.check(rt.lib().syn_cache_commit(self._h, self._sid(sid), int(n_new)))
 
     # ------------------------------------------------------------------ what a step needs
+    def table_width(self, gi: int, sids: list) -> int:
+        """Logical pages of the longest of the sequences (at least 1)."""
+        sids = [self._sid(s) for s in sids]
+        out = C.c_int()
+        rt.check(rt.lib().syn_cache_table_width(self._h, gi, rt.ints(sids), len(sids), C.byref(out)))
+        return out.value
+
     def page_table(self, gi: int, sids: list, width: int | None = None) -> np.ndarray:
         """int32 [len(sids), width]: page of each logical page of each sequence (0 where none)."""
-        rows = [self._slot(sid).pages[gi] for sid in sids]
-        w = max([len(r) for r in rows] + [1])
+        w = self.table_width(gi, sids)
         if width is not None:
             if width < w:
                 raise CacheError(f"page table width {width} is less than {w}")
             w = width
         out = np.zeros((len(sids), w), dtype=np.int32)
-        for i, r in enumerate(rows):
-            out[i, :len(r)] = [max(p, 0) for p in r]
+        sids = [self._sid(s) for s in sids]
+        rt.check(rt.lib().syn_cache_page_table(self._h, gi, rt.ints(sids), len(sids), w, out.ctypes.data))
         return out
 
     def layer_view(self, i: int):
@@ -202,19 +200,7 @@ class SequenceCache:
     # ------------------------------------------------------------------ invariants
     def check(self) -> None:
         """No slot or page lost, held twice or free twice."""
-        free = set(self._free_slots)
-        if len(free) != len(self._free_slots):
-            raise CacheError("a slot is in the free list twice")
-        for i, s in enumerate(self._slots):
-            if s.live == (i in free):
-                raise CacheError(f"slot {i} is {'both live and free' if s.live else 'lost'}")
-        for gi, g in enumerate(self.groups):
-            g.pool.check()
-            held = [p for s in self._slots if s.live for p in s.pages[gi] if p >= 0]
-            if len(held) != len(set(held)):
-                raise CacheError(f"group {gi}: a page is held by two sequences")
-            if len(held) + g.pool.free_pages != g.pool.n_pages:
-                raise CacheError(f"group {gi}: {g.pool.n_pages - len(held) - g.pool.free_pages} pages lost")
+        rt.check(rt.lib().syn_cache_check(self._h))
 
     def bytes_per_token(self) -> int:
         el = torch.empty(0, dtype=self.dtype).element_size()

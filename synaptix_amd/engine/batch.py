@@ -16,29 +16,28 @@ The reference has such per-row device arrays only for its graph decode
 """
 from __future__ import annotations
 
+import ctypes as C
+
 import numpy as np
 import torch
 
 from ..kernels import ops
+from ..kernels import runtime as rt
+
+_NAMES = ("tokens", "tok_seq", "tok_pos", "seq_start", "seq_past", "seq_len", "seq_slot", "want")
 
 
 class StepLayout:
-    """Offsets of the arrays inside the one int32 buffer, for given counts."""
+    """Offsets of the arrays inside the one int32 buffer, for given counts (the native runtime
+    lays the buffer out and fills it; this is its map)."""
 
     def __init__(self, n_tokens: int, n_seqs: int, n_want: int, table_widths: list):
-        self.N, self.B, self.n_want, self.widths = n_tokens, n_seqs, n_want, list(table_widths)
-        off = 0
-        self.off = {}
-        for name, n in (("tokens", n_tokens), ("tok_seq", n_tokens), ("tok_pos", n_tokens),
-                        ("seq_start", n_seqs + 1), ("seq_past", n_seqs), ("seq_len", n_seqs),
-                        ("seq_slot", n_seqs), ("want", n_want)):
-            self.off[name] = (off, n)
-            off += n
-        self.table_off = []
-        for w in self.widths:
-            self.table_off.append((off, n_seqs * w))
-            off += n_seqs * w
-        self.total = max(off, 1)
+        self.N, self.B, self.n_want, self.widths = n_tokens, n_seqs, n_want, [int(w) for w in table_widths]
+        offsets = (C.c_long * (len(_NAMES) + len(self.widths)))()
+        self.total = rt.lib().syn_step_layout(n_tokens, n_seqs, n_want, len(self.widths), rt.ints(self.widths), offsets)
+        counts = (n_tokens, n_tokens, n_tokens, n_seqs + 1, n_seqs, n_seqs, n_seqs, n_want)
+        self.off = {name: (offsets[i], n) for i, (name, n) in enumerate(zip(_NAMES, counts))}
+        self.table_off = [(offsets[len(_NAMES) + g], n_seqs * w) for g, w in enumerate(self.widths)]
 
 
 class StepContext:
@@ -71,24 +70,14 @@ class StepContext:
         return t
 
 
-def fill_host_buffer(layout: StepLayout, host: np.ndarray, token_lists, past, slots, want_rows, tables) -> None:
-    """Write every array of the step into `host` (int32, at least layout.total long)."""
-    o = layout.off
-    pos = 0
-    starts = [0]
-    for i, toks in enumerate(token_lists):
-        n = len(toks)
-        host[o["tokens"][0] + pos:o["tokens"][0] + pos + n] = toks
-        host[o["tok_seq"][0] + pos:o["tok_seq"][0] + pos + n] = i
-        host[o["tok_pos"][0] + pos:o["tok_pos"][0] + pos + n] = np.arange(past[i], past[i] + n, dtype=np.int32)
-        pos += n
-        starts.append(pos)
-    B = layout.B
-    host[o["seq_start"][0]:o["seq_start"][0] + B + 1] = starts
-    host[o["seq_past"][0]:o["seq_past"][0] + B] = past
-    host[o["seq_len"][0]:o["seq_len"][0] + B] = [p + len(t) for p, t in zip(past, token_lists)]
-    host[o["seq_slot"][0]:o["seq_slot"][0] + B] = slots
-    if layout.n_want:
-        host[o["want"][0]:o["want"][0] + layout.n_want] = want_rows
-    for (off, n), w, tab in zip(layout.table_off, layout.widths, tables):
-        host[off:off + n] = tab.reshape(-1)
+def fill_host_buffer(layout: StepLayout, host: np.ndarray, cache, slots, tokens_flat: np.ndarray, counts,
+                     want_rows) -> None:
+    """Write every array of the step into `host` (int32, at least layout.total long): positions
+    and page tables come from the cache's own state."""
+    if host.size < layout.total or host.dtype != np.int32:
+        raise ValueError("the step's host buffer is too small")
+    tokens_flat = np.ascontiguousarray(tokens_flat, dtype=np.int32)
+    want = np.ascontiguousarray(want_rows, dtype=np.int32)
+    rt.check(rt.lib().syn_step_fill(cache._h, len(slots), rt.ints([int(s) for s in slots]),
+                                    rt.longs([int(c) for c in counts]), tokens_flat.ctypes.data, want.size,
+                                    want.ctypes.data, len(layout.widths), rt.ints(layout.widths), host.ctypes.data))

@@ -147,24 +147,18 @@ class Engine:
                     if not (0 <= p < token_lists[i].size):
                         raise StepError(f"slot {slots[i]}: wanted place {p} is outside its {token_lists[i].size} tokens")
                     want_rows.append(int(starts[i]) + int(p))
-        # all pages of the step, or none
-        need = sum(self.cache.pages_needed(s, t.size) for s, t in zip(slots, token_lists))
-        for g in self.cache.groups:
-            if g.pool.free_pages < need:
-                raise CacheFull(f"the step needs {need} more pages, {g.pool.free_pages} of {g.pool.n_pages} are free")
-        for s, t in zip(slots, token_lists):
-            self.cache.reserve(s, t.size)
-
-        tables = [self.cache.page_table(gi, slots) for gi in range(len(self.cache.groups))]
-        layout = StepLayout(int(starts[-1]), len(entries), len(want_rows), [t.shape[1] for t in tables])
-        dev = self._upload(layout, token_lists, past, slots, want_rows, tables)
-        ctx = StepContext(layout, dev, self.dtype, slots, past, [t.size for t in token_lists], self._scratch)
+        counts = [int(t.size) for t in token_lists]
+        self.cache.reserve_step(slots, counts)            # all pages of the step, or none
+        widths = [self.cache.table_width(gi, slots) for gi in range(len(self.cache.groups))]
+        layout = StepLayout(int(starts[-1]), len(entries), len(want_rows), widths)
+        dev = self._upload(layout, slots, np.concatenate(token_lists), counts, want_rows)
+        ctx = StepContext(layout, dev, self.dtype, slots, past, counts, self._scratch)
         return ctx, len(want_rows)
 
-    def _upload(self, layout, token_lists, past, slots, want_rows, tables) -> torch.Tensor:
+    def _upload(self, layout, slots, tokens_flat, counts, want_rows) -> torch.Tensor:
         """The step's arrays on the device, through a pinned buffer and one asynchronous copy."""
         i, host, dev = self._buffers(layout.total)
-        fill_host_buffer(layout, host.numpy(), token_lists, past, slots, want_rows, tables)
+        fill_host_buffer(layout, host.numpy(), self.cache, slots, tokens_flat, counts, want_rows)
         dev[:layout.total].copy_(host[:layout.total], non_blocking=True)
         self._copied[i] = torch.cuda.Event()
         self._copied[i].record()

@@ -15,10 +15,13 @@ Captured are this package's kernels and torch's allocations only; no memset node
 """
 from __future__ import annotations
 
+import ctypes as C
+
 import numpy as np
 import torch
 
 from ..kernels import ops
+from ..kernels import runtime as rt
 from .batch import StepLayout, StepContext
 
 
@@ -51,33 +54,15 @@ class DecodeRunner:
         self.spare = [g.spare_page for g in engine.cache.groups]
 
     def _fill(self, host: np.ndarray, slots, tokens, temps, uniforms):
-        lay, cache, R, B = self.layout, self.engine.cache, self.rows, len(slots)
-        o = lay.off
-        past = [cache.length(s) for s in slots]
-        host[o["tokens"][0]:o["tokens"][0] + R] = 0
-        host[o["tokens"][0]:o["tokens"][0] + B] = tokens
-        host[o["tok_seq"][0]:o["tok_seq"][0] + R] = np.arange(R, dtype=np.int32)
-        pos = np.zeros(R, dtype=np.int32)
-        pos[:B] = past
-        host[o["tok_pos"][0]:o["tok_pos"][0] + R] = pos
-        host[o["seq_start"][0]:o["seq_start"][0] + R + 1] = np.arange(R + 1, dtype=np.int32)
-        host[o["seq_past"][0]:o["seq_past"][0] + R] = pos
-        host[o["seq_len"][0]:o["seq_len"][0] + R] = pos + 1
-        sl = np.full(R, -1, dtype=np.int32)
-        sl[:B] = slots
-        host[o["seq_slot"][0]:o["seq_slot"][0] + R] = sl
-        host[o["want"][0]:o["want"][0] + R] = np.arange(R, dtype=np.int32)
-        for gi, ((off, n), w) in enumerate(zip(lay.table_off, lay.widths)):
-            tab = np.full((R, w), self.spare[gi], dtype=np.int32)
-            if B:
-                tab[:B] = cache.page_table(gi, slots, width=w)
-            host[off:off + n] = tab.reshape(-1)
-        f = host[lay.total:lay.total + 2 * R].view(np.float32)
-        f[:] = 0.0
+        """The padded tables of the step and, behind them, temperatures and uniform numbers."""
+        B = len(slots)
+        t = u = None
         if temps is not None:
-            f[:B] = temps
-            f[R:R + B] = uniforms
-        return past
+            t = (C.c_float * B)(*[float(x) for x in temps])
+            u = (C.c_float * B)(*[float(x) for x in uniforms])
+        rt.check(rt.lib().syn_decode_fill(self.engine.cache._h, self.rows, B, rt.ints([int(s) for s in slots]),
+                                          rt.ints([int(x) for x in tokens]), len(self.widths), rt.ints(self.widths),
+                                          rt.ints(self.spare), t, u, host.ctypes.data))
 
     def _forward(self, ctx):
         eng = self.engine
@@ -97,7 +82,7 @@ class DecodeRunner:
         self.turn ^= 1
         if self.copied[i] is not None:
             self.copied[i].synchronize()
-        past = self._fill(self.host[i].numpy(), slots, tokens, temps, uniforms)
+        self._fill(self.host[i].numpy(), slots, tokens, temps, uniforms)
         self.dev.copy_(self.host[i], non_blocking=True)
         self.copied[i] = torch.cuda.Event()
         self.copied[i].record()

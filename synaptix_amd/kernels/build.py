@@ -1,8 +1,10 @@
-"""Compile the HIP sources for gfx950 with hipcc and load them through ctypes.
+"""Compile the native sources and load them through ctypes.
 
-Two kinds of library:
-  core            every kernel whose sizes are run-time parameters
-  attn_hd<N>      the bf16 MFMA attention kernels, compiled for one head size
+Three kinds of library:
+  core            every kernel whose sizes are run-time parameters (hipcc, gfx950)
+  attn_hd<N>      the bf16 MFMA attention kernels, compiled for one head size (hipcc, gfx950)
+  runtime         host code only: cache bookkeeping, step tables, the sampler's random stream
+                  (the host C++ compiler)
 
 A library is built at its first use if no built file matches the sources, which is how the
 reference treats its kernels too (compiled at first use; crates/synaptix-kernels-cuda/src/kernels/compile.rs).
@@ -25,7 +27,9 @@ ARCH = "gfx950"
 # packed 32-bit float instructions are switched off for all device code
 FLAGS = ["-O3", f"--offload-arch={ARCH}", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden"]
 CORE_SOURCES = ["elementwise.hip", "sampling.hip", "gemm.hip", "attention_f32.hip"]
+RUNTIME_SOURCES = ["runtime.cpp"]
 ATTN_SOURCE = "attention_bf16.hip"
 HEADERS = ["common.h"]
 
@@ -45,6 +49,14 @@ def find_hipcc() -> str:
             return cand
     raise KernelBuildError("hipcc not found (looked at $HIPCC, PATH and $ROCM_PATH/bin); "
                            "the kernels of synaptix_amd cannot be built")
+
+
+def find_host_compiler() -> str:
+    for cand in (os.environ.get("CXX"), "g++", "c++", "clang++"):
+        path = shutil.which(cand) if cand else None
+        if path:
+            return path
+    return find_hipcc()      # it compiles plain C++ as well
 
 
 def lib_dirs() -> list:
@@ -67,16 +79,19 @@ def _writable_dir() -> str:
 
 
 def _digest(sources, defines) -> str:
+    host = list(sources) == RUNTIME_SOURCES
     h = hashlib.sha256()
-    for name in list(sources) + HEADERS:
+    for name in list(sources) + ([] if host else HEADERS):
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(name.encode())
             h.update(f.read())
-    h.update(" ".join(FLAGS + list(defines)).encode())
+    h.update(" ".join((HOST_FLAGS if host else FLAGS) + list(defines)).encode())
     return h.hexdigest()[:16]
 
 
 def _spec(name: str):
+    if name == "runtime":
+        return RUNTIME_SOURCES, []
     if name == "core":
         return CORE_SOURCES, []
     if name.startswith("attn_hd"):
@@ -107,9 +122,14 @@ def compile_library(name: str, quiet: bool = False) -> str:
     out_dir = _writable_dir()
     so = os.path.join(out_dir, f"libsynaptix_{name}.so")
     tmp_so = f"{so}.{os.getpid()}.tmp"
-    cmd = [find_hipcc()] + FLAGS + defines + [os.path.join(CSRC, s) for s in sources] + ["-o", tmp_so]
+    paths = [os.path.join(CSRC, s) for s in sources]
+    if name == "runtime":
+        cmd = [find_host_compiler()] + HOST_FLAGS + paths + ["-o", tmp_so]
+    else:
+        cmd = [find_hipcc()] + FLAGS + defines + paths + ["-o", tmp_so]
     if not quiet:
-        _say(f"compiling {os.path.basename(so)} for {ARCH} ({len(sources)} source file(s)) ...")
+        target = "the host" if name == "runtime" else ARCH
+        _say(f"compiling {os.path.basename(so)} for {target} ({len(sources)} source file(s)) ...")
     t0 = time.time()
     proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, cwd=out_dir)
     done = threading.Event()
@@ -128,7 +148,7 @@ def compile_library(name: str, quiet: bool = False) -> str:
             os.remove(tmp_so)
         except OSError:
             pass
-        raise KernelBuildError(f"hipcc failed for {name} (exit {proc.returncode}):\n{log}")
+        raise KernelBuildError(f"{os.path.basename(cmd[0])} failed for {name} (exit {proc.returncode}):\n{log}")
     os.replace(tmp_so, so)
     with open(so + ".digest", "w") as f:
         f.write(digest)
@@ -154,14 +174,17 @@ def load_library(name: str) -> ctypes.CDLL:
             lib = ctypes.CDLL(so)
         except OSError as e:
             raise KernelBuildError(f"cannot load {so}: {e}") from None
-        lib.syn_last_error.restype = ctypes.c_char_p
+        if name == "runtime":
+            lib.syn_rt_last_error.restype = ctypes.c_char_p
+        else:
+            lib.syn_last_error.restype = ctypes.c_char_p
         _LOADED[name] = lib
         return lib
 
 
 def build_all(head_dims=(16, 32, 64, 128)) -> list:
-    """Compile the core library and the attention library of each head size, in parallel."""
-    names = ["core"] + [f"attn_hd{h}" for h in head_dims]
+    """Compile the runtime, the core library and the attention library of each head size, in parallel."""
+    names = ["runtime", "core"] + [f"attn_hd{h}" for h in head_dims]
     results, errors = {}, []
 
     def work(n):

@@ -191,7 +191,7 @@ class CpuEngine(Engine):
     def _require_gpu(self):
         pass
 
-    def _upload(self, layout, token_lists, past, slots, want_rows, tables):
+    def _upload(self, layout, slots, tokens_flat, counts, want_rows):
         host = np.zeros(layout.total, dtype=np.int32)
-        fill_host_buffer(layout, host, token_lists, past, slots, want_rows, tables)
+        fill_host_buffer(layout, host, self.cache, slots, tokens_flat, counts, want_rows)
         return torch.from_numpy(host)

@@ -34,10 +34,9 @@ def one_sequence_ctx(cache, slot, n_new, dtype):
     from synaptix_amd.engine.batch import StepLayout, StepContext, fill_host_buffer
     past = cache.length(slot)
     cache.reserve(slot, n_new)
-    tables = [cache.page_table(g, [slot]) for g in range(len(cache.groups))]
-    layout = StepLayout(n_new, 1, 0, [t.shape[1] for t in tables])
+    layout = StepLayout(n_new, 1, 0, [cache.table_width(g, [slot]) for g in range(len(cache.groups))])
     host = np.zeros(layout.total, dtype=np.int32)
-    fill_host_buffer(layout, host, [np.zeros(n_new, dtype=np.int64)], [past], [slot], [], tables)
+    fill_host_buffer(layout, host, cache, [slot], np.zeros(n_new, dtype=np.int32), [n_new], [])
     return StepContext(layout, torch.from_numpy(host).to(DEV), dtype, [slot], [past], [n_new], {})
 
 
