@@ -31,9 +31,12 @@ class PagePool:
         self._h = rt.lib().syn_pool_new(n_pages)
 
     def __del__(self):
-        if getattr(self, "_h", None):
-            rt.lib().syn_pool_delete(self._h)
-            self._h = None
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            try:
+                rt.lib().syn_pool_delete(h)
+            except Exception:       # the interpreter is shutting down; the process's memory goes with it
+                pass
 
     @property
     def free_pages(self) -> int:

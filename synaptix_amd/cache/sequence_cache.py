@@ -112,9 +112,12 @@ class SequenceCache:
             g.v = torch.zeros((n, self.n_pages + 1, nd.kv_heads, nd.head_dim, PAGE_TOKENS), dtype=dtype, device=self.device)
 
     def __del__(self):
-        if getattr(self, "_h", None):
-            rt.lib().syn_cache_delete(self._h)
-            self._h = None
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            try:
+                rt.lib().syn_cache_delete(h)
+            except Exception:       # the interpreter is shutting down; the process's memory goes with it
+                pass
 
     @staticmethod
     def _sid(sid) -> int:

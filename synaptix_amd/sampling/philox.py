@@ -23,9 +23,12 @@ class Philox4x32:
         self._h = rt.lib().syn_philox_new(int(seed) & 0xFFFFFFFFFFFFFFFF)
 
     def __del__(self):
-        if getattr(self, "_h", None):
-            rt.lib().syn_philox_delete(self._h)
-            self._h = None
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            try:
+                rt.lib().syn_philox_delete(h)
+            except Exception:       # the interpreter is shutting down; the process's memory goes with it
+                pass
 
     def next_u32(self) -> int:
         return rt.lib().syn_philox_next_u32(self._h)

@@ -28,7 +28,7 @@ TINY_C = dict(num_hidden_layers=2, hidden_size=120, num_attention_heads=6, num_k
               intermediate_size=200, vocab_size=777, rope_theta=5e5, rms_norm_eps=3e-6, max_position_embeddings=1024,
               tie_word_embeddings=False, eos_token_id=None, bos_token_id=None)
 # A middle-sized one: wide enough that the engine takes the kernels which the tiny ones never reach
-# (partial sums over slices of K, x through LDS, the large GEMM tiles), still seconds on the CPU.
+# (partial sums over slices of K, the deep tiles for wide products, the large GEMM tiles), still seconds on the CPU.
 MID_D = dict(num_hidden_layers=2, hidden_size=2048, num_attention_heads=16, num_key_value_heads=4, head_dim=128,
              intermediate_size=2560, vocab_size=33024, rope_theta=1e6, rms_norm_eps=1e-6, max_position_embeddings=2048,
              tie_word_embeddings=True, eos_token_id=None, bos_token_id=None)

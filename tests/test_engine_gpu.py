@@ -96,7 +96,7 @@ def test_batch_rows_do_not_depend_on_their_neighbours():
 
 def test_middle_sized_model_reaches_the_large_kernels():
     """Hidden 2048, head size 128, vocabulary 33024: prompts of hundreds of tokens take the tiled GEMM,
-    single tokens the products cut along K and the wide output product with x through LDS."""
+    single tokens the products cut along K and the wide output product on its deep tiles."""
     name, dtype = "D", "bfloat16"
     V = CONFIGS[name]["vocab_size"]
     reqs = [random_tokens(V, n, 700 + n) for n in (300, 130, 65)]
