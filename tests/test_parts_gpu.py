@@ -237,3 +237,168 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
         tolerance = 1e-4 if dtype == "float32" else 5e-2
         assert (torch.cat(got[0]) - whole[:7]).abs().max() <= tolerance
         assert (torch.cat(got[1]) - whole[7:]).abs().max() <= tolerance
+
+
+# ----------------------------------------------------------------------------- more toy parts
+def test_toy_position_encoding_plugs_into_attention():
+    """Another position encoding, defined here: angles that grow linearly with the index of the
+    pair, on the first 8 of 16 dims.  The mixer only asks its position part for tables."""
+    from synaptix_amd.parts import GqaAttention, Position
+    from synaptix_amd.cache import SequenceCache
+
+    class LinearFrequencies(Position):
+        capacity = 128
+
+        def __init__(self, rotary_dim):
+            self.rotary_dim = rotary_dim
+
+        def host(self):
+            ang = torch.arange(self.capacity, dtype=F32)[:, None] * (0.05 * (1 + torch.arange(self.rotary_dim // 2, dtype=F32)))[None, :]
+            return torch.cos(ang), torch.sin(ang)
+
+        def tables(self, device):
+            c, s = self.host()
+            return c.to(device), s.to(device)
+
+    H, S, nh, nkv, hd, rot = 24, 40, 2, 1, 16, 8
+    pos = LinearFrequencies(rot)
+    for dtype in (F32, BF16):
+        att = GqaAttention("a.", H, nh, nkv, hd, position=pos)
+        w = {n: rnd(s.shape, 40 + i, 0.4).to(dtype) for i, (n, s) in enumerate(att.tensor_specs().items())}
+        att.load(lambda name: w[name].to(DEV))
+        x = rnd((S, H), 50).to(dtype)
+        xf = x.float()
+        q = (xf @ w["a.q_proj.weight"].float().T).view(S, nh, hd)
+        k = (xf @ w["a.k_proj.weight"].float().T).view(S, nkv, hd)
+        v = (xf @ w["a.v_proj.weight"].float().T).view(S, nkv, hd)
+        cos, sin = pos.host()
+        q = torch.cat([P.apply_rope(q[..., :rot], cos, sin, range(S)), q[..., rot:]], -1)
+        k = torch.cat([P.apply_rope(k[..., :rot], cos, sin, range(S)), k[..., rot:]], -1)
+        want = P.attention(q, k, v, 1 / math.sqrt(hd), list(range(S))).reshape(S, nh * hd) @ w["a.o_proj.weight"].float().T
+        cache = SequenceCache([att.cache_need()], 128, 1, dtype, DEV)
+        slot = cache.acquire()
+        got = []
+        for lo, hi in [(0, 33)] + [(i, i + 1) for i in range(33, S)]:
+            ctx = one_sequence_ctx(cache, slot, hi - lo, dtype)
+            d = att.forward(x[lo:hi].to(DEV), ctx, cache.layer_view(0))
+            got.append(d.sum(0) if d.dim() == 3 else d)
+            cache.commit(slot, hi - lo)
+        err = (torch.cat(got).cpu() - want).abs().max()
+        assert err <= (2e-4 if dtype == F32 else 4e-2) * max(1.0, float(want.abs().max())), float(err)
+
+
+def test_toy_feed_forward_with_routing_registers_builds_and_steps(tmp_path):
+    """A feed-forward with routing, defined here: a 32-bit router picks one of three gated MLPs
+    for each token and scales its output by the router's probability.  Registered, built from its
+    own config.json, loaded and stepped without a change to the package; the logits must equal a
+    plain statement of the same model and must not depend on the cut of the tokens into steps."""
+    from dataclasses import dataclass, asdict
+    import json
+    from synaptix_amd import register_architecture, Engine
+    from synaptix_amd.models import DecoderModel, LayerRun, TokenEmbedding, OutputHead
+    from synaptix_amd.parts import FeedForward, RmsNorm, GatedMlp, PreNormBlock, GqaAttention, RotaryHalfSplit
+    from synaptix_amd.parts.linear import linear
+    from synaptix_amd.weights import TensorSpec, save_file, RandomSource
+
+    class TopOneExperts(FeedForward):
+        def __init__(self, prefix, hidden, inter, n_experts):
+            self.prefix, self.hidden = prefix, hidden
+            self.experts = [GatedMlp(f"{prefix}e{e}.", hidden, inter) for e in range(n_experts)]
+            self.router = None
+
+        def tensor_specs(self):
+            specs = {self.prefix + "router.weight": TensorSpec((len(self.experts), self.hidden))}
+            for e in self.experts:
+                specs.update(e.tensor_specs())
+            return specs
+
+        def load(self, get):
+            self.router = get(self.prefix + "router.weight")
+            for e in self.experts:
+                e.load(get)
+
+        def forward(self, h, ctx):
+            logits = linear(h, self.router, torch.float32)                 # 32-bit router
+            prob, pick = torch.softmax(logits, -1).max(-1)
+            out = torch.zeros((h.shape[0], self.hidden), dtype=torch.float32, device=h.device)
+            for e, expert in enumerate(self.experts):
+                rows = torch.nonzero(pick == e).flatten()
+                if rows.numel():
+                    d = expert.forward(h[rows].contiguous(), ctx)
+                    d = d.sum(0) if d.dim() == 3 else d
+                    out[rows] = d * prob[rows, None]
+            return out
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        vocab_size: int = 61
+        hidden_size: int = 32
+        intermediate_size: int = 56
+        n_experts: int = 3
+        max_position_embeddings: int = 64
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(**{k: d[k] for k in cls.__dataclass_fields__ if k in d})
+
+        def to_dict(self):
+            return {**asdict(self), "architectures": ["ToyRouted"]}
+
+    def build(cfg, max_positions=None):
+        H = cfg.hidden_size
+        rope = RotaryHalfSplit(1e4, 16, cfg.max_position_embeddings)
+        blocks = [PreNormBlock(RmsNorm(f"l{l}.n1", H, 1e-5), GqaAttention(f"l{l}.att.", H, 2, 1, 16, position=rope),
+                               RmsNorm(f"l{l}.n2", H, 1e-5),
+                               TopOneExperts(f"l{l}.ff.", H, cfg.intermediate_size, cfg.n_experts)) for l in range(2)]
+        return DecoderModel(cfg, TokenEmbedding("emb", cfg.vocab_size, H), blocks, [LayerRun(0, 0), LayerRun(1, 1)],
+                            RmsNorm("norm", H, 1e-5), OutputHead("head", cfg.vocab_size, H))
+
+    register_architecture("ToyRouted", ToyConfig, build)
+    cfg = ToyConfig()
+    src = RandomSource(build(cfg).tensor_specs(), 9, std=0.3)
+    # the routers are stored in 32-bit and stay so in both modes; everything else is bf16
+    tensors = {n: (src.tensor(n).float() if "router" in n else src.tensor(n)) for n in src.names()}
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    (tmp_path / "config.json").write_text(json.dumps(cfg.to_dict()))
+
+    def plain(ids):
+        t = {n: v.float() for n, v in tensors.items()}
+        x = t["emb"][ids]
+        S, cos_sin = len(ids), P.rope_tables(16, len(ids), 1e4)
+        picks = []
+        for l in range(2):
+            xn = P.rms_norm(x, t[f"l{l}.n1"], 1e-5)
+            q = (xn @ t[f"l{l}.att.q_proj.weight"].T).view(S, 2, 16)
+            k = (xn @ t[f"l{l}.att.k_proj.weight"].T).view(S, 1, 16)
+            v = (xn @ t[f"l{l}.att.v_proj.weight"].T).view(S, 1, 16)
+            q, k = P.apply_rope(q, *cos_sin, range(S)), P.apply_rope(k, *cos_sin, range(S))
+            x = x + P.attention(q, k, v, 0.25, list(range(S))).reshape(S, 32) @ t[f"l{l}.att.o_proj.weight"].T
+            hn = P.rms_norm(x, t[f"l{l}.n2"], 1e-5)
+            prob, pick = torch.softmax(hn @ t[f"l{l}.ff.router.weight"].T, -1).max(-1)
+            picks.append(pick)
+            d = torch.stack([P.swiglu_mlp(hn[i:i + 1], t[f"l{l}.ff.e{int(e)}.gate_proj.weight"],
+                                          t[f"l{l}.ff.e{int(e)}.up_proj.weight"],
+                                          t[f"l{l}.ff.e{int(e)}.down_proj.weight"])[0] for i, e in enumerate(pick)])
+            x = x + d * prob[:, None]
+        return P.rms_norm(x, t["norm"], 1e-5) @ t["head"].T, picks
+
+    ids = [3, 17, 44, 9, 60, 21, 5, 38, 12, 50, 7]
+    want, picks = plain(ids)
+    assert len(set(int(p) for p in torch.cat(picks))) == 3          # every expert is used
+    eng = Engine.load(str(tmp_path), dtype="float32", max_tokens=128, max_slots=2)
+    a = eng.acquire()
+    whole = eng.step([(a, ids)], want="all").cpu()
+    assert (whole - want).abs().max() <= 2e-4 * max(1.0, float(want.abs().max()))
+    eng.release(a)
+    a = eng.acquire()
+    cut = [eng.step([(a, ids[:4])], want="all")] + [eng.step([(a, [t])], want="last") for t in ids[4:]]
+    assert (torch.cat(cut).cpu() - whole).abs().max() <= 1e-4
+
+    eng = Engine.load(str(tmp_path), dtype="bfloat16", max_tokens=128, max_slots=2)
+    assert eng.model.blocks[0].feed_forward.router.dtype == torch.float32 and eng.model.blocks[0].feed_forward.experts[0].w_down.dtype == BF16
+    a = eng.acquire()
+    whole16 = eng.step([(a, ids)], want="all").cpu()
+    eng.release(a)
+    a = eng.acquire()
+    cut = [eng.step([(a, ids[:4])], want="all")] + [eng.step([(a, [t])], want="last") for t in ids[4:]]
+    assert (torch.cat(cut).cpu() - whole16).abs().max() <= 5e-2 * max(1.0, float(whole16.abs().max()))
