@@ -32,8 +32,13 @@ TINY_C = dict(num_hidden_layers=2, hidden_size=120, num_attention_heads=6, num_k
 MID_D = dict(num_hidden_layers=2, hidden_size=2048, num_attention_heads=16, num_key_value_heads=4, head_dim=128,
              intermediate_size=2560, vocab_size=33024, rope_theta=1e6, rms_norm_eps=1e-6, max_position_embeddings=2048,
              tie_word_embeddings=True, eos_token_id=None, bos_token_id=None)
-SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": MID_D}
+# A tiny one for long contexts.  theta is a power of two, so that the rotation's frequencies
+# theta^(-2i/16) = 2^(-2i) and with them the angles at any position are exact in 32-bit, whichever
+# power routine computes them: at position 6000 a last-bit difference in a frequency would
+# otherwise be an angle error of 4e-4, above the 32-bit tolerance of these tests.
+LONG_L = dict(TINY_A, rope_theta=65536.0, max_position_embeddings=16384)
+SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3, "L": 4}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": MID_D, "L": LONG_L}
 
 _made = {}
 _tmp = None

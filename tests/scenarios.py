@@ -98,6 +98,23 @@ def long_decoding(make_engine, name, dtype, n_decode):
     assert_logits_close(got[-8:], want[-8:], dtype, f"{name} {dtype} long decoding, last positions")
 
 
+def long_context(make_engine, dtype, n_prompt=6000, n_decode=4):
+    """Thousands of tokens: page tables wider than 64 pages, attention over ~100 key blocks in the
+    prompt and, token by token, over many splits; positions where rounding of angles would show."""
+    name = "L"
+    V = CONFIGS[name]["vocab_size"]
+    toks = random_tokens(V, n_prompt + n_decode, 9)
+    want = plain_logits(name, toks)
+    eng = make_engine(name, dtype, n_prompt + 128, False)
+    s = eng.acquire()
+    places = [0, 63, 64, 4095, 4096, n_prompt - 2, n_prompt - 1]
+    got = eng.step([(s, toks[:n_prompt])], want=[places])
+    assert_logits_close(got, want[places], dtype, f"{dtype} long prompt")
+    dec = torch.cat([eng.step([(s, [t])], want="last") for t in toks[n_prompt:]])
+    assert_logits_close(dec, want[n_prompt:], dtype, f"{dtype} decoding after a long prompt")
+    eng.release(s)
+
+
 def first_tokens(make_engine, name, dtype):
     """Prompts of one and two tokens; the very first position; a chunk that starts at position 1."""
     V = CONFIGS[name]["vocab_size"]

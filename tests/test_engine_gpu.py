@@ -63,6 +63,11 @@ def test_long_decoding(name, n, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_long_context(dtype):
+    scenarios.long_context(make_engine, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_first_tokens(name, dtype):
     scenarios.first_tokens(make_engine, name, dtype)
