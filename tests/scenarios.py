@@ -98,6 +98,33 @@ def long_decoding(make_engine, name, dtype, n_decode):
     assert_logits_close(got[-8:], want[-8:], dtype, f"{name} {dtype} long decoding, last positions")
 
 
+def wide_batch(make_engine, name, dtype, n_seqs=70, n_decode=3):
+    """More sequences than 64 in one batch: the products leave the kernels for few rows, the
+    captured decode step takes a bucket of 96 rows with 26 of padding."""
+    V = CONFIGS[name]["vocab_size"]
+    reqs = [random_tokens(V, 2 + (7 * i) % 23 + n_decode, 500 + i) for i in range(n_seqs)]
+    eng = make_engine(name, dtype, 64 * n_seqs, False)
+    slots = [eng.acquire() for _ in reqs]
+    heads = [len(r) - n_decode for r in reqs]
+    lg = eng.step([(s, r[:h]) for s, r, h in zip(slots, reqs, heads)], want="last")
+    got = [[lg[i:i + 1]] for i in range(n_seqs)]
+    runner = eng.decode_runner(n_seqs, 64) if eng.graph_ok else None
+    for d in range(n_decode):
+        toks = [r[h + d] for r, h in zip(reqs, heads)]
+        if runner is not None and d > 0:                  # the first single-token step eagerly, the rest replayed
+            _, lg = runner.step(slots, toks)
+        else:
+            lg = eng.step([(s, [t]) for s, t in zip(slots, toks)], want="last")
+        for i in range(n_seqs):
+            got[i].append(lg[i:i + 1].clone())
+    for i in (0, 1, 17, 33, 64, 65, n_seqs - 1):
+        want = plain_logits(name, reqs[i])[heads[i] - 1:]
+        assert_logits_close(torch.cat(got[i]), want, dtype, f"{name} {dtype} sequence {i} of {n_seqs}")
+    for s in slots:
+        eng.release(s)
+    eng.cache.check()
+
+
 def long_context(make_engine, dtype, n_prompt=6000, n_decode=4):
     """Thousands of tokens: page tables wider than 64 pages, attention over ~100 key blocks in the
     prompt and, token by token, over many splits; positions where rounding of angles would show."""

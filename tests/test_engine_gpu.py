@@ -63,6 +63,12 @@ def test_long_decoding(name, n, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_wide_batch(name, dtype):
+    scenarios.wide_batch(make_engine, name, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_long_context(dtype):
     scenarios.long_context(make_engine, dtype)
 
