@@ -9,8 +9,9 @@
 //                  M <= 64: 32 or 64 rows of x, 64 (or 32) rows of W, 128 (or 256) deep: the rows of
 //                  W arrive as whole 256-byte pieces, which streams them faster than loading MFMA
 //                  fragments (64 bytes a row) straight from memory.  K may be cut into slices
-//                  whose partial sums the reader adds; x may be the gated activation of a fused
-//                  [gate | up] row, computed on its way into LDS.
+//                  whose partial sums the reader adds.  With PAIRED, W holds the rows of a gate and of
+//                  an up projection in turns of 16 and the kernel stores silu(gate) * up, half
+//                  as wide, without the two products ever being stored.
 //
 // Reference counterparts: crates/synaptix-kernels-cuda/src/best_cu/gemm/gemm_bf16.cu (TN family,
 // mma.sync m16n8k16), best_cu/gemv/mma_gemv.cu:19-133 (M == 1), best_cu/gemm/gemm_f32.cu (SIMT).
@@ -182,7 +183,7 @@ static void launch_skinny(const bf16* x, const bf16* w, void* out, int out_is_f3
 // D[m = 8*(j/4) + 4*(lane/32) + j%4][n = lane%32], j = 0..15.
 // LDS tiles are double-buffered: while one k-tile is multiplied the next is on its way from memory
 // into registers, and is stored into the other buffer before the barrier.
-template <int BM, int BN, int BK, int WM, int WN, bool KTAIL, bool GATED>
+template <int BM, int BN, int BK, int WM, int WN, bool KTAIL, bool PAIRED>
 __global__ void __launch_bounds__(64 * WM * WN)
 gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
                   int M, int N, int K, int k_slice) {
@@ -220,7 +221,7 @@ gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* 
 #pragma unroll
   for (int i = 0; i < XL; ++i) {
     xin[i] = !FEW || m0 + lrow + RPP * i < M;
-    xg[i] = x + (size_t)min(m0 + lrow + RPP * i, M - 1) * (GATED ? 2 * K : K) + lchunk;
+    xg[i] = x + (size_t)min(m0 + lrow + RPP * i, M - 1) * K + lchunk;
   }
 #pragma unroll
   for (int i = 0; i < WL; ++i) wg[i] = w + (size_t)min(n0 + lrow + RPP * i, N - 1) * K + lchunk;
@@ -236,7 +237,7 @@ gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* 
   // blockIdx.y = which slice of K (k_slice elements, a multiple of 32) this workgroup sums, as in gemm_skinny
   const int k_begin = FEW ? (int)blockIdx.y * k_slice : 0, k_end = FEW ? min(K, k_begin + k_slice) : K;
   const int nk = (k_end - k_begin + BK - 1) / BK;
-  bf16x8 rx[XL], ru[GATED ? XL : 1], rw[WL];
+  bf16x8 rx[XL], rw[WL];
   auto fetch = [&](int kt) {
     // K is a multiple of 8: a chunk lies inside or outside as a whole
     const int k = k_begin + kt * BK;
@@ -244,7 +245,6 @@ gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* 
 #pragma unroll
     for (int i = 0; i < XL; ++i) {
       rx[i] = (kin && xin[i]) ? *(const bf16x8*)(xg[i] + k) : zero;
-      if constexpr (GATED) ru[i] = (kin && xin[i]) ? *(const bf16x8*)(xg[i] + K + k) : zero;
     }
 #pragma unroll
     for (int i = 0; i < WL; ++i) rw[i] = kin ? *(const bf16x8*)(wg[i] + k) : zero;
@@ -252,18 +252,6 @@ gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* 
   auto stash = [&](int buf) {
     bf16* xs = smem + buf * (BM + BN) * LD;
     bf16* ws = xs + BM * LD;
-    if constexpr (GATED) {
-      // x = silu(g) * u of the fused [g | u] row, in 32-bit, rounded once
-#pragma unroll
-      for (int i = 0; i < XL; ++i)
-        if (xin[i]) {  // rows beyond M stay zero and cost no exponentials
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const float g = (float)rx[i][e];
-            rx[i][e] = (bf16)(g / (1.f + expf(-g)) * (float)ru[i][e]);
-          }
-        }
-    }
 #pragma unroll
     for (int i = 0; i < XL; ++i) *(bf16x8*)(xs + (lrow + RPP * i) * LD + lchunk) = rx[i];
 #pragma unroll
@@ -303,6 +291,15 @@ gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* 
       for (int e = 0; e < 16; ++e) {
         const int m = m0 + wm + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
         const int n = n0 + wn + j * 32 + lane % 32;
+        if constexpr (PAIRED) {
+          // columns n % 32 < 16 are gate rows, the 16 after them the up rows of the same outputs
+          // (N is a multiple of 32 here): a lane of the first kind gets its partner's value
+          const float up = __shfl_xor(acc[i][j][e], 16, SYN_WAVE);
+          const float g = acc[i][j][e];
+          if (m < M && n < N && lane % 32 < 16)
+            ((bf16*)out)[(size_t)m * (N / 2) + (n0 + wn + j * 32) / 2 + lane % 16] = (bf16)(g / (1.f + expf(-g)) * up);
+          continue;
+        }
         if (m < M && n < N) {
           if (out_is_f32)
             ((float*)out)[((size_t)(FEW ? blockIdx.y : 0) * M + m) * N + n] = acc[i][j][e];
@@ -312,7 +309,7 @@ gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* 
       }
 }
 
-template <int BM, int BN, int BK, int WM, int WN, bool GATED = false>
+template <int BM, int BN, int BK, int WM, int WN, bool PAIRED = false>
 static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
                         hipStream_t stream, int slices = 1) {
   SYN_CHECK(slices == 1 || BM <= 64, "gemm: slices of K only with the tiles for few rows");
@@ -324,19 +321,19 @@ static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32,
   const size_t lds = (size_t)2 * (BM + BN) * (BK + 8) * sizeof(bf16);
   static bool raised = false;
   if (lds > 65536 && !raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, WM, WN, false, GATED>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, WM, WN, false, PAIRED>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, WM, WN, true, GATED>,
+      e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, WM, WN, true, PAIRED>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     SYN_CHECK(e == hipSuccess, "gemm: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
     raised = true;
   }
   if (K % BK == 0 && k_slice % BK == 0)
-    gemm_tiled_kernel<BM, BN, BK, WM, WN, false, GATED>
+    gemm_tiled_kernel<BM, BN, BK, WM, WN, false, PAIRED>
         <<<dim3(grid, slices), 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
   else
-    gemm_tiled_kernel<BM, BN, BK, WM, WN, true, GATED>
+    gemm_tiled_kernel<BM, BN, BK, WM, WN, true, PAIRED>
         <<<dim3(grid, slices), 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
   return 0;
 }
@@ -394,25 +391,28 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   return 0;
 }
 
-// out = (silu(g) * u) . w^T for rows [g | u] of gate_up [M, 2K] (bf16, M <= 64), w [N, K]: the
-// activation is applied while x is on its way into LDS and is never stored.  dtype and slices as in
-// syn_gemm (1 = bf16 out, 2 = float out, slices of K only with float out).
-SYN_EXPORT int syn_gemm_gated(const void* gate_up, const void* w, void* out, int dtype, int M, int N, int K,
-                              int slices, hipStream_t stream) {
-  SYN_CHECK(M > 0 && N > 0 && K > 0, "gemm_gated: empty shape M=%d N=%d K=%d", M, N, K);
-  SYN_CHECK(dtype == 1 || dtype == 2, "gemm_gated: bf16 operands only (dtype code %d)", dtype);
-  SYN_CHECK(M <= 64, "gemm_gated: at most 64 rows (M = %d)", M);
-  SYN_CHECK(slices >= 1 && slices <= 64 && (slices == 1 || dtype == 2), "gemm_gated: %d slices of K need a float output",
-            slices);
-  SYN_CHECK(K % 8 == 0 && (uintptr_t)gate_up % 16 == 0 && (uintptr_t)w % 16 == 0,
-            "gemm_gated: K = %d must be a multiple of 8 and the operands 16-byte aligned", K);
-  const bf16* xb = (const bf16*)gate_up;
+// out[M, N/2] = silu(x . Wg^T) * (x . Wu^T), bf16, where w [N, K] holds the rows of Wg and of Wu in
+// turns of 16: rows 32b .. 32b+15 are rows 16b .. 16b+15 of Wg, rows 32b+16 .. 32b+31 those of Wu.
+// The activation is applied to the 32-bit sums and rounded once.
+SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, int N, int K, hipStream_t stream) {
+  SYN_CHECK(M > 0 && N > 0 && K > 0, "gemm_swiglu: empty shape M=%d N=%d K=%d", M, N, K);
+  SYN_CHECK(N % 32 == 0, "gemm_swiglu: %d paired rows are no multiple of 32", N);
+  SYN_CHECK(K % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0,
+            "gemm_swiglu: K = %d must be a multiple of 8 and the operands 16-byte aligned", K);
+  const bf16* xb = (const bf16*)x;
   const bf16* wb = (const bf16*)w;
-  const int out_is_f32 = dtype == 2;
   int rc;
-  if (M <= 32) rc = launch_tiled<32, 64, 128, 1, 2, true>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
-  else rc = launch_tiled<64, 64, 128, 2, 2, true>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
+  if (M <= 32) {
+    if (N >= 65536) rc = launch_tiled<32, 32, 256, 1, 1, true>(xb, wb, out, 0, M, N, K, stream);
+    else rc = launch_tiled<32, 64, 128, 1, 2, true>(xb, wb, out, 0, M, N, K, stream);
+  } else if (M <= 64) {
+    rc = launch_tiled<64, 64, 128, 2, 2, true>(xb, wb, out, 0, M, N, K, stream);
+  } else {
+    const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+    if (t256 >= 192) rc = launch_tiled<256, 256, 64, 4, 2, true>(xb, wb, out, 0, M, N, K, stream);
+    else rc = launch_tiled<128, 128, 64, 2, 2, true>(xb, wb, out, 0, M, N, K, stream);
+  }
   if (rc) return rc;
-  SYN_LAUNCH_CHECK("gemm_gated");
+  SYN_LAUNCH_CHECK("gemm_swiglu");
   return 0;
 }

@@ -138,26 +138,28 @@ def gemm(x, w, out, force_simt=False):
           slices, _stream())
 
 
-def gemm_gated(gate_up, w, out):
-    """out = (silu(g) * u) . w^T for rows [g | u] of gate_up [M, 2K] (bf16, M <= 64) and w [N, K]:
-    the gated activation inside the product, so that it is never stored.  out is [M, N] in bf16
-    or float, or float partial sums [S, M, N] over slices of K."""
-    _need(gate_up, "gemm_gated.gate_up", _BF16, (None, None))
-    M, K2 = gate_up.shape
-    if K2 % 2 or M > 64:
-        raise KernelError(f"gemm_gated: gate_up {tuple(gate_up.shape)} needs an even width and at most 64 rows")
-    K = K2 // 2
-    _need(w, "gemm_gated.w", _BF16, (None, K))
-    N = w.shape[0]
-    slices = 1
-    if out.dim() == 3:
-        slices = out.shape[0]
-        _need(out, "gemm_gated.out", _F32, (slices, M, N))
-        code = 2
-    else:
-        _need(out, "gemm_gated.out", (_BF16, _F32), (M, N))
-        code = 2 if out.dtype == _F32 else 1
-    _call(load_library("core"), "syn_gemm_gated", _ptr(gate_up), _ptr(w), _ptr(out), code, M, N, K, slices, _stream())
+PAIR = 16   # rows of the gate and of the up projection alternate in turns of this many
+
+
+def pair_rows(gate, up):
+    """The weight of gemm_swiglu: rows of `gate` and of `up` [I, K] in turns of 16 -> [2 I, K]."""
+    I, K = gate.shape
+    if up.shape != gate.shape or I % PAIR:
+        raise KernelError(f"pair_rows: shapes {tuple(gate.shape)}, {tuple(up.shape)} (rows in turns of {PAIR})")
+    return torch.stack([gate.view(I // PAIR, PAIR, K), up.view(I // PAIR, PAIR, K)], 1).reshape(2 * I, K).contiguous()
+
+
+def gemm_swiglu(x, w_paired, out):
+    """out[M, I] = silu(x . Wg^T) * (x . Wu^T) in bf16 with w_paired = pair_rows(Wg, Wu): the
+    activation on the 32-bit sums inside the product, so that the two products are never stored."""
+    _need(x, "gemm_swiglu.x", _BF16, (None, None))
+    M, K = x.shape
+    _need(w_paired, "gemm_swiglu.w", _BF16, (None, K))
+    N = w_paired.shape[0]
+    if N % (2 * PAIR) or K % 8:
+        raise KernelError(f"gemm_swiglu: {N} paired rows, K = {K} (multiples of {2 * PAIR} and of 8)")
+    _need(out, "gemm_swiglu.out", _BF16, (M, N // 2))
+    _call(load_library("core"), "syn_gemm_swiglu", _ptr(x), _ptr(w_paired), _ptr(out), M, N, K, _stream())
 
 
 def gemm_slices(M, N, K, dtype):

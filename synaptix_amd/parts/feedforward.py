@@ -10,7 +10,7 @@ import torch
 from ..kernels import ops
 from ..weights.source import TensorSpec
 from .base import Part
-from .linear import gated_linear_for_sum, linear, linear_for_sum
+from .linear import linear, linear_for_sum
 
 
 class FeedForward(Part):
@@ -26,6 +26,7 @@ class GatedMlp(FeedForward):
             raise ValueError(f"activation {activation!r} is not built (silu only)")
         self.prefix, self.hidden, self.intermediate = prefix, hidden, intermediate
         self.w_gate_up = self.w_down = None
+        self.paired = False      # gate and up rows in turns of 16: the activation runs inside the product
 
     def tensor_specs(self):
         p = self.prefix
@@ -37,14 +38,16 @@ class GatedMlp(FeedForward):
 
     def load(self, get):
         p = self.prefix
-        self.w_gate_up = torch.cat([get(p + "gate_proj.weight"), get(p + "up_proj.weight")], 0)
+        gate, up = get(p + "gate_proj.weight"), get(p + "up_proj.weight")
+        self.paired = (gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16
+                       and self.intermediate % ops.PAIR == 0 and self.hidden % 8 == 0)
+        self.w_gate_up = ops.pair_rows(gate, up) if self.paired else torch.cat([gate, up], 0)
         self.w_down = get(p + "down_proj.weight")
 
     def forward(self, h, ctx):
-        gu = linear(h, self.w_gate_up, h.dtype)
-        fused = gated_linear_for_sum(gu, self.w_down)
-        if fused is not None:
-            return fused
         m = torch.empty((h.shape[0], self.intermediate), dtype=h.dtype, device=h.device)
-        ops.swiglu(gu, m)
+        if self.paired and h.dtype == torch.bfloat16:
+            ops.gemm_swiglu(h, self.w_gate_up, m)
+        else:
+            ops.swiglu(linear(h, self.w_gate_up, h.dtype), m)
         return linear_for_sum(m, self.w_down)

@@ -36,17 +36,3 @@ def linear_for_sum(x, w):
     ops.gemm(x, w, out)
     return out
 
-
-def gated_linear_for_sum(gate_up, w):
-    """(silu(g) * u) . W^T for rows [g | u] of gate_up, as linear_for_sum gives it, with the
-    activation inside the product where the product is cut along K and has at most 16 rows (every
-    workgroup of the product computes the activation of its k range again, which costs more than
-    the activation's own kernel saves once there are more rows: measured at 64); None where it
-    is not, and the caller applies the activation on its own."""
-    M, K = gate_up.shape[0], gate_up.shape[1] // 2
-    N = w.shape[0]
-    if w.dtype != gate_up.dtype or M > 16 or ops.gemm_slices(M, N, K, gate_up.dtype) <= 1:
-        return None
-    out = torch.empty((ops.gemm_slices(M, N, K, gate_up.dtype), M, N), dtype=torch.float32, device=gate_up.device)
-    ops.gemm_gated(gate_up, w, out)
-    return out

@@ -60,10 +60,15 @@ def gemm(x, w, out, force_simt=False):
     out.copy_((x.to(F32) @ w.to(F32).T).to(out.dtype))
 
 
-def gemm_gated(gate_up, w, out):
-    K = gate_up.shape[1] // 2
-    g, u = gate_up[:, :K].to(F32), gate_up[:, K:].to(F32)
-    gemm((g / (1 + torch.exp(-g)) * u).to(gate_up.dtype), w, out)
+PAIR = 16
+
+
+def gemm_swiglu(x, w_paired, out):
+    N, K = w_paired.shape
+    w = w_paired.view(N // (2 * PAIR), 2, PAIR, K)
+    g = x.to(F32) @ w[:, 0].reshape(N // 2, K).to(F32).T
+    u = x.to(F32) @ w[:, 1].reshape(N // 2, K).to(F32).T
+    out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
 
 
 def gemm_slices(M, N, K, dtype):
@@ -168,7 +173,7 @@ def sample_rows(logits, temperature, uniform, out):
         out[r] = int(hit[0]) if hit.numel() else x.numel() - 1
 
 
-ALL = ["embed", "add_rmsnorm", "rmsnorm_rows", "swiglu", "gemm", "gemm_gated", "gemm_slices", "qk_norm_rope_kv_write", "attention_f32",
+ALL = ["embed", "add_rmsnorm", "rmsnorm_rows", "swiglu", "gemm", "gemm_swiglu", "gemm_slices", "qk_norm_rope_kv_write", "attention_f32",
        "attention_prefill_bf16", "decode_splits", "attention_decode_bf16", "sample_rows"]
 
 

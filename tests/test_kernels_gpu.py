@@ -188,28 +188,25 @@ def test_gemm_bf16_partial_sums_over_slices_of_k(ops, M, N, K, S):
     close(got2, want2, 1e-4, 1e-4, "gathered rows of residual + slices")
 
 
-@pytest.mark.parametrize("M,N,K,S", [(1, 48, 64, 1), (8, 4096, 12288, 8), (7, 100, 1000, 3), (33, 70, 136, 1),
-                                     (64, 130, 2048, 4)])
-def test_gemm_with_gated_activation_inside(ops, M, N, K, S):
-    """(silu(g) * u) . W^T from the fused [g | u] rows equals the activation kernel followed by the
-    product, value for value: the activation is rounded to bf16 once in both."""
-    gu, w = rnd((M, 2 * K), 18, BF16).to(DEV), rnd((N, K), 19, BF16).to(DEV)
-    act = torch.empty((M, K), dtype=BF16, device=DEV)
-    ops.swiglu(gu, act)
-    g, u = gu[:, :K].cpu().float(), gu[:, K:].cpu().float()
-    close(act, (g / (1 + torch.exp(-g)) * u).to(BF16), 2e-2, 1e-2, "activation kernel")
-    want = (act.cpu().double() @ w.cpu().double().T).float()
-    shape = (S, M, N) if S > 1 else (M, N)
-    out = torch.full(shape, float("nan"), dtype=F32, device=DEV)
-    ops.gemm_gated(gu, w, out)
-    got = out.sum(0) if S > 1 else out
-    close(got, want, 1e-3 * math.sqrt(K), what=f"gated product {M}x{N}x{K}, {S} slice(s)")
-    if S == 1:
-        out16 = torch.empty((M, N), dtype=BF16, device=DEV)
-        ops.gemm_gated(gu, w, out16)
-        close(out16, want, 1e-3 * math.sqrt(K) + 0.02, 1e-2, "gated product, bf16 out")
-    with pytest.raises(Exception, match="64 rows"):
-        ops.gemm_gated(torch.zeros((65, 2 * K), dtype=BF16, device=DEV), w, torch.empty((65, N), dtype=F32, device=DEV))
+@pytest.mark.parametrize("M,I,K", [(1, 48, 64), (8, 2560, 4096), (7, 112, 1000), (33, 80, 136), (64, 1024, 512),
+                                   (300, 400, 264), (2048, 3072, 256), (8, 32784, 72)])
+def test_gemm_with_the_gated_activation_inside(ops, M, I, K):
+    """silu(x . Wg^T) * (x . Wu^T) from one product over the rows of Wg and Wu in turns of 16,
+    against the two products and the activation in 64-bit; every tile shape of the kernel."""
+    x, wg, wu = rnd((M, K), 18, BF16), rnd((I, K), 19, BF16), rnd((I, K), 20, BF16)
+    paired = ops.pair_rows(wg.to(DEV), wu.to(DEV))
+    assert paired.shape == (2 * I, K)
+    assert torch.equal(paired[16:32].cpu(), wu[:16]) and torch.equal(paired[32:48].cpu(), wg[16:32])
+    out = torch.full((M, I), float("nan"), dtype=BF16, device=DEV)
+    ops.gemm_swiglu(x.to(DEV), paired, out)
+    g, u = x.double() @ wg.double().T, x.double() @ wu.double().T
+    want = (g / (1 + torch.exp(-g)) * u).float()
+    # products of standard deviation sqrt(K); one bf16 rounding of the result
+    close(out, want, 2e-3 * K + 0.02, 1e-2, f"gated product {M}x{I}x{K}")
+    with pytest.raises(Exception, match="turns of 16"):
+        ops.pair_rows(wg[:24].to(DEV), wu[:24].to(DEV))
+    with pytest.raises(Exception, match="paired rows"):
+        ops.gemm_swiglu(x.to(DEV), paired[:48], torch.empty((M, 24), dtype=BF16, device=DEV))
 
 
 def test_gemm_bf16_paths_agree(ops):
