@@ -41,6 +41,14 @@ class StateLayerView:
     state: torch.Tensor
 
 
+@dataclass
+class Snapshot:
+    """A point in a sequence that `SequenceCache.restore` goes back to."""
+    slot: int
+    length: int
+    states: dict                      # cache layer -> copy of the slot's state
+
+
 class _GroupPool:
     """The page pool of one group, as the native cache keeps it."""
 
@@ -170,6 +178,24 @@ class SequenceCache:
     def commit(self, sid: int, n_new: int) -> None:
         """The step has written n_new tokens; windows give back the pages that fell out of reach."""
         rt.check(rt.lib().syn_cache_commit(self._h, self._sid(sid), int(n_new)))
+
+    # ------------------------------------------------------------------ going back
+    def truncate(self, sid: int, length: int) -> None:
+        """Go back to an earlier length; the positions behind it are written again by later steps.
+        Enough for keys and values; a fixed-size state needs `restore` of a snapshot taken there."""
+        rt.check(rt.lib().syn_cache_truncate(self._h, self._sid(sid), int(length)))
+
+    def snapshot(self, sid: int) -> "Snapshot":
+        """The sequence's length and a copy of its fixed-size states: a point to come back to.  A
+        running state cannot be rewound by a length (the reference snapshots it likewise,
+        crates/synaptix-models/llm/common/src/model.rs:377-492)."""
+        return Snapshot(self._sid(sid), self.length(sid), {i: st[sid].clone() for i, st in self._state.items()})
+
+    def restore(self, snap: "Snapshot") -> None:
+        """Back to the snapshot's point: the length, and the states as they were there."""
+        self.truncate(snap.slot, snap.length)
+        for i, saved in snap.states.items():
+            self._state[i][snap.slot].copy_(saved)
 
     # ------------------------------------------------------------------ what a step needs
     def table_width(self, gi: int, sids: list) -> int:

@@ -334,6 +334,28 @@ RT_API int syn_cache_commit(void* h, int sid, long n_new) {
   return OK;
 }
 
+// Go back to an earlier length of the sequence (what lies behind it is written again).  Pages stay
+// held; a group with a window must still hold every page that a query at `length` sees.
+RT_API int syn_cache_truncate(void* h, int sid, long length) {
+  Cache* c = (Cache*)h;
+  Slot* s = c->live_slot(sid);
+  if (!s) return MISUSE;
+  if (length < 0 || length > s->length)
+    return fail(MISUSE, "slot %d holds %ld tokens and cannot go back to %ld", sid, s->length, length);
+  for (size_t g = 0; g < c->pools.size(); ++g) {
+    const long w = c->windows[g];
+    if (w < 0) continue;
+    const long first_needed = std::max(0L, length - w + 1) / PAGE_TOKENS;
+    const std::vector<int>& pages = s->pages[g];
+    for (long i = first_needed; i < pages_for(length) && i < (long)pages.size(); ++i)
+      if (pages[i] < 0)
+        return fail(MISUSE, "slot %d: the window of group %d has given back a page that length %ld needs", sid,
+                    (int)g, length);
+  }
+  s->length = length;
+  return OK;
+}
+
 RT_API int syn_cache_table_width(void* h, int group, const int* sids, int n, int* out) {
   Cache* c = (Cache*)h;
   int w = 1;

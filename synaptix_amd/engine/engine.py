@@ -92,6 +92,14 @@ class Engine:
     def length(self, slot: int) -> int:
         return self.cache.length(slot)
 
+    def snapshot(self, slot: int):
+        """A point of the sequence to come back to with `restore` (its length and running states)."""
+        return self.cache.snapshot(slot)
+
+    def restore(self, snap) -> None:
+        """Back to a snapshot: later steps write the positions behind it again."""
+        self.cache.restore(snap)
+
     # ------------------------------------------------------------------ the step
     def _require_gpu(self):
         if self.device is None or self.device.type != "cuda":

@@ -39,6 +39,7 @@ _SIGNATURES = {
     "syn_cache_reserve": (_I, [_P, _I, _L]),
     "syn_cache_reserve_step": (_I, [_P, _I, _IP, _LP]),
     "syn_cache_commit": (_I, [_P, _I, _L]),
+    "syn_cache_truncate": (_I, [_P, _I, _L]),
     "syn_cache_table_width": (_I, [_P, _I, _IP, _I, _IP]),
     "syn_cache_page_table": (_I, [_P, _I, _IP, _I, _I, _P]),
     "syn_cache_live_slots": (_I, [_P, _IP]),

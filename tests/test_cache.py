@@ -151,3 +151,30 @@ def test_random_walk_keeps_every_invariant():
         c.release(s)
     c.check()
     assert c.free_slots == 12 and all(g.pool.free_pages == 40 for g in c.groups)
+
+
+def test_going_back_to_a_snapshot():
+    """A length can be rewound; a running state cannot, so a snapshot keeps a copy of it.  A
+    window that has already given a page back refuses to go back behind it."""
+    c = make(needs=[KvNeed(2, 16), StateNeed((3,)), KvNeed(2, 16, window=70)], max_slots=2)
+    s = c.acquire()
+    c.reserve(s, 40), c.commit(s, 40)
+    c.layer_view(1).state[s] += 5.0
+    snap = c.snapshot(s)
+    c.reserve(s, 30), c.commit(s, 30)
+    c.layer_view(1).state[s] += 1.0
+    held = c.groups[0].pool.free_pages
+    c.restore(snap)
+    assert c.length(s) == 40 and c.layer_view(1).state[s].tolist() == [5.0, 5.0, 5.0]
+    assert c.groups[0].pool.free_pages == held              # the pages stay with the sequence
+    c.reserve(s, 30), c.commit(s, 30)                       # and are written again without new ones
+    assert c.groups[0].pool.free_pages == held and c.length(s) == 70
+    with pytest.raises(CacheError, match="cannot go back"):
+        c.truncate(s, 71)
+    c.reserve(s, 130), c.commit(s, 130)                     # 200 tokens: the window has let page 0 and 1 go
+    with pytest.raises(CacheError, match="window"):
+        c.restore(snap)
+    c.truncate(s, 199)                                      # within what the window still holds
+    c.check()
+    c.release(s)
+    c.check()

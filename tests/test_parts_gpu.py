@@ -237,6 +237,18 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
         tolerance = 1e-4 if dtype == "float32" else 5e-2
         assert (torch.cat(got[0]) - whole[:7]).abs().max() <= tolerance
         assert (torch.cat(got[1]) - whole[7:]).abs().max() <= tolerance
+        # back to a snapshot: the running state is restored with the length, and the same tokens
+        # give the same logits again
+        eng.release(a2), eng.release(b2)
+        c = eng.acquire()
+        eng.step([(c, toks[0][:4])], want=None)
+        snap = eng.snapshot(c)
+        first = eng.step([(c, toks[0][4:])], want="all")
+        eng.restore(snap)
+        assert eng.length(c) == 4
+        again = eng.step([(c, toks[0][4:])], want="all")
+        assert torch.equal(first, again)
+        assert (first - whole[4:7]).abs().max() <= tolerance
 
 
 # ----------------------------------------------------------------------------- more toy parts
