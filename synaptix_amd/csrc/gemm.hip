@@ -5,7 +5,7 @@
 //   gemm_skinny    bf16, M == 1: the weight matrix is streamed once from HBM through
 //                  v_mfma_f32_16x16x32_bf16; the waves of a workgroup split K and sum in LDS.
 //   gemm_tiled     bf16: tiles of x and W in LDS, double-buffered, v_mfma_f32_32x32x16_bf16.
-//                  M > 64: 256x256x64 tiles with 8 waves (or 128x128x64 with 4).
+//                  M > 64: 256x256x64 or 256x192x64 tiles with 8 waves, or 128x128x64 with 4.
 //                  M <= 64: 32 or 64 rows of x, 64 (or 32) rows of W, 128 (or 256) deep: the rows of
 //                  W arrive as whole 256-byte pieces, which streams them faster than loading MFMA
 //                  fragments (64 bytes a row) straight from memory.  K may be cut into slices
@@ -338,6 +338,22 @@ static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32,
   return 0;
 }
 
+// Which of the large tiles for M > 64: 0 = 256 x 256, 1 = 256 x 192 (both 8 waves, one workgroup a
+// compute unit), 2 = 128 x 128 (4 waves, two workgroups a compute unit, about 15 % less efficient).
+// The estimate is the number of rounds over the 256 compute units times the work of a tile; it
+// reproduces what was measured at 2048 rows for N = 4096, 6144 and 24576 (a tie goes to the larger tile).
+static int pick_large_tile(int M, int N) {
+  auto rounds = [](long tiles, long slots) { return (tiles + slots - 1) / slots; };
+  auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+  const double cost[3] = {(double)rounds(tiles(256, 256), 256) * 256 * 256,
+                          (double)rounds(tiles(256, 192), 256) * 256 * 192,
+                          (double)rounds(tiles(128, 128), 512) * 2 * 128 * 128 * 1.15};
+  int best = 0;
+  if (cost[1] < cost[best]) best = 1;
+  if (cost[2] < cost[best]) best = 2;
+  return best;
+}
+
 // ------------------------------------------------------------------ entry point
 // dtype: 0 = float in, float out; 1 = bf16 in, bf16 out; 2 = bf16 in, float out.
 // slices > 1 (bf16 in, float out, M <= 64 only): out is [slices, M, N], slice s holds the sum over its
@@ -380,10 +396,9 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   } else if (M <= 64) {
     rc = launch_tiled<64, 64, 128, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
   } else {
-    // 256 x 256 tiles (8 waves) where they keep at least three quarters of the compute units busy,
-    // 128 x 128 tiles (4 waves) for smaller problems
-    const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-    if (t256 >= 192) rc = launch_tiled<256, 256, 64, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
+    const int shape = pick_large_tile(M, N);
+    if (shape == 0) rc = launch_tiled<256, 256, 64, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else if (shape == 1) rc = launch_tiled<256, 192, 64, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
     else rc = launch_tiled<128, 128, 64, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
   }
   if (rc) return rc;
@@ -408,8 +423,9 @@ SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, i
   } else if (M <= 64) {
     rc = launch_tiled<64, 64, 128, 2, 2, true>(xb, wb, out, 0, M, N, K, stream);
   } else {
-    const long t256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-    if (t256 >= 192) rc = launch_tiled<256, 256, 64, 4, 2, true>(xb, wb, out, 0, M, N, K, stream);
+    const int shape = pick_large_tile(M, N);
+    if (shape == 0) rc = launch_tiled<256, 256, 64, 4, 2, true>(xb, wb, out, 0, M, N, K, stream);
+    else if (shape == 1) rc = launch_tiled<256, 192, 64, 4, 2, true>(xb, wb, out, 0, M, N, K, stream);
     else rc = launch_tiled<128, 128, 64, 2, 2, true>(xb, wb, out, 0, M, N, K, stream);
   }
   if (rc) return rc;

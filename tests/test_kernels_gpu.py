@@ -189,7 +189,7 @@ def test_gemm_bf16_partial_sums_over_slices_of_k(ops, M, N, K, S):
 
 
 @pytest.mark.parametrize("M,I,K", [(1, 48, 64), (8, 2560, 4096), (7, 112, 1000), (33, 80, 136), (64, 1024, 512),
-                                   (300, 400, 264), (2048, 3072, 256), (8, 32784, 72)])
+                                   (300, 400, 264), (2048, 3072, 256), (1000, 6272, 136), (8, 32784, 72)])
 def test_gemm_with_the_gated_activation_inside(ops, M, I, K):
     """silu(x . Wg^T) * (x . Wu^T) from one product over the rows of Wg and Wu in turns of 16,
     against the two products and the activation in 64-bit; every tile shape of the kernel."""
