@@ -5,7 +5,9 @@
 //   gemm_skinny    bf16, M == 1: the weight matrix is streamed once from HBM through
 //                  v_mfma_f32_16x16x32_bf16; the waves of a workgroup split K and sum in LDS.
 //   gemm_tiled     bf16: tiles of x and W in LDS, double-buffered, v_mfma_f32_32x32x16_bf16.
-//                  M > 64: 256x256x64 or 256x192x64 tiles with 8 waves, or 128x128x64 with 4.
+//                  M > 64: 256x256x64 or 256x192x64 tiles with 8 waves, or 128x128x64 with 4; when K
+//                  is a multiple of 64 by gemm_direct, whose loads write LDS without passing
+//                  through registers.
 //                  M <= 64: 32 or 64 rows of x, 64 (or 32) rows of W, 128 (or 256) deep: the rows of
 //                  W arrive as whole 256-byte pieces, which streams them faster than loading MFMA
 //                  fragments (64 bytes a row) straight from memory.  K may be cut into slices
@@ -177,6 +179,57 @@ static void launch_skinny(const bf16* x, const bf16* w, void* out, int out_is_f3
   gemm_skinny_kernel<MB, RT, WAVES, U><<<grid, WAVES * SYN_WAVE, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
 }
 
+// ------------------------------------------------------------------ shared by the tiled kernels
+// Which tile: workgroup b runs on XCD b % 8, and each XCD has an L2 of its own.  Tiles are grouped
+// into panels of PM x PN (m fastest); a panel goes to one XCD, so the workgroups that run there at
+// the same time share rows of x and of W in its L2.  False for the launches that pad the last panels.
+__device__ __forceinline__ bool tile_of_workgroup(int M, int N, int BM, int BN, int& tm, int& tn) {
+  const int tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM;
+  const int PM = min(8, tiles_m), PN = 4;
+  const int panels_m = (tiles_m + PM - 1) / PM;
+  const int xcd = (int)blockIdx.x % 8, local = (int)blockIdx.x / 8;
+  const int panel = (local / (PM * PN)) * 8 + xcd, in_panel = local % (PM * PN);
+  tm = (panel % panels_m) * PM + in_panel % PM;
+  tn = (panel / panels_m) * PN + in_panel / PM;
+  return tm < tiles_m && tn < tiles_n;
+}
+
+static int tile_grid(int M, int N, int BM, int BN) {
+  const int tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM;
+  const int PM = tiles_m < 8 ? tiles_m : 8, PN = 4;
+  const int panels = ((tiles_m + PM - 1) / PM) * ((tiles_n + PN - 1) / PN);
+  return (panels + 7) / 8 * 8 * PM * PN;
+}
+
+// The accumulators of a wave (TM x TN tiles of MFMA 32x32: D[m = 8*(e/4) + 4*(lane/32) + e%4][n = lane%32])
+// to memory.  mw, nw: the first row and column of the wave's part.  PAIRED: columns n % 32 < 16 are
+// gate rows, the 16 after them the up rows of the same outputs (N is a multiple of 32 then): a lane of
+// the first kind gets its partner's value and stores silu(gate) * up, half as wide.
+template <int TM, int TN, bool PAIRED>
+__device__ __forceinline__ void store_tiles(const f32x16 (&acc)[TM][TN], void* __restrict__ out, int out_is_f32,
+                                            size_t slice, int M, int N, int mw, int nw, int lane) {
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = mw + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+        const int n = nw + j * 32 + lane % 32;
+        if constexpr (PAIRED) {
+          const float up = __shfl_xor(acc[i][j][e], 16, SYN_WAVE);
+          const float g = acc[i][j][e];
+          if (m < M && n < N && lane % 32 < 16)
+            ((bf16*)out)[(size_t)m * (N / 2) + (nw + j * 32) / 2 + lane % 16] = (bf16)(g / (1.f + expf(-g)) * up);
+        } else if (m < M && n < N) {
+          if (out_is_f32)
+            ((float*)out)[(slice * M + m) * N + n] = acc[i][j][e];
+          else
+            ((bf16*)out)[(size_t)m * N + n] = (bf16)acc[i][j][e];
+        }
+      }
+}
+
 // ------------------------------------------------------------------ tiled, bf16
 // Block tile BM (m) x BN (n) x BK (k); WM x WN waves, each (BM/WM) x (BN/WN) of MFMA 32x32x16 tiles.
 // MFMA 32x32x16: A = x rows, B = W rows; lane holds row lane%32, k = 8*(lane/32) .. +8;
@@ -198,16 +251,8 @@ gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* 
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];  // [2][(BM + BN) * LD]
   const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE;
   const int wm = (wave / WN) * (BM / WM), wn = (wave % WN) * (BN / WN);
-  // Which tile: workgroup b runs on XCD b % 8, and each XCD has an L2 of its own.  Tiles are grouped
-  // into panels of PM x PN (m fastest); a panel goes to one XCD, so the workgroups that run there at
-  // the same time share rows of x and of W in its L2.
-  const int tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM;
-  const int PM = min(8, tiles_m), PN = 4;
-  const int panels_m = (tiles_m + PM - 1) / PM;
-  const int xcd = (int)blockIdx.x % 8, local = (int)blockIdx.x / 8;
-  const int panel = (local / (PM * PN)) * 8 + xcd, in_panel = local % (PM * PN);
-  const int tm = (panel % panels_m) * PM + in_panel % PM, tn = (panel / panels_m) * PN + in_panel / PM;
-  if (tm >= tiles_m || tn >= tiles_n) return;
+  int tm, tn;
+  if (!tile_of_workgroup(M, N, BM, BN, tm, tn)) return;
   const int m0 = tm * BM, n0 = tn * BN;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
@@ -283,30 +328,7 @@ gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* 
     __syncthreads();
   }
 
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int m = m0 + wm + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
-        const int n = n0 + wn + j * 32 + lane % 32;
-        if constexpr (PAIRED) {
-          // columns n % 32 < 16 are gate rows, the 16 after them the up rows of the same outputs
-          // (N is a multiple of 32 here): a lane of the first kind gets its partner's value
-          const float up = __shfl_xor(acc[i][j][e], 16, SYN_WAVE);
-          const float g = acc[i][j][e];
-          if (m < M && n < N && lane % 32 < 16)
-            ((bf16*)out)[(size_t)m * (N / 2) + (n0 + wn + j * 32) / 2 + lane % 16] = (bf16)(g / (1.f + expf(-g)) * up);
-          continue;
-        }
-        if (m < M && n < N) {
-          if (out_is_f32)
-            ((float*)out)[((size_t)(FEW ? blockIdx.y : 0) * M + m) * N + n] = acc[i][j][e];
-          else
-            ((bf16*)out)[(size_t)m * N + n] = (bf16)acc[i][j][e];
-        }
-      }
+  store_tiles<TM, TN, PAIRED>(acc, out, out_is_f32, FEW ? blockIdx.y : 0, M, N, m0 + wm, n0 + wn, lane);
 }
 
 template <int BM, int BN, int BK, int WM, int WN, bool PAIRED = false>
@@ -314,10 +336,7 @@ static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32,
                         hipStream_t stream, int slices = 1) {
   SYN_CHECK(slices == 1 || BM <= 64, "gemm: slices of K only with the tiles for few rows");
   const int k_slice = ((K + slices - 1) / slices + 31) / 32 * 32;
-  const int tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM;
-  const int PM = tiles_m < 8 ? tiles_m : 8, PN = 4;
-  const int panels = ((tiles_m + PM - 1) / PM) * ((tiles_n + PN - 1) / PN);
-  const int grid = (panels + 7) / 8 * 8 * PM * PN;
+  const int grid = tile_grid(M, N, BM, BN);
   const size_t lds = (size_t)2 * (BM + BN) * (BK + 8) * sizeof(bf16);
   static bool raised = false;
   if (lds > 65536 && !raised) {
@@ -338,6 +357,115 @@ static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32,
   return 0;
 }
 
+// ------------------------------------------------------------------ tiled, loads straight into LDS
+// The same tiles for M > 64 and K a multiple of 64, with global_load_lds_dwordx4: a load writes its
+// 16 bytes a lane into LDS without passing through registers, so a k-tile on its way costs no
+// registers and no LDS store instructions, and the wait for it is the last thing before the barrier.
+// An instruction of a wave fills 1 KB of LDS in lane order: 8 rows of 64 k-values, unpadded.  To keep
+// the fragment reads free of bank conflicts all the same, slot s of row r holds the row's 16-byte
+// chunk s ^ ((r >> 1) & 7): the swizzle is applied to the global address of the lane that fills the
+// slot, and again by the reader.  Measured 10 to 20 % faster than staging through registers.
+template <int BM, int BN, int WM, int WN, bool PAIRED>
+__global__ void __launch_bounds__(64 * WM * WN)
+gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
+                   int M, int N, int K) {
+  constexpr int BK = 64;
+  constexpr int WAVES = WM * WN;
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+  constexpr int ROWS = BM + BN;
+  constexpr int PASSES = ROWS / (8 * WAVES);   // instructions of a wave for one k-tile
+  static_assert(ROWS % (8 * WAVES) == 0 && TM >= 1 && TN >= 1, "tile shape");
+  extern __shared__ __attribute__((aligned(16))) bf16 smem[];  // [2][ROWS][BK]
+  const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE;
+  const int wm = (wave / WN) * (BM / WM), wn = (wave % WN) * (BN / WN);
+  int tm, tn;
+  if (!tile_of_workgroup(M, N, BM, BN, tm, tn)) return;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  // pass p: the wave fills tile rows (p * WAVES + wave) * 8 .. + 8 (x rows first, then W rows; rows
+  // beyond M or N repeat the last valid one and their results are never stored)
+  const bf16* src[PASSES];
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    const int row = (p * WAVES + wave) * 8 + lane / 8;
+    const int chunk = (lane % 8) ^ ((row >> 1) & 7);
+    src[p] = (row < BM ? x + (size_t)min(m0 + row, M - 1) * K : w + (size_t)min(n0 + row - BM, N - 1) * K) + chunk * 8;
+  }
+  auto fetch = [&](int kt, int buf) {
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      bf16* dst = smem + (size_t)buf * ROWS * BK + (size_t)(p * WAVES + wave) * 8 * BK;  // the same for all lanes
+      __builtin_amdgcn_global_load_lds((const void*)(src[p] + (size_t)kt * BK),
+                                       (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    }
+  };
+  // all loads of this wave have written LDS: vmcnt(0), the other counters left alone
+  auto loads_landed = [] { __builtin_amdgcn_s_waitcnt(0x0f70); };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const int nk = K / BK;
+  const int fr = lane % 32, fh = lane / 32;
+  fetch(0, 0);
+  loads_landed();
+  __syncthreads();
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < nk) fetch(kt + 1, buf ^ 1);  // the other buffer was last read before the previous barrier
+    const bf16* xs = smem + (size_t)buf * ROWS * BK;
+    const bf16* ws = xs + BM * BK;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      bf16x8 a[TM], b[TN];
+      const int c = 2 * ks + fh;  // the 16-byte chunk of a row that this lane multiplies
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int row = wm + i * 32 + fr;
+        a[i] = *(const bf16x8*)(xs + row * BK + (c ^ ((row >> 1) & 7)) * 8);
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int row = wn + j * 32 + fr;
+        b[j] = *(const bf16x8*)(ws + row * BK + (c ^ (((row + BM) >> 1) & 7)) * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    loads_landed();
+    __syncthreads();
+  }
+  store_tiles<TM, TN, PAIRED>(acc, out, out_is_f32, 0, M, N, m0 + wm, n0 + wn, lane);
+}
+
+template <int BM, int BN, int WM, int WN, bool PAIRED = false>
+static int launch_direct(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
+                         hipStream_t stream) {
+  const size_t lds = (size_t)2 * (BM + BN) * 64 * sizeof(bf16);
+  static bool raised = false;
+  if (lds > 65536 && !raised) {
+    const hipError_t e = hipFuncSetAttribute((const void*)gemm_direct_kernel<BM, BN, WM, WN, PAIRED>,
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    SYN_CHECK(e == hipSuccess, "gemm: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
+    raised = true;
+  }
+  gemm_direct_kernel<BM, BN, WM, WN, PAIRED>
+      <<<tile_grid(M, N, BM, BN), 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K);
+  return 0;
+}
+
+// M > 64: the tile shape by pick_large_tile; loads straight into LDS where K allows it
+template <bool PAIRED>
+static int launch_large(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
+                        hipStream_t stream);
+
 // Which of the large tiles for M > 64: 0 = 256 x 256, 1 = 256 x 192 (both 8 waves, one workgroup a
 // compute unit), 2 = 128 x 128 (4 waves, two workgroups a compute unit, about 15 % less efficient).
 // The estimate is the number of rounds over the 256 compute units times the work of a tile; it
@@ -352,6 +480,20 @@ static int pick_large_tile(int M, int N) {
   if (cost[1] < cost[best]) best = 1;
   if (cost[2] < cost[best]) best = 2;
   return best;
+}
+
+template <bool PAIRED>
+static int launch_large(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
+                        hipStream_t stream) {
+  const int shape = pick_large_tile(M, N);
+  if (K % 64 == 0) {
+    if (shape == 0) return launch_direct<256, 256, 2, 4, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
+    if (shape == 1) return launch_direct<256, 192, 4, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
+    return launch_direct<128, 128, 1, 4, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
+  }
+  if (shape == 0) return launch_tiled<256, 256, 64, 4, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
+  if (shape == 1) return launch_tiled<256, 192, 64, 4, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
+  return launch_tiled<128, 128, 64, 2, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
 }
 
 // ------------------------------------------------------------------ entry point
@@ -396,10 +538,7 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   } else if (M <= 64) {
     rc = launch_tiled<64, 64, 128, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
   } else {
-    const int shape = pick_large_tile(M, N);
-    if (shape == 0) rc = launch_tiled<256, 256, 64, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else if (shape == 1) rc = launch_tiled<256, 192, 64, 4, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else rc = launch_tiled<128, 128, 64, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream);
+    rc = launch_large<false>(xb, wb, out, out_is_f32, M, N, K, stream);
   }
   if (rc) return rc;
   SYN_LAUNCH_CHECK("gemm");
@@ -423,10 +562,7 @@ SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, i
   } else if (M <= 64) {
     rc = launch_tiled<64, 64, 128, 2, 2, true>(xb, wb, out, 0, M, N, K, stream);
   } else {
-    const int shape = pick_large_tile(M, N);
-    if (shape == 0) rc = launch_tiled<256, 256, 64, 4, 2, true>(xb, wb, out, 0, M, N, K, stream);
-    else if (shape == 1) rc = launch_tiled<256, 192, 64, 4, 2, true>(xb, wb, out, 0, M, N, K, stream);
-    else rc = launch_tiled<128, 128, 64, 2, 2, true>(xb, wb, out, 0, M, N, K, stream);
+    rc = launch_large<true>(xb, wb, out, 0, M, N, K, stream);
   }
   if (rc) return rc;
   SYN_LAUNCH_CHECK("gemm_swiglu");

@@ -141,6 +141,7 @@ def test_gemm_f32(ops, M, N, K):
     (65, 130, 104), (128, 128, 32), (200, 300, 1000), (513, 257, 4096),
     (5, 30, 20), (70, 50, 36),          # K no multiple of 8: the plain kernel takes them
     (2048, 6144, 512), (1000, 12300, 136),   # large enough for the 256 x 256 tiles with 8 waves, ragged edges
+    (1000, 12544, 128), (300, 200, 64),   # K a multiple of 64: loads straight into LDS, every tile shape
     (8, 40000, 256), (40, 33000, 72), (64, 50000, 1000),   # wide
     (1, 9000, 520), (1, 70000, 136),                       # one row: W straight from memory, K over the waves
     (8, 70000, 264), (20, 66000, 72),                      # few rows, very wide: 32-row tiles, 256 deep
@@ -189,7 +190,8 @@ def test_gemm_bf16_partial_sums_over_slices_of_k(ops, M, N, K, S):
 
 
 @pytest.mark.parametrize("M,I,K", [(1, 48, 64), (8, 2560, 4096), (7, 112, 1000), (33, 80, 136), (64, 1024, 512),
-                                   (300, 400, 264), (2048, 3072, 256), (1000, 6272, 136), (8, 32784, 72)])
+                                   (300, 400, 264), (2048, 3072, 256), (1000, 6272, 136), (8, 32784, 72),
+                                   (1000, 6272, 128), (300, 400, 192)])
 def test_gemm_with_the_gated_activation_inside(ops, M, I, K):
     """silu(x . Wg^T) * (x . Wu^T) from one product over the rows of Wg and Wu in turns of 16,
     against the two products and the activation in 64-bit; every tile shape of the kernel."""
