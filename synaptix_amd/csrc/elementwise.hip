@@ -357,6 +357,122 @@ __global__ void qk_norm_rope_kv_write_kernel(const TIn* __restrict__ qkv, int n_
   }
 }
 
+// The same for the q and k heads of bf16 rows whose head size is 8 * LPH with LPH = 2, 4, .. 32 lanes
+// a head and whose rotation covers the whole head (or is absent): a lane holds 8 values of a head
+// (16-byte load and store), the sum of squares is reduced over the LPH lanes of the head, and the
+// partner of a rotated pair sits LPH / 2 lanes away.  A block takes 256 / LPH heads of one token.
+template <int LPH>
+__global__ void __launch_bounds__(256)
+qk_heads_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ q_out, bf16* __restrict__ k_pages,
+                const int* __restrict__ page_table, int table_stride, const int* __restrict__ tok_seq,
+                const int* __restrict__ tok_pos, const void* __restrict__ q_gain, const void* __restrict__ k_gain,
+                int gain_is_f32, float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                int n_tokens, int nh, int nkv, int n_active) {
+  constexpr int HD = LPH * 8, HPB = 256 / LPH, half = HD / 2;
+  constexpr int TPB = 4;  // tokens a block takes, their loads in flight together
+  const int head_raw = blockIdx.y * HPB + threadIdx.x / LPH;  // q heads, then k heads
+  const int head = min(head_raw, n_active - 1);                // idle lanes repeat the last head: shuffles need them
+  const int c = threadIdx.x % LPH;                             // which 8 values of the head
+  const bool is_q = head < nh, low = c < LPH / 2;
+  const void* gain = is_q ? q_gain : k_gain;
+  float g[8];
+  if (gain) {
+    if (gain_is_f32) {
+      const float4 g0 = ((const float4*)gain)[c * 2], g1 = ((const float4*)gain)[c * 2 + 1];
+      g[0] = g0.x, g[1] = g0.y, g[2] = g0.z, g[3] = g0.w, g[4] = g1.x, g[5] = g1.y, g[6] = g1.z, g[7] = g1.w;
+    } else {
+      const bf16x8 gb = ((const bf16x8*)gain)[c];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) g[e] = (float)gb[e];
+    }
+  }
+  bf16x8 raw[TPB];
+  int pos[TPB];
+  float4 cs[TPB][2], sn[TPB][2];
+#pragma unroll
+  for (int t = 0; t < TPB; ++t) {
+    const int tok = min((int)blockIdx.x * TPB + t, n_tokens - 1);
+    raw[t] = *(const bf16x8*)(qkv + ((size_t)tok * (nh + 2 * nkv) + head) * HD + c * 8);
+    pos[t] = tok_pos[tok];
+  }
+  if (cos_t) {
+#pragma unroll
+    for (int t = 0; t < TPB; ++t) {
+      const float4* c4 = (const float4*)(cos_t + (size_t)pos[t] * half + (low ? c : c - LPH / 2) * 8);
+      const float4* s4 = (const float4*)(sin_t + (size_t)pos[t] * half + (low ? c : c - LPH / 2) * 8);
+      cs[t][0] = c4[0], cs[t][1] = c4[1], sn[t][0] = s4[0], sn[t][1] = s4[1];
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < TPB; ++t) {
+    const int tok = (int)blockIdx.x * TPB + t;
+    float v[8];
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      v[e] = (float)raw[t][e];
+      ss += v[e] * v[e];
+    }
+    if (gain) {
+#pragma unroll
+      for (int off = LPH / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, SYN_WAVE);
+      const float inv = rsqrtf(ss / (float)HD + eps);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = g[e] * v[e] * inv;
+    }
+    if (cos_t) {
+      const float cc[8] = {cs[t][0].x, cs[t][0].y, cs[t][0].z, cs[t][0].w, cs[t][1].x, cs[t][1].y, cs[t][1].z, cs[t][1].w};
+      const float sc[8] = {sn[t][0].x, sn[t][0].y, sn[t][0].z, sn[t][0].w, sn[t][1].x, sn[t][1].y, sn[t][1].z, sn[t][1].w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float partner = __shfl_xor(v[e], LPH / 2, SYN_WAVE);
+        v[e] = low ? v[e] * cc[e] - partner * sc[e] : v[e] * cc[e] + partner * sc[e];
+      }
+    }
+    if (head_raw >= n_active || tok >= n_tokens) continue;
+    bf16x8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (bf16)v[e];
+    if (is_q) {
+      *(bf16x8*)(q_out + ((size_t)tok * nh + head) * HD + c * 8) = o;
+    } else {
+      const int page = page_table[(size_t)tok_seq[tok] * table_stride + pos[t] / SYN_PAGE];
+      *(bf16x8*)(k_pages + (((size_t)page * nkv + (head - nh)) * SYN_PAGE + pos[t] % SYN_PAGE) * HD + c * 8) = o;
+    }
+  }
+}
+
+// The v heads of the same rows: 64 tokens x 32 dims a block go through LDS, so that a transposed row
+// of a page (64 positions of one dim) is written as one 128-byte piece wherever positions are
+// consecutive.
+#define V_DIMS 32
+__global__ void __launch_bounds__(256)
+v_block_write_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ v_pages, const int* __restrict__ page_table,
+                     int table_stride, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, int n_tokens,
+                     int nh, int nkv, int hd) {
+  constexpr int LD = V_DIMS + 2, PAIRS = V_DIMS / 2;
+  __shared__ __attribute__((aligned(16))) bf16 vtile[64 * LD];
+  __shared__ size_t dst_base[SYN_PAGE];
+  const int tid = threadIdx.x, t0 = blockIdx.x * 64, kvh = blockIdx.y, d0 = blockIdx.z * V_DIMS;
+  const int heads = nh + 2 * nkv;
+  for (int idx = tid; idx < 64 * PAIRS; idx += 256) {
+    const int j = idx / PAIRS, pr = idx % PAIRS;
+    if (t0 + j < n_tokens && d0 + 2 * pr < hd)   // head sizes are even
+      *(uint32_t*)(vtile + j * LD + 2 * pr) =
+          *(const uint32_t*)(qkv + ((size_t)(t0 + j) * heads + nh + nkv + kvh) * hd + d0 + 2 * pr);
+  }
+  if (tid < 64 && t0 + tid < n_tokens) {
+    const int tok = t0 + tid, pos = tok_pos[tok];
+    const int page = page_table[(size_t)tok_seq[tok] * table_stride + pos / SYN_PAGE];
+    dst_base[tid] = ((size_t)page * nkv + kvh) * SYN_PAGE * hd + pos % SYN_PAGE;
+  }
+  __syncthreads();
+  const int j = tid % 64;
+  if (t0 + j < n_tokens)
+    for (int d = tid / 64; d < V_DIMS && d0 + d < hd; d += 4)
+      v_pages[dst_base[j] + (size_t)(d0 + d) * SYN_PAGE] = vtile[j * LD + d];
+}
+
 SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, int n_parts, void* q_out, void* k_pages, void* v_pages,
                                          int is_f32, const int* page_table, int table_stride, const int* tok_seq,
                                          const int* tok_pos, const void* q_gain, const void* k_gain, int gain_is_f32,
@@ -368,6 +484,36 @@ SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, int n_parts, void* q_o
   SYN_CHECK(hd % 2 == 0, "qk_norm_rope_kv_write: head size %d is odd", hd);
   SYN_CHECK((cos_t == nullptr) == (sin_t == nullptr), "qk_norm_rope_kv_write: cos and sin come together");
   SYN_CHECK(n_parts >= 0 && n_parts <= 64, "qk_norm_rope_kv_write: %d partial sums", n_parts);
+  // prompts in bf16: the kernels that move 16 bytes a lane, where the head size and the rotation allow them
+  const int lph = hd / 8;
+  const bool fast = !is_f32 && n_parts == 0 && hd % 8 == 0 && lph >= 2 && lph <= 32 && (lph & (lph - 1)) == 0 &&
+                    (cos_t == nullptr || rot == hd) && (uintptr_t)qkv % 16 == 0 && (uintptr_t)q_out % 16 == 0 &&
+                    (uintptr_t)k_pages % 16 == 0 && (uintptr_t)q_gain % 16 == 0 && (uintptr_t)k_gain % 16 == 0 &&
+                    (uintptr_t)cos_t % 16 == 0 && (uintptr_t)sin_t % 16 == 0;
+  if (fast) {
+    const int n_active = write_kv ? nh + nkv : nh;
+    const int hpb = 256 / lph;
+    const dim3 grid((n_tokens + 3) / 4, (n_active + hpb - 1) / hpb);
+#define SYN_QKH(L)                                                                                                  \
+  qk_heads_kernel<L><<<grid, 256, 0, stream>>>((const bf16*)qkv, (bf16*)q_out, (bf16*)k_pages, page_table,          \
+                                               table_stride, tok_seq, tok_pos, q_gain, k_gain, gain_is_f32, eps,     \
+                                               cos_t, sin_t, n_tokens, nh, nkv, n_active)
+    switch (lph) {
+      case 2: SYN_QKH(2); break;
+      case 4: SYN_QKH(4); break;
+      case 8: SYN_QKH(8); break;
+      case 16: SYN_QKH(16); break;
+      default: SYN_QKH(32); break;
+    }
+#undef SYN_QKH
+    SYN_LAUNCH_CHECK("qk_heads");
+    if (write_kv) {
+      v_block_write_kernel<<<dim3((n_tokens + 63) / 64, nkv, (hd + V_DIMS - 1) / V_DIMS), 256, 0, stream>>>(
+          (const bf16*)qkv, (bf16*)v_pages, page_table, table_stride, tok_seq, tok_pos, n_tokens, nh, nkv, hd);
+      SYN_LAUNCH_CHECK("v_block_write");
+    }
+    return 0;
+  }
   const int wpb = 4;
   const int heads = nh + 2 * nkv;
   dim3 grid(n_tokens, (heads + wpb - 1) / wpb);
