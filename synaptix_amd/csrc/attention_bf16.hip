@@ -349,18 +349,28 @@ constexpr int DEC_MAX_WAVES = HD > 128 ? 4 : 8;  // as many as keep their ~190 r
 
 // Like attn_block for one column block, but every K and V fragment of the block is requested before
 // the first product needs one: a block costs one trip to memory instead of two.
-__device__ __forceinline__ void attn_block_decode(AttnState<1>& st, const QFrag& qf, const bf16* __restrict__ kpage,
-                                                  const bf16* __restrict__ vpage, int key0, int qpos, int lo,
-                                                  int kv_len, float scale, int lane) {
-  const int r16 = lane % 16, g4 = lane / 16;
+struct KvBlock {
   kfrag_t ka[4][KSTEPS];
   bf16x8 va[2][DT];
+};
+
+__device__ __forceinline__ void load_block_decode(KvBlock& b, const bf16* __restrict__ kpage,
+                                                  const bf16* __restrict__ vpage, int lane) {
+  const int r16 = lane % 16, g4 = lane / 16;
 #pragma unroll
-  for (int t = 0; t < 4; ++t) load_row(ka[t], kpage + (size_t)tile_row_key(t, r16) * HD, lane);
+  for (int t = 0; t < 4; ++t) load_row(b.ka[t], kpage + (size_t)tile_row_key(t, r16) * HD, lane);
 #pragma unroll
   for (int h = 0; h < 2; ++h)
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) va[h][dt] = *(const bf16x8*)(vpage + (size_t)(dt * 16 + r16) * SYN_PAGE + h * 32 + 8 * g4);
+    for (int dt = 0; dt < DT; ++dt)
+      b.va[h][dt] = *(const bf16x8*)(vpage + (size_t)(dt * 16 + r16) * SYN_PAGE + h * 32 + 8 * g4);
+}
+
+__device__ __forceinline__ void attn_block_decode(AttnState<1>& st, const QFrag& qf, const KvBlock& blk, int key0,
+                                                  int qpos, int lo, int kv_len, float scale, int lane) {
+  const int g4 = lane / 16;
+  const auto& ka = blk.ka;
+  const auto& va = blk.va;
 
   f32x4 s[4];
 #pragma unroll
@@ -420,12 +430,36 @@ __device__ __forceinline__ void attn_block_decode(AttnState<1>& st, const QFrag&
   }
 }
 
+// What the kernel needs to take q, k and v of the new tokens from the fused projection itself
+// instead of from a kernel before it: rows [q heads | k heads | v heads] of one token a sequence, as
+// bf16 (n_parts == 0) or as n_parts float partial sums of a product cut along K.
+struct QkvIntake {
+  const void* qkv;
+  int n_parts;
+  size_t part_stride;
+  const void* q_gain;  // RMSNorm gains of the q and k heads, or nullptr
+  const void* k_gain;
+  int gain_is_f32;
+  float eps;
+  const float* cos_t;  // rotation tables [positions][rot / 2], or nullptr
+  const float* sin_t;
+  int rot;
+  int own_kv;  // the layer writes its k and v into the cache (else it reads a cache that another layer wrote)
+};
+
+// FUSED: the workgroup first makes its q heads from the projection (sum of the partial sums,
+// RMSNorm, rotation: all in 32-bit, rounded once to bf16 into LDS).  With own_kv the workgroup of
+// split 0 makes the new k and v of its kv head likewise, writes them into the cache for later steps,
+// and adds the new key to its result as one more partial state; the loop over the cache then covers
+// the older keys only, so nothing is read that this launch writes.
+template <bool FUSED>
 __global__ void __launch_bounds__(DEC_MAX_WAVES * SYN_WAVE)
-attn_decode_split_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages,
-                         const bf16* __restrict__ v_pages, const int* __restrict__ page_table, int table_stride,
-                         const int* __restrict__ seq_len, float* __restrict__ partial, bf16* __restrict__ out,
-                         float scale, int window, int nh, int nkv, int n_splits, int cols_alloc) {
-  // LDS: sm[waves][16] running maxima, sl[waves][16] sums, so[waves][cols_alloc][HD + 4] outputs
+attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages, bf16* __restrict__ v_pages,
+                         const int* __restrict__ page_table, int table_stride, const int* __restrict__ seq_len,
+                         float* __restrict__ partial, bf16* __restrict__ out, float scale, int window, int nh, int nkv,
+                         int n_splits, int cols_alloc, QkvIntake in) {
+  // LDS: sm[waves][16] running maxima, sl[waves][16] sums, so[waves][cols_alloc][HD + 4] outputs;
+  // FUSED: then xs[waves][HD] floats, snew[16] scores of the new key, qs[cols_alloc][HD], knew[HD], vnew[HD] bf16
   extern __shared__ float dec_lds[];
   const int n_waves = blockDim.x / SYN_WAVE;
   float* sm = dec_lds;
@@ -441,18 +475,140 @@ attn_decode_split_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
   const int hg = chunk * 16 + col;  // head inside the group
   const bool valid = hg < g;
   const int n_cols = min(16, g - chunk * 16);
+  const bool new_key = FUSED && in.own_kv;            // the newest key is not read from the cache
+  const bool adds_new = new_key && split == 0;        // this workgroup makes it and adds it
 
-  QFrag qf;
+  // keys read from the cache: all of them, or all but the newest; the blocks of this split; the first
+  // block of this wave is requested at once, before the workgroup prepares its q heads
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-  load_q(qf, valid ? q + ((size_t)seq * nh + kvh * g + hg) * HD : nullptr, lane);
-  AttnState<1> st;
-  attn_init(st);
-  const int b_lo = lo / SYN_PAGE, b_hi = pos / SYN_PAGE;
+  const int n_old = new_key ? kv_len - 1 : kv_len;
+  const int q_lim = new_key ? pos - 1 : pos;  // the last key position that the loop may see
+  const int b_lo = lo / SYN_PAGE, b_hi = n_old > 0 ? (n_old - 1) / SYN_PAGE : b_lo - 1;
   const int per = (b_hi - b_lo + n_splits) / n_splits;  // ceil((b_hi - b_lo + 1) / n_splits)
   const int b0 = b_lo + split * per, b1 = min(b_hi + 1, b0 + per);
+  auto page_of = [&](int kb) {
+    return ((size_t)page_table[(size_t)seq * table_stride + kb] * nkv + kvh) * SYN_PAGE * HD;
+  };
+  KvBlock blk;
+  if (b0 + wave < b1) {
+    const size_t base = page_of(b0 + wave);
+    load_block_decode(blk, k_pages + base, v_pages + base, lane);
+  }
+
+  float* xs = so + (size_t)n_waves * cols_alloc * SO_LD;
+  float* snew = xs + n_waves * HD;
+  bf16* qs = (bf16*)(snew + 16);
+  bf16* knew = qs + cols_alloc * HD;
+  bf16* vnew = knew + HD;
+  if constexpr (FUSED) {
+    const int heads = nh + 2 * nkv, half = in.rot / 2;
+    const int n_items = n_cols + (adds_new ? 2 : 0);  // q heads of this chunk, then k and v of the kv head
+    for (int it0 = 0; it0 < n_items; it0 += n_waves) {  // the same number of rounds for every wave: barriers inside
+      const int it = it0 + wave;
+      const bool active = it < n_items;
+      const int kind = it < n_cols ? 0 : (it == n_cols ? 1 : 2);
+      const int head = kind == 0 ? kvh * g + chunk * 16 + it : (kind == 1 ? nh + kvh : nh + nkv + kvh);
+      float* x = xs + wave * HD;
+      // the angles of this lane's dims are requested now, together with the values, not after the barrier
+      constexpr int PER = (HD + 2 * SYN_WAVE - 1) / (2 * SYN_WAVE);
+      float cs[PER][2], sn[PER][2];
+      const bool rotate = active && kind != 2 && in.cos_t != nullptr;
+      if (rotate) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+          const int d = 2 * lane + i * 2 * SYN_WAVE;
+#pragma unroll
+          for (int e = 0; e < 2; ++e) {
+            const bool in_rot = d + e < in.rot && d + e < HD;
+            const int idx = d + e < half ? d + e : d + e - half;
+            cs[i][e] = in_rot ? in.cos_t[(size_t)pos * half + idx] : 1.f;
+            sn[i][e] = in_rot ? in.sin_t[(size_t)pos * half + idx] : 0.f;
+          }
+        }
+      }
+      if (active) {
+        const size_t at = ((size_t)seq * heads + head) * HD;
+        float ss = 0.f;
+        for (int d = 2 * lane; d < HD; d += 2 * SYN_WAVE) {
+          float v0, v1;
+          if (in.n_parts > 0) {
+            const float* src = (const float*)in.qkv + at + d;
+            v0 = 0.f, v1 = 0.f;
+            for (int p0 = 0; p0 < in.n_parts; p0 += 8) {  // eight partial sums in flight together, added in order
+              float2 t[8];
+#pragma unroll
+              for (int u = 0; u < 8; ++u)
+                t[u] = p0 + u < in.n_parts ? *(const float2*)(src + (size_t)(p0 + u) * in.part_stride) : make_float2(0.f, 0.f);
+#pragma unroll
+              for (int u = 0; u < 8; ++u) v0 += t[u].x, v1 += t[u].y;
+            }
+          } else {
+            const bf16* src = (const bf16*)in.qkv + at;
+            v0 = (float)src[d], v1 = (float)src[d + 1];
+          }
+          x[d] = v0, x[d + 1] = v1;
+          ss += v0 * v0 + v1 * v1;
+        }
+        const void* gain = kind == 0 ? in.q_gain : (kind == 1 ? in.k_gain : nullptr);
+        if (gain) {
+          ss = wave_sum(ss);
+          const float inv = rsqrtf(ss / (float)HD + in.eps);
+          for (int d = 2 * lane; d < HD; d += 2 * SYN_WAVE) {
+            x[d] = load_gain(gain, in.gain_is_f32, d) * x[d] * inv;
+            x[d + 1] = load_gain(gain, in.gain_is_f32, d + 1) * x[d + 1] * inv;
+          }
+        }
+      }
+      __syncthreads();  // lanes read what other lanes of their wave wrote
+      if (active) {
+        auto rotated = [&](int d, float c, float sine) {
+          float o = x[d];
+          if (rotate && d < in.rot) o = d < half ? x[d] * c - x[d + half] * sine : x[d] * c + x[d - half] * sine;
+          return (bf16)o;
+        };
+        bf16* dst = kind == 0 ? qs + it * HD : (kind == 1 ? knew : vnew);
+        const size_t page_base = ((size_t)page_table[(size_t)seq * table_stride + pos / SYN_PAGE] * nkv + kvh) * SYN_PAGE * HD;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+          const int d = 2 * lane + i * 2 * SYN_WAVE;
+          if (d >= HD) break;
+          const bf16 o0 = rotated(d, cs[i][0], sn[i][0]), o1 = rotated(d + 1, cs[i][1], sn[i][1]);
+          dst[d] = o0, dst[d + 1] = o1;
+          if (kind == 1) {
+            bf16* row = k_pages + page_base + (size_t)(pos % SYN_PAGE) * HD;
+            row[d] = o0, row[d + 1] = o1;
+          } else if (kind == 2) {
+            bf16* colp = v_pages + page_base + pos % SYN_PAGE;
+            colp[(size_t)d * SYN_PAGE] = o0, colp[(size_t)(d + 1) * SYN_PAGE] = o1;
+          }
+        }
+      }
+      __syncthreads();  // xs is written again in the next round; qs, knew, vnew are read below
+    }
+    if (adds_new) {
+      // the new key's score for every head of the chunk, from the rounded q and k as the products see them
+      for (int c = wave; c < n_cols; c += n_waves) {
+        float dot = 0.f;
+        for (int d = lane; d < HD; d += SYN_WAVE) dot += (float)qs[c * HD + d] * (float)knew[d];
+        dot = wave_sum(dot);
+        if (lane == 0) snew[c] = dot * scale;
+      }
+    }
+  }
+
+  QFrag qf;
+  if constexpr (FUSED)
+    load_q(qf, valid ? qs + col * HD : nullptr, lane);
+  else
+    load_q(qf, valid ? q + ((size_t)seq * nh + kvh * g + hg) * HD : nullptr, lane);
+  AttnState<1> st;
+  attn_init(st);
   for (int kb = b0 + wave; kb < b1; kb += n_waves) {
-    const size_t base = ((size_t)page_table[(size_t)seq * table_stride + kb] * nkv + kvh) * SYN_PAGE * HD;
-    attn_block_decode(st, qf, k_pages + base, v_pages + base, kb * SYN_PAGE, valid ? pos : -1, lo, kv_len, scale, lane);
+    if (kb != b0 + wave) {  // the first block is already on its way
+      const size_t base = page_of(kb);
+      load_block_decode(blk, k_pages + base, v_pages + base, lane);
+    }
+    attn_block_decode(st, qf, blk, kb * SYN_PAGE, valid ? q_lim : -1, lo, n_old, scale, lane);
   }
   float l = st.l[0];
   l += __shfl_xor(l, 16, SYN_WAVE);
@@ -470,7 +626,7 @@ attn_decode_split_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
   __syncthreads();
   for (int idx = threadIdx.x; idx < n_cols * HD; idx += blockDim.x) {
     const int c = idx / HD, d = idx % HD;
-    float m = -INFINITY;
+    float m = adds_new ? snew[c] : -INFINITY;
     for (int w = 0; w < n_waves; ++w) m = fmaxf(m, sm[w * 16 + c]);
     float acc = 0.f, lsum = 0.f;
     for (int w = 0; w < n_waves; ++w) {
@@ -479,6 +635,11 @@ attn_decode_split_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
       const float f = __expf(mw - m);
       acc += f * so[((size_t)w * cols_alloc + c) * SO_LD + d];
       lsum += f * sl[w * 16 + c];
+    }
+    if (adds_new) {  // the new key: weight exp(score - m), value vnew
+      const float f = __expf(snew[c] - m);
+      acc += f * (float)vnew[d];
+      lsum += f;
     }
     const int head = kvh * g + chunk * 16 + c;
     if (n_splits == 1) {
@@ -532,10 +693,9 @@ attn_decode_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ o
 }
 
 // workspace: n_seqs * nh * n_splits * (HD + 2) floats (unused with one split)
-SYN_EXPORT int syn_attention_decode_bf16(const void* q, const void* k_pages, const void* v_pages,
-                                         const int* page_table, int table_stride, const int* seq_len, int n_seqs,
-                                         void* out, float* workspace, int n_splits, float scale, int window, int nh,
-                                         int nkv, int hd, hipStream_t stream) {
+static int launch_decode(const void* q, const QkvIntake* in, void* k_pages, void* v_pages, const int* page_table,
+                         int table_stride, const int* seq_len, int n_seqs, void* out, float* workspace, int n_splits,
+                         float scale, int window, int nh, int nkv, int hd, hipStream_t stream) {
   SYN_CHECK(hd == HD, "attention_decode: library built for head size %d, called with %d", HD, hd);
   SYN_CHECK(n_seqs > 0 && nh > 0 && nkv > 0 && n_splits > 0, "attention_decode: empty input");
   SYN_CHECK(nh % nkv == 0, "attention_decode: %d heads do not divide into %d kv heads", nh, nkv);
@@ -544,19 +704,62 @@ SYN_EXPORT int syn_attention_decode_bf16(const void* q, const void* k_pages, con
   // waves a workgroup: as many as the LDS for their states allows (up to 8), but no more than make
   // about 2,048 waves in all: at large batches four waves a workgroup are plenty
   const int cols_alloc = nh / nkv < 16 ? nh / nkv : 16;
+  auto lds_for = [&](int waves) {
+    size_t b = (size_t)waves * (32 + (size_t)cols_alloc * (HD + 4)) * sizeof(float);
+    if (in) b += ((size_t)waves * HD + 16) * sizeof(float) + (size_t)(cols_alloc + 2) * HD * sizeof(bf16);
+    return b;
+  };
   int waves = DEC_MAX_WAVES;
-  while (waves > 2 && ((size_t)waves * (32 + (size_t)cols_alloc * (HD + 4)) * sizeof(float) > 64 * 1024 ||
-                       (long)n_seqs * nkv * chunks * n_splits * waves > 2048))
-    waves /= 2;
-  if (waves < 4 && (size_t)4 * (32 + (size_t)cols_alloc * (HD + 4)) * sizeof(float) <= 64 * 1024) waves = 4;
-  const size_t lds = (size_t)waves * (32 + (size_t)cols_alloc * (HD + 4)) * sizeof(float);
-  attn_decode_split_kernel<<<dim3(n_seqs, nkv * chunks, n_splits), waves * SYN_WAVE, lds, stream>>>(
-      (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, page_table, table_stride, seq_len, workspace,
-      (bf16*)out, scale, window, nh, nkv, n_splits, cols_alloc);
+  while (waves > 2 && (lds_for(waves) > 64 * 1024 || (long)n_seqs * nkv * chunks * n_splits * waves > 2048)) waves /= 2;
+  if (waves < 4 && lds_for(4) <= 64 * 1024) waves = 4;
+  const size_t lds = lds_for(waves);
+  SYN_CHECK(lds <= 64 * 1024, "attention_decode: %zu bytes of LDS for %d heads a group", lds, nh / nkv);
+  const dim3 grid(n_seqs, nkv * chunks, n_splits);
+  if (in)
+    attn_decode_split_kernel<true><<<grid, waves * SYN_WAVE, lds, stream>>>(
+        nullptr, (bf16*)k_pages, (bf16*)v_pages, page_table, table_stride, seq_len, workspace, (bf16*)out, scale,
+        window, nh, nkv, n_splits, cols_alloc, *in);
+  else
+    attn_decode_split_kernel<false><<<grid, waves * SYN_WAVE, lds, stream>>>(
+        (const bf16*)q, (bf16*)k_pages, (bf16*)v_pages, page_table, table_stride, seq_len, workspace, (bf16*)out,
+        scale, window, nh, nkv, n_splits, cols_alloc, QkvIntake{});
   SYN_LAUNCH_CHECK("attention_decode_split");
   if (n_splits > 1) {
     attn_decode_merge_kernel<<<n_seqs * nh, SYN_WAVE, 0, stream>>>(workspace, (bf16*)out, n_splits);
     SYN_LAUNCH_CHECK("attention_decode_merge");
   }
   return 0;
+}
+
+SYN_EXPORT int syn_attention_decode_bf16(const void* q, const void* k_pages, const void* v_pages,
+                                         const int* page_table, int table_stride, const int* seq_len, int n_seqs,
+                                         void* out, float* workspace, int n_splits, float scale, int window, int nh,
+                                         int nkv, int hd, hipStream_t stream) {
+  return launch_decode(q, nullptr, (void*)k_pages, (void*)v_pages, page_table, table_stride, seq_len, n_seqs, out,
+                       workspace, n_splits, scale, window, nh, nkv, hd, stream);
+}
+
+// The same for one new token a sequence whose q, k and v come straight from the fused projection:
+// qkv [n_seqs, (nh + 2 nkv) * hd] in bf16 (n_parts == 0), or n_parts float partial sums of that
+// shape one after another.  q/k RMSNorm (gains may be null), rotation at position seq_len - 1 (tables
+// may be null; `rot` dims rotate), and with own_kv the write of the new k and v into the cache happen
+// inside the attention kernel.
+SYN_EXPORT int syn_attention_decode_fused_bf16(const void* qkv, int n_parts, void* k_pages, void* v_pages,
+                                               const int* page_table, int table_stride, const int* seq_len,
+                                               int n_seqs, void* out, float* workspace, int n_splits, float scale,
+                                               int window, int nh, int nkv, int hd, const void* q_gain,
+                                               const void* k_gain, int gain_is_f32, float eps, const float* cos_t,
+                                               const float* sin_t, int rot, int own_kv, hipStream_t stream) {
+  SYN_CHECK(rot % 2 == 0 && rot >= 0 && rot <= hd, "attention_decode_fused: rotary size %d does not fit head size %d",
+            rot, hd);
+  SYN_CHECK((cos_t == nullptr) == (sin_t == nullptr), "attention_decode_fused: cos and sin come together");
+  SYN_CHECK(n_parts >= 0 && n_parts <= 64, "attention_decode_fused: %d partial sums", n_parts);
+  QkvIntake in;
+  in.qkv = qkv;
+  in.n_parts = n_parts;
+  in.part_stride = (size_t)n_seqs * (nh + 2 * nkv) * hd;
+  in.q_gain = q_gain, in.k_gain = k_gain, in.gain_is_f32 = gain_is_f32, in.eps = eps;
+  in.cos_t = cos_t, in.sin_t = sin_t, in.rot = rot, in.own_kv = own_kv;
+  return launch_decode(nullptr, &in, k_pages, v_pages, page_table, table_stride, seq_len, n_seqs, out, workspace,
+                       n_splits, scale, window, nh, nkv, hd, stream);
 }

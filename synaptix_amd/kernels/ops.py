@@ -302,6 +302,52 @@ def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspa
           int(window or 0), nh, nkv, hd, _stream())
 
 
+def attention_decode_fused_bf16(qkv, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
+                                n_heads, n_kv_heads, head_dim, q_gain, k_gain, eps, cos, sin, write_kv=True):
+    """attention_decode_bf16 for one new token a sequence whose q, k and v come straight from the
+    fused projection: qkv [B, (nh + 2 nkv) * hd] in bf16, or float partial sums [S, B, ...] that are
+    added first.  The q/k RMSNorm (if gains are given), the rotation at position seq_len - 1 (if
+    tables are given) and, with write_kv, the write of the new k and v into the cache pages happen
+    inside the attention kernel; seq_len [B] counts the new token."""
+    nh, nkv, hd = n_heads, n_kv_heads, head_dim
+    width = (nh + 2 * nkv) * hd
+    n_parts = 0
+    if qkv.dim() == 3:
+        n_parts = qkv.shape[0]
+        _need(qkv, "attention_decode_fused.qkv", _F32, (n_parts, None, width))
+        B = qkv.shape[1]
+    else:
+        _need(qkv, "attention_decode_fused.qkv", _BF16, (None, width))
+        B = qkv.shape[0]
+    _check_pages(k_pages, v_pages, _BF16, nkv, hd, "attention_decode_fused")
+    _need(page_table, "attention_decode_fused.page_table", _I32, (None, None))
+    if page_table.shape[0] < B:
+        raise KernelError(f"attention_decode_fused: page table has {page_table.shape[0]} rows for {B} sequences")
+    _need(seq_len, "attention_decode_fused.seq_len", _I32, (B,))
+    _need(out, "attention_decode_fused.out", _BF16, (B, nh * hd))
+    _need(workspace, "attention_decode_fused.workspace", _F32)
+    if workspace.numel() < B * nh * n_splits * (hd + 2):
+        raise KernelError(f"attention_decode_fused: workspace of {workspace.numel()} floats is too small")
+    gain_f32 = 0
+    if (q_gain is None) != (k_gain is None):
+        raise KernelError("attention_decode_fused: q and k gains come together")
+    if q_gain is not None:
+        _need(q_gain, "attention_decode_fused.q_gain", (_BF16, _F32), (hd,))
+        _need(k_gain, "attention_decode_fused.k_gain", q_gain.dtype, (hd,))
+        gain_f32 = _is_f32(q_gain)
+    rot = 0
+    if cos is not None:
+        _need(cos, "attention_decode_fused.cos", _F32, (None, None))
+        _need(sin, "attention_decode_fused.sin", _F32, tuple(cos.shape))
+        rot = 2 * cos.shape[1]
+        if rot > hd:
+            raise KernelError(f"attention_decode_fused: rotary size {rot} exceeds head size {hd}")
+    _call(_attn_lib(hd), "syn_attention_decode_fused_bf16", _ptr(qkv), n_parts, _ptr(k_pages), _ptr(v_pages),
+          _ptr(page_table), page_table.shape[1], _ptr(seq_len), B, _ptr(out), _ptr(workspace), int(n_splits),
+          ctypes.c_float(scale), int(window or 0), nh, nkv, hd, _ptr(q_gain), _ptr(k_gain), gain_f32,
+          ctypes.c_float(eps), _ptr(cos), _ptr(sin), rot, 1 if write_kv else 0, _stream())
+
+
 # ----------------------------------------------------------------------------- sampling
 
 def sample_rows(logits, temperature, uniform, out):

@@ -83,14 +83,22 @@ class GqaAttention(Mixer):
             raise ValueError(f"position {ctx.max_position} is beyond the position encoding's capacity {cap}")
         qkv = linear_for_sum(h, self.w_qkv) if ops.gemm_slices(N, self.w_qkv.shape[0], self.hidden, act) > 1 \
             else linear(h, self.w_qkv, act)             # partial sums over slices of K, or the plain product
-        q = torch.empty((N, nh * hd), dtype=act, device=h.device)
         cos, sin = self.position.tables(h.device)
         table = ctx.page_table(cache.group)
+        o = torch.empty((N, nh * hd), dtype=act, device=h.device)
+        window = self.window or 0
+        if act == torch.bfloat16 and ctx.one_token_each:
+            # single tokens: the attention kernel takes q, k and v from the projection itself
+            splits = ctx.decode_splits(nkv, cache.group)
+            work = ctx.scratch("attention_decode", N * nh * splits * (hd + 2))
+            ops.attention_decode_fused_bf16(qkv, cache.k_pages, cache.v_pages, table, ctx.seq_len, o, work, splits,
+                                            self.scale, window, nh, nkv, hd, self.q_gain, self.k_gain,
+                                            self.qk_norm_eps or 0.0, cos, sin, write_kv=owner)
+            return linear_for_sum(o, self.w_o)
+        q = torch.empty((N, nh * hd), dtype=act, device=h.device)
         ops.qk_norm_rope_kv_write(qkv, q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos,
                                   self.q_gain, self.k_gain, self.qk_norm_eps or 0.0, cos, sin, nh, nkv, hd,
                                   write_kv=owner)
-        o = torch.empty((N, nh * hd), dtype=act, device=h.device)
-        window = self.window or 0
         if act == torch.float32:
             ops.attention_f32(q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos, o, self.scale, window,
                               nh, nkv, hd)

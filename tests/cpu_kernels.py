@@ -158,6 +158,18 @@ def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspa
         out[b] = o.reshape(-1).to(out.dtype)
 
 
+def attention_decode_fused_bf16(qkv, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
+                                n_heads, n_kv_heads, head_dim, q_gain, k_gain, eps, cos, sin, write_kv=True):
+    B = qkv.shape[-2]
+    q = torch.empty((B, n_heads * head_dim), dtype=torch.bfloat16)
+    tok_seq = torch.arange(B, dtype=torch.int32)
+    tok_pos = (seq_len - 1).to(torch.int32)
+    qk_norm_rope_kv_write(qkv, q, k_pages, v_pages, page_table, tok_seq, tok_pos, q_gain, k_gain, eps, cos, sin,
+                          n_heads, n_kv_heads, head_dim, write_kv=write_kv)
+    attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
+                          n_heads, n_kv_heads, head_dim)
+
+
 def sample_rows(logits, temperature, uniform, out):
     for r in range(logits.shape[0]):
         x = logits[r]
@@ -174,7 +186,7 @@ def sample_rows(logits, temperature, uniform, out):
 
 
 ALL = ["embed", "add_rmsnorm", "rmsnorm_rows", "swiglu", "gemm", "gemm_swiglu", "gemm_slices", "qk_norm_rope_kv_write", "attention_f32",
-       "attention_prefill_bf16", "decode_splits", "attention_decode_bf16", "sample_rows"]
+       "attention_prefill_bf16", "decode_splits", "attention_decode_bf16", "attention_decode_fused_bf16", "sample_rows"]
 
 
 def install(monkeypatch):

@@ -380,6 +380,58 @@ def test_attention_decode_bf16(ops, nh, nkv, hd, lens, window, splits):
     close(out, want, 2e-2, 1e-2, what="attention decode bf16")
 
 
+@pytest.mark.parametrize("nh,nkv,hd,rot,norm,lens,window,splits,parts,own", [
+    (4, 2, 16, 16, True, [1, 5, 64, 65, 200], 0, 1, 0, True),        # a first token, page edges
+    (8, 2, 128, 128, True, [700, 33, 129], 0, 4, 8, True),           # float partial sums, splits
+    (6, 2, 48, 32, True, [300, 64], 0, 3, 3, True),                  # partial rotation, head size 48
+    (4, 1, 64, 64, False, [500, 2], 100, 2, 0, True),                # no q/k norm, a window
+    (40, 2, 32, 0, True, [90, 300], 0, 2, 2, True),                  # no rotation, 20 heads a group (two chunks)
+    (8, 4, 128, 128, True, [257, 1000], 0, 8, 4, False),             # reads a cache that another layer wrote
+])
+def test_attention_decode_with_qkv_intake(ops, nh, nkv, hd, rot, norm, lens, window, splits, parts, own):
+    """Decode attention that makes q, k and v from the fused projection itself equals the q/k kernel
+    followed by plain decode attention: the same outputs and the same cache contents afterwards."""
+    B, heads = len(lens), nh + 2 * nkv
+    width = max((T + 63) // 64 for T in lens) + 2
+    table = shuffled_table(B, width, 5)
+    k, v = make_cache(B * width, nkv, hd, BF16, 60)
+    fill_sequences(k, v, table, lens, nkv, hd, BF16, 61)
+    qkv_full = rnd((B, heads * hd), 62, F32)
+    if parts:
+        cut = torch.rand((parts, 1, 1), generator=torch.Generator().manual_seed(63)) + 0.1
+        qkv = (qkv_full[None] * (cut / cut.sum())).contiguous()       # float partial sums that add up to it
+    else:
+        qkv = qkv_full.to(BF16)
+    qg = (1 + 0.2 * rnd((hd,), 64)).to(BF16) if norm else None
+    kg = (1 + 0.2 * rnd((hd,), 65)).to(BF16) if norm else None
+    cos = sin = None
+    if rot:
+        ang = torch.arange(max(lens) + 1, dtype=F32)[:, None] * (0.3 / (1 + torch.arange(rot // 2, dtype=F32)))[None, :]
+        cos, sin = torch.cos(ang), torch.sin(ang)
+    seq_len = torch.tensor(lens, dtype=I32)
+    tok_seq, tok_pos = torch.arange(B, dtype=I32), seq_len - 1
+    scale = 1 / math.sqrt(hd)
+    # the two-kernel way, on the CPU reference
+    k_ref, v_ref = k.clone(), v.clone()
+    q_ref = torch.empty((B, nh * hd), dtype=BF16)
+    ref.qk_norm_rope_kv_write(qkv, q_ref, k_ref, v_ref, table, tok_seq, tok_pos, qg, kg, 1e-5, cos, sin, nh, nkv, hd,
+                              write_kv=own)
+    want = torch.empty((B, nh * hd), dtype=F32)
+    ref.attention_f32(q_ref.float(), k_ref.float(), v_ref.float(), table, tok_seq, tok_pos, want, scale, window, nh, nkv, hd)
+    d = lambda t: None if t is None else t.to(DEV)
+    kd, vd = d(k), d(v)
+    out = torch.empty((B, nh * hd), dtype=BF16, device=DEV)
+    work = torch.empty(B * nh * splits * (hd + 2), dtype=F32, device=DEV)
+    ops.attention_decode_fused_bf16(d(qkv), kd, vd, d(table), d(seq_len), out, work, splits, scale, window, nh, nkv, hd,
+                                    d(qg), d(kg), 1e-5, d(cos), d(sin), write_kv=own)
+    close(out, want, 2e-2, 1e-2, what="decode attention with q/k/v intake")
+    # the cache afterwards: the new rows written (or nothing touched)
+    close(kd, k_ref.float(), 2e-2, 1e-2, what="k pages after the step")
+    close(vd, v_ref.float(), 2e-2, 1e-2, what="v pages after the step")
+    if not own:
+        assert torch.equal(kd.cpu(), k) and torch.equal(vd.cpu(), v)
+
+
 def test_attention_far_key_stands_out(ops):
     """One key among hundreds is made to dominate: the output must be that key's value, in every
     kernel.  A kernel that loses a page, a split or the cache's start would not show it with
