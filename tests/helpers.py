@@ -37,8 +37,14 @@ MID_D = dict(num_hidden_layers=2, hidden_size=2048, num_attention_heads=16, num_
 # power routine computes them: at position 6000 a last-bit difference in a frequency would
 # otherwise be an angle error of 4e-4, above the 32-bit tolerance of these tests.
 LONG_L = dict(TINY_A, rope_theta=65536.0, max_position_embeddings=16384)
-SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3, "L": 4}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": MID_D, "L": LONG_L}
+# Awkward sizes: a width that is no multiple of 8 (the MFMA products refuse it: plain products), a
+# head size with no kernel built ahead of time and no power of two, as many kv heads as heads, an
+# intermediate size that cannot be paired, an odd vocabulary.
+ODD_E = dict(num_hidden_layers=2, hidden_size=52, num_attention_heads=2, num_key_value_heads=2, head_dim=80,
+             intermediate_size=30, vocab_size=101, rope_theta=2e4, rms_norm_eps=2e-5, max_position_embeddings=300,
+             tie_word_embeddings=True, eos_token_id=None, bos_token_id=None)
+SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3, "L": 4, "E": 5}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": MID_D, "L": LONG_L, "E": ODD_E}
 
 _made = {}
 _tmp = None

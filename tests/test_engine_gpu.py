@@ -63,6 +63,15 @@ def test_long_decoding(name, n, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_awkward_sizes(dtype):
+    """A width of 52, head size 80, intermediate size 30, vocabulary 101: every kernel either takes
+    the size or hands it to its general form; whole, one by one, and in unequal batches."""
+    scenarios.whole(make_engine, "E", dtype)
+    scenarios.last_tokens_one_by_one(make_engine, "E", dtype, tail=32)
+    scenarios.unequal_batches(make_engine, "E", dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["A", "C"])
 def test_wide_batch(name, dtype):
     scenarios.wide_batch(make_engine, name, dtype)
