@@ -24,7 +24,7 @@ import torch
 
 from ..kernels import runtime as rt
 from ..parts.base import KvNeed, StateNeed
-from .pages import PAGE_TOKENS, CacheFull, CacheError, pages_for
+from .pages import PAGE_TOKENS, CacheError, pages_for
 
 
 @dataclass

@@ -14,7 +14,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
-from ..cache import SequenceCache, CacheFull, CacheError, PAGE_TOKENS, pages_for
+from ..cache import SequenceCache, CacheError, PAGE_TOKENS, pages_for
 from ..config.registry import load_config, resolve_architecture
 from ..kernels import ops
 from ..weights import FolderSource, RandomSource, load_weights

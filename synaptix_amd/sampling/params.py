@@ -2,7 +2,7 @@
 GenerationConfig (crates/synaptix-models/llm/common/src/generate.rs:17-56)."""
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Optional
 
 

@@ -7,7 +7,6 @@ Each function has the signature and the meaning of its namesake in synaptix_amd.
 """
 from __future__ import annotations
 
-import math
 
 import numpy as np
 import torch

@@ -5,7 +5,7 @@ from __future__ import annotations
 
 import torch
 
-from helpers import CONFIGS, plain_logits, plain_model, random_tokens, assert_logits_close, model_folder
+from helpers import CONFIGS, plain_logits, plain_model, random_tokens, assert_logits_close
 from synaptix_amd.engine.generate import generate, GenerationConfig
 import plain_qwen3 as P
 

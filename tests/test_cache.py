@@ -4,7 +4,7 @@ import random
 import pytest
 import torch
 
-from synaptix_amd.cache import SequenceCache, PagePool, CacheFull, CacheError, PAGE_TOKENS, pages_for
+from synaptix_amd.cache import SequenceCache, PagePool, CacheFull, CacheError, pages_for
 from synaptix_amd.parts import KvNeed, StateNeed
 
 

@@ -1,10 +1,9 @@
 """Configuration and registry (no GPU)."""
 import json
-import os
 
 import pytest
 
-from synaptix_amd import Qwen3Config, ConfigError, load_config, known_architectures, register_architecture
+from synaptix_amd import Qwen3Config, ConfigError, load_config, known_architectures
 from synaptix_amd.config import resolve_architecture
 from helpers import TINY_A, TINY_B
 

@@ -2,7 +2,6 @@
 request alone and whole; with the last 32 tokens one by one; in batches of unequal lengths one
 after another (slots used again); long decoding; the first tokens; generation; the replay
 program as a user runs it."""
-import json
 import os
 
 import numpy as np

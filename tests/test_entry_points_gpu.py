@@ -1,6 +1,5 @@
 """Greedy generation through the entry points a user has: the Python pipeline and the command line."""
 import json
-import os
 import subprocess
 import sys
 

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 import cpu_kernels
-from synaptix_amd.cache import SequenceCache, CacheFull
+from synaptix_amd.cache import SequenceCache
 from synaptix_amd.engine.generate import generate, plan_batch, GenerationConfig
 from synaptix_amd.parts import KvNeed
 from synaptix_amd.sampling import Philox4x32, SequenceSampler, apply_filters

@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import plain_qwen3 as P
-from helpers import plain_model, random_tokens, CONFIGS
+from helpers import plain_model, random_tokens
 
 F64 = torch.float64
 
