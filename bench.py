@@ -51,6 +51,7 @@ def main() -> int:
 
     import torch
     from synaptix_amd import Qwen3Config, Engine
+    from synaptix_amd.kernels import ops
 
     torch.manual_seed(0)
     cfg = Qwen3Config.from_dict({**QWEN3_8B, "num_hidden_layers": args.layers})
@@ -131,6 +132,11 @@ def main() -> int:
             points[f"decode_b{b}_hbm_frac"] = round(step_bytes / step_s / 1e9 / HBM_PEAK_GBS, 4)
 
     achieved = main_bytes / main_step / 1e9
+    # what this machine gives to kernels that only read, or only multiply: measured, beside the vendor's peaks
+    read_gbs, mfma_tflops = ops.measure_ceilings(eng.device)
+    measured = {"hbm_read_GBs": round(read_gbs, 1), "mfma_bf16_TFLOPs": round(mfma_tflops, 1),
+                "decode_frac_of_read": round(achieved / read_gbs, 4),
+                "prefill_frac_of_mfma": round(pre_flops / pre_s / (mfma_tflops * 1e12), 4)}
     line = {
         "metric": "decode tok/s at batch 8 (+ batch 1/64 in points) and prefill tok/s at 2048 tokens, Qwen3-8B shape bf16",
         "value": round(main_rate, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -145,6 +151,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
         "points": points,
+        "measured": measured,
     }
     print(json.dumps(line))
     return 0

@@ -28,7 +28,7 @@ ARCH = "gfx950"
 FLAGS = ["-O3", f"--offload-arch={ARCH}", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden"]
-CORE_SOURCES = ["elementwise.hip", "sampling.hip", "gemm.hip", "attention_f32.hip"]
+CORE_SOURCES = ["elementwise.hip", "sampling.hip", "gemm.hip", "attention_f32.hip", "probes.hip"]
 RUNTIME_SOURCES = ["runtime.cpp"]
 ATTN_SOURCE = "attention_bf16.hip"
 HEADERS = ["common.h"]

@@ -361,3 +361,34 @@ def sample_rows(logits, temperature, uniform, out):
     _need(out, "sample_rows.out", _I32, (R,))
     _call(load_library("core"), "syn_sample_rows", _ptr(logits), _ptr(temperature),
           _ptr(uniform if temperature is not None else None), _ptr(out), R, V, _stream())
+
+
+# ----------------------------------------------------------------------------- what the machine gives
+
+def measure_ceilings(device="cuda:0", read_bytes=1 << 30, repeats=5):
+    """(memory read rate in GB/s, bf16 MFMA rate in TFLOP/s) of kernels that do nothing else: the
+    best of `repeats` passes over a buffer of read_bytes, and of a launch that keeps every matrix
+    unit busy from registers.  Measurements, to stand beside the vendor's peaks."""
+    lib = load_library("core")
+    buf = torch.empty(read_bytes // 4, dtype=torch.int32, device=device).zero_()
+    sink = torch.zeros(4, dtype=torch.int32, device=device)
+    fsink = torch.zeros(4, dtype=torch.float32, device=device)
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def best(launch):
+        launch()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(repeats):
+            start.record()
+            launch()
+            end.record()
+            end.synchronize()
+            times.append(start.elapsed_time(end) * 1e-3)
+        return min(times)
+
+    t_read = best(lambda: _call(lib, "syn_probe_read", _ptr(buf), ctypes.c_size_t(buf.numel() * 4), _ptr(sink), _stream()))
+    groups, iters = 256 * 8, 4096
+    t_mfma = best(lambda: _call(lib, "syn_probe_mfma", groups, iters, _ptr(fsink), _stream()))
+    flops = groups * 4 * iters * 4 * 2 * 32 * 32 * 16
+    return buf.numel() * 4 / t_read / 1e9, flops / t_mfma / 1e12

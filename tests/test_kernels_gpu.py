@@ -546,3 +546,10 @@ def test_sample_rows_frequencies(ops):
     freq = torch.bincount(out.cpu().long(), minlength=V).float() / R
     p = torch.softmax(logits[0] / 0.8, 0)
     assert (freq - p).abs().max() < 0.012
+
+
+def test_measured_ceilings_are_plausible(ops):
+    """The two probes run and report rates of the right order for this kind of machine."""
+    read_gbs, mfma_tflops = ops.measure_ceilings(DEV, read_bytes=1 << 28, repeats=2)
+    assert 500 < read_gbs < 8000 * 1.05, read_gbs          # below the HBM peak, far above PCIe
+    assert 100 < mfma_tflops < 2500 * 1.05, mfma_tflops    # below the bf16 peak
