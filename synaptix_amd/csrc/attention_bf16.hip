@@ -674,13 +674,23 @@ attn_decode_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ o
     const float w = ms == -INFINITY ? 0.f : __expf(ms - m);  // a split that had no keys weighs nothing
     l += s < n_splits ? w * p[(size_t)s * PART + 1] : 0.f;
     const int cnt = min(SYN_WAVE, n_splits - s0);
-    for (int j = 0; j < cnt; ++j) {
-      const float wj = __shfl(w, j, SYN_WAVE);
-      if (wj == 0.f) continue;
+    for (int j0 = 0; j0 < cnt; j0 += 8) {  // eight splits' values in flight together, added in their order
+      constexpr int NI = (HD + SYN_WAVE - 1) / SYN_WAVE;
+      float vals[8][NI];
 #pragma unroll
-      for (int i = 0; i < (HD + SYN_WAVE - 1) / SYN_WAVE; ++i) {
-        const int d = lane + i * SYN_WAVE;
-        if (d < HD) wsum[i] += wj * p[(size_t)(s0 + j) * PART + 2 + d];
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+          const int d = lane + i * SYN_WAVE;
+          vals[u][i] = (j0 + u < cnt && d < HD) ? p[(size_t)(s0 + j0 + u) * PART + 2 + d] : 0.f;
+        }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const float wj = __shfl(w, min(j0 + u, SYN_WAVE - 1), SYN_WAVE);
+        if (j0 + u < cnt && wj != 0.f) {  // the same for the whole wave; a split without keys may hold anything
+#pragma unroll
+          for (int i = 0; i < NI; ++i) wsum[i] += wj * vals[u][i];
+        }
       }
     }
   }
