@@ -3,7 +3,8 @@
 //   gemm_simt      any shape and type; plain FMA.  The whole 32-bit path, and bf16 shapes that
 //                  the MFMA kernels refuse (K not a multiple of 8, unaligned rows).
 //   gemm_skinny    bf16, M == 1: the weight matrix is streamed once from HBM through
-//                  v_mfma_f32_16x16x32_bf16; the waves of a workgroup split K and sum in LDS.
+//                  v_mfma_f32_16x16x32_bf16; the waves of a workgroup split K and sum in LDS
+//                  (also over paired gate/up rows, with the gated activation as the epilogue).
 //   gemm_tiled     bf16: tiles of x and W in LDS, double-buffered, v_mfma_f32_32x32x16_bf16.
 //                  M > 64: 256x256x64 or 256x192x64 tiles with 8 waves, or 128x128x64 with 4; when K
 //                  is a multiple of 64 by gemm_direct, whose loads write LDS without passing
@@ -66,117 +67,95 @@ gemm_simt_kernel(const TIn* __restrict__ x, const TIn* __restrict__ w, TOut* __r
     }
 }
 
-// ------------------------------------------------------------------ skinny, bf16, one row of x (or a few)
+// ------------------------------------------------------------------ skinny, bf16, one row of x (up to 16)
 // MFMA 16x16x32: A = x rows (m), B = W rows (n), D[m = 4*(lane/16)+j][n = lane%16].
 // Both operands: lane holds row lane%16, k = 8*(lane/16) .. +8, one 16-byte load.
-// A workgroup owns RT*16 rows of W; its WAVES waves take k-chunks of 32 round-robin, so that at
-// any moment the workgroup reads WAVES*64 contiguous bytes of each row.
-template <int MB, int RT, int WAVES, int U>
-__global__ void __launch_bounds__(WAVES * SYN_WAVE)
+// A workgroup owns TILES * 16 rows of W, 16 for each group of KWAVES waves; the waves of a group take
+// k-chunks of 32 round-robin, so that at any moment the group reads KWAVES*64 contiguous bytes of each
+// row, and their partial tiles are summed in LDS in a fixed order.  PAIRED (TILES == 2): the first 16
+// rows are gate rows, the second the up rows of the same outputs, and silu(gate) * up is stored.
+template <int TILES, int KWAVES, int U, bool PAIRED>
+__global__ void __launch_bounds__(TILES * KWAVES * SYN_WAVE)
 gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
-                   int M, int N, int K, int k_slice) {
-  // blockIdx.y = which slice of K this workgroup sums (k_slice elements, a multiple of 32); with
-  // more than one slice the output is float [slices, M, N] and whoever reads it adds the slices
-  extern __shared__ float part[];  // [WAVES][MB*RT*4][64]
+                   int M, int N, int K) {
+  static_assert(!PAIRED || TILES == 2, "a pair is two tiles");
+  constexpr int WAVES = TILES * KWAVES;
+  __shared__ float part[WAVES][4][64];
   const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
+  const int tile = wave / KWAVES, kw = wave % KWAVES;
   const int r16 = lane % 16, kq = (lane / 16) * 8;
-  const int n0 = blockIdx.x * (RT * 16);
+  const int n0 = (blockIdx.x * TILES + tile) * 16;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
   // Rows of W beyond N are read from the last valid row (their results are never stored); rows of x
   // beyond M are not loaded at all: the fewer lanes a load of x has, the less it costs.
-  const bf16* wrow[RT];
-#pragma unroll
-  for (int r = 0; r < RT; ++r) wrow[r] = w + (size_t)min(n0 + r * 16 + r16, N - 1) * K + kq;
-  const bf16* xrow[MB];
-  bool xok[MB];
-#pragma unroll
-  for (int b = 0; b < MB; ++b) {
-    xok[b] = b * 16 + r16 < M;
-    xrow[b] = x + (size_t)min(b * 16 + r16, M - 1) * K + kq;
-  }
-  f32x4 acc[MB][RT];
-#pragma unroll
-  for (int b = 0; b < MB; ++b)
-#pragma unroll
-    for (int r = 0; r < RT; ++r) acc[b][r] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  const bf16* wrow = w + (size_t)min(n0 + r16, N - 1) * K + kq;
+  const bool xok = r16 < M;
+  const bf16* xrow = x + (size_t)min(r16, M - 1) * K + kq;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 
   // U chunks of 32 at a time: all loads of a group are issued before the first product needs them,
-  // so that a wave keeps U * RT KiB of the weight stream in flight
+  // so that a wave keeps U KiB of the weight stream in flight
   constexpr int GROUP = 32 * U;
-  const int k_begin = (int)blockIdx.y * k_slice, k_end = min(K, k_begin + k_slice);
-  const int k_full = k_begin + (k_end - k_begin) / (WAVES * GROUP) * (WAVES * GROUP);
-  for (int k0 = k_begin + wave * GROUP; k0 < k_full; k0 += WAVES * GROUP) {
-    bf16x8 bw[U][RT], ax[U][MB];
+  const int k_full = K / (KWAVES * GROUP) * (KWAVES * GROUP);
+  for (int k0 = kw * GROUP; k0 < k_full; k0 += KWAVES * GROUP) {
+    bf16x8 bw[U], ax[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-#pragma unroll
-      for (int r = 0; r < RT; ++r) bw[u][r] = __builtin_nontemporal_load((const bf16x8*)(wrow[r] + k0 + u * 32));
-#pragma unroll
-      for (int b = 0; b < MB; ++b) ax[u][b] = xok[b] ? *(const bf16x8*)(xrow[b] + k0 + u * 32) : zero;
+      bw[u] = __builtin_nontemporal_load((const bf16x8*)(wrow + k0 + u * 32));
+      ax[u] = xok ? *(const bf16x8*)(xrow + k0 + u * 32) : zero;
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int b = 0; b < MB; ++b)
-#pragma unroll
-        for (int r = 0; r < RT; ++r)
-          acc[b][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[u][b], bw[u][r], acc[b][r], 0, 0, 0);
+    for (int u = 0; u < U; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[u], bw[u], acc, 0, 0, 0);
   }
   // what is left of K, chunk by chunk; K is a multiple of 8, so a lane's 8 elements lie inside or
   // outside as a whole
-  for (int k0 = k_full + wave * 32; k0 < k_end; k0 += WAVES * 32) {
-    const bool kin = k0 + kq < k_end;
-#pragma unroll
-    for (int b = 0; b < MB; ++b) {
-      const bf16x8 ax = (kin && xok[b]) ? *(const bf16x8*)(xrow[b] + k0) : zero;
-#pragma unroll
-      for (int r = 0; r < RT; ++r) {
-        const bf16x8 bw = kin ? *(const bf16x8*)(wrow[r] + k0) : zero;
-        acc[b][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, bw, acc[b][r], 0, 0, 0);
-      }
-    }
+  for (int k0 = k_full + kw * 32; k0 < K; k0 += KWAVES * 32) {
+    const bool kin = k0 + kq < K;
+    const bf16x8 ax = (kin && xok) ? *(const bf16x8*)(xrow + k0) : zero;
+    const bf16x8 bw = kin ? *(const bf16x8*)(wrow + k0) : zero;
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, bw, acc, 0, 0, 0);
   }
 
-  // sum the waves' partial tiles in a fixed order
-  constexpr int SLOTS = MB * RT * 4;
 #pragma unroll
-  for (int b = 0; b < MB; ++b)
-#pragma unroll
-    for (int r = 0; r < RT; ++r)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) part[((size_t)wave * SLOTS + (b * RT + r) * 4 + j) * 64 + lane] = acc[b][r][j];
+  for (int j = 0; j < 4; ++j) part[wave][j][lane] = acc[j];
   __syncthreads();
-  for (int idx = threadIdx.x; idx < SLOTS * 64; idx += WAVES * SYN_WAVE) {
+  auto summed = [&](int t, int j, int ln) {
     float s = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < WAVES; ++wv) s += part[(size_t)wv * SLOTS * 64 + idx];
-    const int slot = idx / 64, ln = idx % 64;
-    const int j = slot % 4, r = (slot / 4) % RT, b = slot / (4 * RT);
-    const int m = b * 16 + 4 * (ln / 16) + j, n = n0 + r * 16 + ln % 16;
-    if (m < M && n < N) {
-      if (out_is_f32)
-        ((float*)out)[((size_t)blockIdx.y * M + m) * N + n] = s;
-      else
-        ((bf16*)out)[(size_t)m * N + n] = (bf16)s;
+    for (int q = 0; q < KWAVES; ++q) s += part[t * KWAVES + q][j][ln];
+    return s;
+  };
+  if constexpr (PAIRED) {
+    for (int idx = threadIdx.x; idx < 4 * 64; idx += WAVES * SYN_WAVE) {
+      const int j = idx / 64, ln = idx % 64;
+      const int m = 4 * (ln / 16) + j, col = (int)blockIdx.x * 16 + ln % 16;  // N / 2 outputs, 16 a workgroup
+      if (m < M && 2 * col < N) {
+        const float g = summed(0, j, ln), up = summed(1, j, ln);
+        ((bf16*)out)[(size_t)m * (N / 2) + col] = (bf16)(g / (1.f + expf(-g)) * up);
+      }
+    }
+  } else {
+    for (int idx = threadIdx.x; idx < TILES * 4 * 64; idx += WAVES * SYN_WAVE) {
+      const int t = idx / 256, j = (idx / 64) % 4, ln = idx % 64;
+      const int m = 4 * (ln / 16) + j, n = (blockIdx.x * TILES + t) * 16 + ln % 16;
+      if (m < M && n < N) {
+        const float v = summed(t, j, ln);
+        if (out_is_f32)
+          ((float*)out)[(size_t)m * N + n] = v;
+        else
+          ((bf16*)out)[(size_t)m * N + n] = (bf16)v;
+      }
     }
   }
 }
 
-template <int MB, int RT, int WAVES, int U>
+template <int TILES, int KWAVES, int U, bool PAIRED = false>
 static void launch_skinny(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
-                          int slices, hipStream_t stream) {
-  const int k_slice = ((K + slices - 1) / slices + 31) / 32 * 32;
-  const dim3 grid((N + RT * 16 - 1) / (RT * 16), slices);
-  const size_t lds = (size_t)WAVES * MB * RT * 4 * 64 * sizeof(float);
-  static bool raised = false;
-  if (lds > 65536 && !raised) {
-    if (hipFuncSetAttribute((const void*)gemm_skinny_kernel<MB, RT, WAVES, U>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return;  // the launch reports the refusal
-    raised = true;
-  }
-  gemm_skinny_kernel<MB, RT, WAVES, U><<<grid, WAVES * SYN_WAVE, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
+                          hipStream_t stream) {
+  const int rows = TILES * 16;
+  gemm_skinny_kernel<TILES, KWAVES, U, PAIRED>
+      <<<(N + rows - 1) / rows, TILES * KWAVES * SYN_WAVE, 0, stream>>>(x, w, out, out_is_f32, M, N, K);
 }
 
 // ------------------------------------------------------------------ shared by the tiled kernels
@@ -529,8 +508,8 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   int rc = 0;
   if (M == 1 && slices == 1) {
     // one row: fragments of W straight from memory, K split over the waves
-    if (N <= 8192) launch_skinny<1, 1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
-    else launch_skinny<1, 1, 8, 4>(xb, wb, out, out_is_f32, M, N, K, slices, stream);
+    if (N <= 8192) launch_skinny<1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
+    else launch_skinny<1, 8, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
   } else if (M <= 32) {
     // few rows: memory-bound; small tiles (many workgroups), deep in K (long pieces of each row)
     if (N >= 65536) rc = launch_tiled<32, 32, 256, 1, 1>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
@@ -555,8 +534,11 @@ SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, i
             "gemm_swiglu: K = %d must be a multiple of 8 and the operands 16-byte aligned", K);
   const bf16* xb = (const bf16*)x;
   const bf16* wb = (const bf16*)w;
-  int rc;
-  if (M <= 32) {
+  int rc = 0;
+  if (M == 1) {
+    // one row: fragments of W straight from memory; eight waves on the gate rows, eight on the up rows
+    launch_skinny<2, 8, 4, true>(xb, wb, out, 0, M, N, K, stream);
+  } else if (M <= 32) {
     if (N >= 65536) rc = launch_tiled<32, 32, 256, 1, 1, true>(xb, wb, out, 0, M, N, K, stream);
     else rc = launch_tiled<32, 64, 128, 1, 2, true>(xb, wb, out, 0, M, N, K, stream);
   } else if (M <= 64) {

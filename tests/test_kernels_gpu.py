@@ -189,7 +189,7 @@ def test_gemm_bf16_partial_sums_over_slices_of_k(ops, M, N, K, S):
     close(got2, want2, 1e-4, 1e-4, "gathered rows of residual + slices")
 
 
-@pytest.mark.parametrize("M,I,K", [(1, 48, 64), (8, 2560, 4096), (7, 112, 1000), (33, 80, 136), (64, 1024, 512),
+@pytest.mark.parametrize("M,I,K", [(1, 48, 64), (1, 2560, 4096), (1, 1008, 1096), (8, 2560, 4096), (7, 112, 1000), (33, 80, 136), (64, 1024, 512),
                                    (300, 400, 264), (2048, 3072, 256), (1000, 6272, 136), (8, 32784, 72),
                                    (1000, 6272, 128), (300, 400, 192)])
 def test_gemm_with_the_gated_activation_inside(ops, M, I, K):
