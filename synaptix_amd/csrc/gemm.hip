@@ -258,7 +258,7 @@ gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* 
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  // blockIdx.y = which slice of K (k_slice elements, a multiple of 32) this workgroup sums, as in gemm_skinny
+  // blockIdx.y = which slice of K (k_slice elements, a multiple of 128) this workgroup sums
   const int k_begin = FEW ? (int)blockIdx.y * k_slice : 0, k_end = FEW ? min(K, k_begin + k_slice) : K;
   const int nk = (k_end - k_begin + BK - 1) / BK;
   bf16x8 rx[XL], rw[WL];
@@ -314,7 +314,7 @@ template <int BM, int BN, int BK, int WM, int WN, bool PAIRED = false>
 static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
                         hipStream_t stream, int slices = 1) {
   SYN_CHECK(slices == 1 || BM <= 64, "gemm: slices of K only with the tiles for few rows");
-  const int k_slice = ((K + slices - 1) / slices + 31) / 32 * 32;
+  const int k_slice = ((K + slices - 1) / slices + 127) / 128 * 128;  // the same cut as launch_direct makes
   const int grid = tile_grid(M, N, BM, BN);
   const size_t lds = (size_t)2 * (BM + BN) * (BK + 8) * sizeof(bf16);
   static bool raised = false;
@@ -327,7 +327,8 @@ static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32,
     SYN_CHECK(e == hipSuccess, "gemm: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
     raised = true;
   }
-  if (K % BK == 0 && k_slice % BK == 0)
+  // whole k-tiles only, and no slice that begins at or beyond the end of K: then no chunk needs a check
+  if (K % BK == 0 && k_slice % BK == 0 && (long)(slices - 1) * k_slice < K)
     gemm_tiled_kernel<BM, BN, BK, WM, WN, false, PAIRED>
         <<<dim3(grid, slices), 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
   else
@@ -337,43 +338,56 @@ static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32,
 }
 
 // ------------------------------------------------------------------ tiled, loads straight into LDS
-// The same tiles for M > 64 and K a multiple of 64, with global_load_lds_dwordx4: a load writes its
-// 16 bytes a lane into LDS without passing through registers, so a k-tile on its way costs no
-// registers and no LDS store instructions, and the wait for it is the last thing before the barrier.
-// An instruction of a wave fills 1 KB of LDS in lane order: 8 rows of 64 k-values, unpadded.  To keep
-// the fragment reads free of bank conflicts all the same, slot s of row r holds the row's 16-byte
-// chunk s ^ ((r >> 1) & 7): the swizzle is applied to the global address of the lane that fills the
-// slot, and again by the reader.  Measured 10 to 20 % faster than staging through registers.
-template <int BM, int BN, int WM, int WN, bool PAIRED>
+// The same tiles with global_load_lds_dwordx4: a load writes its 16 bytes a lane into LDS without
+// passing through registers, so a k-tile on its way costs no registers and no LDS store
+// instructions, and the wait for it is the last thing before the barrier.  K (and every slice of
+// it) must be a multiple of BK.  An instruction of a wave fills 1 KB of LDS in lane order: 8 rows of
+// 64 k-values or 4 rows of 128, unpadded.  To keep the fragment reads free of bank conflicts all the
+// same, slot s of row r holds the row's 16-byte chunk s ^ swizzle(r): the swizzle is applied to the
+// global address of the lane that fills the slot, and again by the reader.  Measured 10 to 20 %
+// faster than staging through registers for prompts, and for single tokens from 16 rows of x on.
+template <int BK>
+__device__ __forceinline__ int direct_swizzle(int row) {
+  // BK = 64: a row is 128 bytes, two rows span the 64 banks; BK = 128: a row spans them all
+  return BK == 64 ? (row >> 1) & 7 : row & (BK / 8 - 1);
+}
+
+template <int BM, int BN, int BK, int WM, int WN, bool PAIRED>
 __global__ void __launch_bounds__(64 * WM * WN)
 gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
-                   int M, int N, int K) {
-  constexpr int BK = 64;
+                   int M, int N, int K, int k_slice) {
+  static_assert(BK == 64 || BK == 128, "k-tiles of 64 or 128");
   constexpr int WAVES = WM * WN;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   constexpr int ROWS = BM + BN;
-  constexpr int PASSES = ROWS / (8 * WAVES);   // instructions of a wave for one k-tile
-  static_assert(ROWS % (8 * WAVES) == 0 && TM >= 1 && TN >= 1, "tile shape");
+  constexpr int CPR = BK / 8;                    // 16-byte chunks in a row of a k-tile
+  constexpr int RPI = 64 / CPR;                  // rows an instruction of a wave fills
+  constexpr int PASSES = ROWS / (RPI * WAVES);   // instructions of a wave for one k-tile
+  static_assert(ROWS % (RPI * WAVES) == 0 && TM >= 1 && TN >= 1, "tile shape");
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];  // [2][ROWS][BK]
   const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE;
   const int wm = (wave / WN) * (BM / WM), wn = (wave % WN) * (BN / WN);
   int tm, tn;
   if (!tile_of_workgroup(M, N, BM, BN, tm, tn)) return;
   const int m0 = tm * BM, n0 = tn * BN;
+  // blockIdx.y = which slice of K (k_slice elements, a multiple of BK) this workgroup sums
+  const int k_begin = (int)blockIdx.y * k_slice, k_end = min(K, k_begin + k_slice);
+  const int nk = max(0, (k_end - k_begin) / BK);
 
-  // pass p: the wave fills tile rows (p * WAVES + wave) * 8 .. + 8 (x rows first, then W rows; rows
+  // pass p: the wave fills tile rows (p * WAVES + wave) * RPI .. + RPI (x rows first, then W rows; rows
   // beyond M or N repeat the last valid one and their results are never stored)
   const bf16* src[PASSES];
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
-    const int row = (p * WAVES + wave) * 8 + lane / 8;
-    const int chunk = (lane % 8) ^ ((row >> 1) & 7);
-    src[p] = (row < BM ? x + (size_t)min(m0 + row, M - 1) * K : w + (size_t)min(n0 + row - BM, N - 1) * K) + chunk * 8;
+    const int row = (p * WAVES + wave) * RPI + lane / CPR;
+    const int chunk = (lane % CPR) ^ direct_swizzle<BK>(row);
+    src[p] = (row < BM ? x + (size_t)min(m0 + row, M - 1) * K : w + (size_t)min(n0 + row - BM, N - 1) * K) +
+             k_begin + chunk * 8;
   }
   auto fetch = [&](int kt, int buf) {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
-      bf16* dst = smem + (size_t)buf * ROWS * BK + (size_t)(p * WAVES + wave) * 8 * BK;  // the same for all lanes
+      bf16* dst = smem + (size_t)buf * ROWS * BK + (size_t)(p * WAVES + wave) * RPI * BK;  // the same for all lanes
       __builtin_amdgcn_global_load_lds((const void*)(src[p] + (size_t)kt * BK),
                                        (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
     }
@@ -389,9 +403,8 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  const int nk = K / BK;
   const int fr = lane % 32, fh = lane / 32;
-  fetch(0, 0);
+  if (nk > 0) fetch(0, 0);  // a slice beyond the end of K stores zeros
   loads_landed();
   __syncthreads();
   for (int kt = 0; kt < nk; ++kt) {
@@ -406,12 +419,12 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
         const int row = wm + i * 32 + fr;
-        a[i] = *(const bf16x8*)(xs + row * BK + (c ^ ((row >> 1) & 7)) * 8);
+        a[i] = *(const bf16x8*)(xs + row * BK + (c ^ direct_swizzle<BK>(row)) * 8);
       }
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         const int row = wn + j * 32 + fr;
-        b[j] = *(const bf16x8*)(ws + row * BK + (c ^ (((row + BM) >> 1) & 7)) * 8);
+        b[j] = *(const bf16x8*)(ws + row * BK + (c ^ direct_swizzle<BK>(row + BM)) * 8);
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -421,22 +434,25 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
     loads_landed();
     __syncthreads();
   }
-  store_tiles<TM, TN, PAIRED>(acc, out, out_is_f32, 0, M, N, m0 + wm, n0 + wn, lane);
+  store_tiles<TM, TN, PAIRED>(acc, out, out_is_f32, blockIdx.y, M, N, m0 + wm, n0 + wn, lane);
 }
 
-template <int BM, int BN, int WM, int WN, bool PAIRED = false>
+// slices > 1 only with a float output [slices, M, N]; K must be a multiple of BK
+template <int BM, int BN, int BK, int WM, int WN, bool PAIRED = false>
 static int launch_direct(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
-                         hipStream_t stream) {
-  const size_t lds = (size_t)2 * (BM + BN) * 64 * sizeof(bf16);
+                         hipStream_t stream, int slices = 1) {
+  SYN_CHECK(K % BK == 0, "gemm: K = %d is no multiple of the k-tile %d", K, BK);
+  const int k_slice = ((K + slices - 1) / slices + 127) / 128 * 128;  // a multiple of BK
+  const size_t lds = (size_t)2 * (BM + BN) * BK * sizeof(bf16);
   static bool raised = false;
   if (lds > 65536 && !raised) {
-    const hipError_t e = hipFuncSetAttribute((const void*)gemm_direct_kernel<BM, BN, WM, WN, PAIRED>,
+    const hipError_t e = hipFuncSetAttribute((const void*)gemm_direct_kernel<BM, BN, BK, WM, WN, PAIRED>,
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     SYN_CHECK(e == hipSuccess, "gemm: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
     raised = true;
   }
-  gemm_direct_kernel<BM, BN, WM, WN, PAIRED>
-      <<<tile_grid(M, N, BM, BN), 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K);
+  gemm_direct_kernel<BM, BN, BK, WM, WN, PAIRED>
+      <<<dim3(tile_grid(M, N, BM, BN), slices), 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
   return 0;
 }
 
@@ -466,9 +482,9 @@ static int launch_large(const bf16* x, const bf16* w, void* out, int out_is_f32,
                         hipStream_t stream) {
   const int shape = pick_large_tile(M, N);
   if (K % 64 == 0) {
-    if (shape == 0) return launch_direct<256, 256, 2, 4, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
-    if (shape == 1) return launch_direct<256, 192, 4, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
-    return launch_direct<128, 128, 1, 4, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
+    if (shape == 0) return launch_direct<256, 256, 64, 2, 4, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
+    if (shape == 1) return launch_direct<256, 192, 64, 4, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
+    return launch_direct<128, 128, 64, 1, 4, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
   }
   if (shape == 0) return launch_tiled<256, 256, 64, 4, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
   if (shape == 1) return launch_tiled<256, 192, 64, 4, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
@@ -511,11 +527,14 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
     if (N <= 8192) launch_skinny<1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
     else launch_skinny<1, 8, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
   } else if (M <= 32) {
-    // few rows: memory-bound; small tiles (many workgroups), deep in K (long pieces of each row)
+    // few rows: memory-bound; small tiles (many workgroups), deep in K (long pieces of each row);
+    // straight into LDS where K allows it (the same speed at 8 rows, a quarter faster at 16 and 32)
     if (N >= 65536) rc = launch_tiled<32, 32, 256, 1, 1>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
+    else if (K % 128 == 0) rc = launch_direct<32, 64, 128, 1, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
     else rc = launch_tiled<32, 64, 128, 1, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
   } else if (M <= 64) {
-    rc = launch_tiled<64, 64, 128, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
+    if (K % 128 == 0) rc = launch_direct<64, 64, 128, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
+    else rc = launch_tiled<64, 64, 128, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
   } else {
     rc = launch_large<false>(xb, wb, out, out_is_f32, M, N, K, stream);
   }
@@ -540,9 +559,11 @@ SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, i
     launch_skinny<2, 8, 4, true>(xb, wb, out, 0, M, N, K, stream);
   } else if (M <= 32) {
     if (N >= 65536) rc = launch_tiled<32, 32, 256, 1, 1, true>(xb, wb, out, 0, M, N, K, stream);
+    else if (K % 128 == 0) rc = launch_direct<32, 64, 128, 1, 2, true>(xb, wb, out, 0, M, N, K, stream);
     else rc = launch_tiled<32, 64, 128, 1, 2, true>(xb, wb, out, 0, M, N, K, stream);
   } else if (M <= 64) {
-    rc = launch_tiled<64, 64, 128, 2, 2, true>(xb, wb, out, 0, M, N, K, stream);
+    if (K % 128 == 0) rc = launch_direct<64, 64, 128, 2, 2, true>(xb, wb, out, 0, M, N, K, stream);
+    else rc = launch_tiled<64, 64, 128, 2, 2, true>(xb, wb, out, 0, M, N, K, stream);
   } else {
     rc = launch_large<true>(xb, wb, out, 0, M, N, K, stream);
   }

@@ -52,7 +52,7 @@ def swiglu(gate_up, out):
 def gemm(x, w, out, force_simt=False):
     if out.dim() == 3:                      # partial sums over slices of K
         S, K = out.shape[0], x.shape[1]
-        step = ((K + S - 1) // S + 31) // 32 * 32
+        step = ((K + S - 1) // S + 127) // 128 * 128
         for s in range(S):
             out[s] = x[:, s * step:(s + 1) * step].to(F32) @ w[:, s * step:(s + 1) * step].to(F32).T
         return

@@ -157,7 +157,7 @@ def test_gemm_bf16(ops, out_dtype, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K,S", [(1, 48, 4096, 4), (8, 4096, 4096, 4), (8, 100, 1000, 3), (16, 64, 12288, 8),
-                                     (40, 70, 2048, 2), (64, 130, 520, 5)])
+                                     (40, 70, 2048, 2), (64, 130, 520, 5), (8, 96, 1536, 5), (50, 200, 3072, 7)])
 def test_gemm_bf16_partial_sums_over_slices_of_k(ops, M, N, K, S):
     """[S, M, N]: slice s holds the sum over its part of K; the slices add up to the product, also
     when K is no multiple of the slice and the last slices are short or empty."""
@@ -166,7 +166,7 @@ def test_gemm_bf16_partial_sums_over_slices_of_k(ops, M, N, K, S):
     ops.gemm(x.to(DEV), w.to(DEV), out)
     want = (x.double() @ w.double().T).float()
     close(out.sum(0), want, 1e-3 * math.sqrt(K), what=f"sum of {S} slices")
-    step = ((K + S - 1) // S + 31) // 32 * 32
+    step = ((K + S - 1) // S + 127) // 128 * 128
     first = (x[:, :step].double() @ w[:, :step].double().T).float()
     close(out[0], first, 1e-3 * math.sqrt(step), what="first slice")
     # the consumer adds the slices: resid + sum(delta) normed
