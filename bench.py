@@ -58,7 +58,7 @@ def main() -> int:
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
     new_tokens = args.warmup + args.steps + 8
     per_seq = (PROMPT + new_tokens + 63) // 64 * 64
-    eng = Engine.from_config(cfg, seed=0, dtype="bfloat16", max_tokens=max(batches) * per_seq, max_seq=8192)
+    eng = Engine.from_config(cfg, seed=0, dtype="bfloat16", max_tokens=max(batches) * per_seq + 64, max_seq=8192)
     g = torch.Generator().manual_seed(0)
 
     def prompt():
@@ -97,6 +97,13 @@ def main() -> int:
                 tokens = []
             tokens += first
         longest = PROMPT + warmup + steps + 8
+        if not args.no_graph:
+            # the captured step is built before anything is timed (with a sequence of its own, one
+            # token long; the other rows are padding), so that also a run without warm-up times steps only
+            spare = eng.acquire()
+            eng.step([(spare, [0])], want=None)
+            eng.decode_runner(batch, longest).step([spare], [0])
+            eng.release(spare)
 
         def one_step(tokens):
             if args.no_graph:
