@@ -44,6 +44,7 @@ class Engine:
         self.device = model.device
         self._require_gpu()
         self.vocab = model.vocab
+        model.check(self.dtype)          # sizes that no kernel takes in this type are refused here
         max_positions = getattr(model.config, "max_position_embeddings", None)
         for b in model.blocks:
             cap = getattr(getattr(b.mixer, "position", None), "capacity", None)

@@ -111,6 +111,11 @@ class DecoderModel:
             p.load(get)
         self.device = self.embedding.table.device
 
+    def check(self, dtype) -> None:
+        """Every part is asked whether its kernels take its sizes in `dtype`."""
+        for p in self._parts():
+            p.check(dtype)
+
     # ------------------------------------------------------------------ cache
     def cache_needs(self) -> list:
         """Need of each cache layer, from the mixer of the run that owns it."""

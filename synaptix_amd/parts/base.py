@@ -23,6 +23,10 @@ class Part:
     def load(self, get) -> None:
         """Fetch the tensors; `get(name)` returns the tensor on the device in its kept type."""
 
+    def check(self, dtype) -> None:
+        """Raise if no kernel takes this part's sizes in the engine's type `dtype`: asked once when an
+        engine is made, so that a size is refused before the first step, not in the middle of it."""
+
 
 @dataclass(frozen=True)
 class KvNeed:

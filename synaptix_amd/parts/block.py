@@ -37,6 +37,10 @@ class PreNormBlock(Block):
         for p in self._parts():
             p.load(get)
 
+    def check(self, dtype):
+        for p in self._parts():
+            p.check(dtype)
+
     def forward(self, resid, pending, ctx, cache, owner=True):
         h = self.norm1.add_apply(resid, pending, ctx.act_dtype)
         a = self.mixer.forward(h, ctx, cache, owner)

@@ -75,6 +75,13 @@ class GqaAttention(Mixer):
     def cache_need(self):
         return KvNeed(self.nkv, self.hd, self.window)
 
+    def check(self, dtype):
+        if self.hd % 2 or self.hd > ops.MAX_HEAD_DIM:
+            raise ValueError(f"{self.prefix}: head size {self.hd} must be even and at most {ops.MAX_HEAD_DIM}")
+        if dtype == torch.bfloat16 and self.hd % 16:
+            raise ValueError(f"{self.prefix}: the bf16 attention kernels take head sizes in steps of 16 "
+                             f"(16, 32, ..., {ops.MAX_HEAD_DIM}); {self.hd} runs in float32 only")
+
     def forward(self, h, ctx, cache, owner=True):
         nh, nkv, hd = self.nh, self.nkv, self.hd
         N, act = h.shape[0], h.dtype

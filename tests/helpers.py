@@ -43,8 +43,10 @@ LONG_L = dict(TINY_A, rope_theta=65536.0, max_position_embeddings=16384)
 ODD_E = dict(num_hidden_layers=2, hidden_size=52, num_attention_heads=2, num_key_value_heads=2, head_dim=80,
              intermediate_size=30, vocab_size=101, rope_theta=2e4, rms_norm_eps=2e-5, max_position_embeddings=300,
              tie_word_embeddings=True, eos_token_id=None, bos_token_id=None)
-SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3, "L": 4, "E": 5}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": MID_D, "L": LONG_L, "E": ODD_E}
+# A head size that only the 32-bit path takes (the bf16 attention kernels take steps of 16).
+ODD_F = dict(TINY_A, head_dim=24, num_attention_heads=3, num_key_value_heads=1)
+SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3, "L": 4, "E": 5, "F": 6}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": MID_D, "L": LONG_L, "E": ODD_E, "F": ODD_F}
 
 _made = {}
 _tmp = None

@@ -13,7 +13,7 @@ import plain_qwen3 as P
 def lengths_for(name):
     # the batches of BASELINE's tiny configurations, plus lengths around a page's edge
     return {"A": [5, 17, 11, 64, 65], "B": [1, 33, 7, 64, 130], "C": [3, 70, 129, 40, 200],
-            "E": [2, 66, 9, 130, 31]}[name]
+            "E": [2, 66, 9, 130, 31], "F": [4, 65, 20]}[name]
 
 
 def requests_for(name, tail=0):

@@ -87,3 +87,16 @@ def test_batch_rows_do_not_depend_on_their_neighbours():
     b = [eng.acquire() for _ in prompts]
     y = eng.step(list(zip(b, prompts))[::-1], want="last")
     assert torch.equal(x, y.flip(0))
+
+
+def test_a_head_size_without_a_kernel_is_refused_when_the_engine_is_made(tmp_path):
+    """Head size 24: the bf16 attention kernels take steps of 16; the 32-bit path takes any even size."""
+    from synaptix_amd import Qwen3Config, write_random_model
+    from helpers import TINY_A
+    cfg = Qwen3Config.from_dict(dict(TINY_A, head_dim=24))
+    write_random_model(str(tmp_path), cfg, 1)
+    with pytest.raises(ValueError, match="steps of 16"):
+        cpu_kernels.CpuEngine.load(str(tmp_path), dtype="bfloat16", max_tokens=128, device="cpu")
+    eng = cpu_kernels.CpuEngine.load(str(tmp_path), dtype="float32", max_tokens=128, device="cpu")
+    s = eng.acquire()
+    assert eng.step([(s, [1, 2, 3])], want="last").shape == (1, cfg.vocab_size)

@@ -70,6 +70,13 @@ def test_awkward_sizes(dtype):
     scenarios.unequal_batches(make_engine, "E", dtype)
 
 
+def test_head_size_24_runs_in_32_bit_and_is_refused_in_bf16():
+    scenarios.whole(make_engine, "F", "float32")
+    scenarios.last_tokens_one_by_one(make_engine, "F", "float32", tail=8)
+    with pytest.raises(ValueError, match="steps of 16"):
+        make_engine("F", "bfloat16", 256)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["A", "C"])
 def test_wide_batch(name, dtype):
