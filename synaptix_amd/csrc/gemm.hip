@@ -6,9 +6,9 @@
 //                  v_mfma_f32_16x16x32_bf16; the waves of a workgroup split K and sum in LDS
 //                  (also over paired gate/up rows, with the gated activation as the epilogue).
 //   gemm_tiled     bf16: tiles of x and W in LDS, double-buffered, v_mfma_f32_32x32x16_bf16.
-//                  M > 64: 256x256x64 or 256x192x64 tiles with 8 waves, or 128x128x64 with 4; when K
-//                  is a multiple of 64 by gemm_direct, whose loads write LDS without passing
-//                  through registers.
+//                  M > 64: 256x256x64, 256x192x64 or 128x128x64 tiles; when K is a multiple of 64 by
+//                  gemm_pipelined, whose loads write LDS without passing through registers and are
+//                  issued, like the fragment reads, one behind each MFMA.
 //                  M <= 64: 32 or 64 rows of x, 64 (or 32) rows of W, 128 (or 256) deep: the rows of
 //                  W arrive as whole 256-byte pieces, which streams them faster than loading MFMA
 //                  fragments (64 bytes a row) straight from memory.  K may be cut into slices
@@ -19,6 +19,8 @@
 // Reference counterparts: crates/synaptix-kernels-cuda/src/best_cu/gemm/gemm_bf16.cu (TN family,
 // mma.sync m16n8k16), best_cu/gemv/mma_gemv.cu:19-133 (M == 1), best_cu/gemm/gemm_f32.cu (SIMT).
 // The tilings here are made for 64-lane waves and MFMA operand layouts, not translated.
+#include <type_traits>
+
 #include "common.h"
 
 // ------------------------------------------------------------------ SIMT, any type
@@ -456,21 +458,197 @@ static int launch_direct(const bf16* x, const bf16* w, void* out, int out_is_f32
   return 0;
 }
 
+// ------------------------------------------------------------------ tiled, M > 64: software-pipelined
+// The k-tile of 64 is four k-steps of 8 (or more) MFMAs a wave.  What the plain loop above leaves to
+// the compiler is laid out by hand here, because each of these was measured to cost matrix-unit time:
+//   * the fragments of k-step s + 1 are read from LDS while the MFMAs of step s run (two sets of
+//     fragment registers), and the reads are placed one behind each MFMA: a wave issues in order, and
+//     an MFMA keeps the matrix unit busy for 32 cycles in which the read behind it costs nothing;
+//   * the barrier of a k-tile stands before the MFMAs of its last k-step; behind it the loads of the
+//     tile after the next and the first fragments of the next tile are issued, again one behind each MFMA;
+//   * the loads go through a buffer descriptor (a base in scalar registers, a 32-bit offset a lane, the
+//     k offset as a scalar): a load is then two instructions (LDS address into M0, the load), where a
+//     64-bit address a lane costs vector adds and takes longer to issue.
+// Counters showed the texture addresser busy about 25 cycles for each 1 KB load of 8 rows x 128 bytes,
+// 1,600 of the 2,048 cycles that the MFMAs of a 256x256x64 tile take: loads that arrive in a burst
+// hold up the waves that issue them, so their spread matters more than their number.
+struct BufferView {
+#if defined(__HIP_DEVICE_COMPILE__)   // the host pass of the compiler has no such type
+  __amdgpu_buffer_rsrc_t r;
+#endif
+};
+__device__ __forceinline__ BufferView buffer_view(const void* base, size_t bytes) {
+  BufferView v;
+#if defined(__HIP_DEVICE_COMPILE__)
+  v.r = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)(bytes > 0xffffffffull ? 0xffffffffull : bytes), 0x00020000);
+#endif
+  return v;
+}
+// 16 bytes a lane from base + lane_bytes + uniform_bytes to lds + 16 * lane (lds is the same for all lanes)
+__device__ __forceinline__ void buffer_to_lds16(const BufferView& v, void* lds, unsigned lane_bytes, int uniform_bytes) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(v.r, (__attribute__((address_space(3))) void*)lds, 16, lane_bytes, uniform_bytes, 0, 0);
+#endif
+}
+
+template <int BM, int BN, int WM, int WN, bool PAIRED>
+__global__ void __launch_bounds__(64 * WM * WN)
+gemm_pipelined_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
+                      int M, int N, int K) {
+  constexpr int BK = 64;
+  constexpr int WAVES = WM * WN;
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+  constexpr int ROWS = BM + BN;
+  constexpr int RPI = 8;                           // rows of 128 bytes that one load of a wave fills
+  constexpr int PASSES = ROWS / (RPI * WAVES);     // loads of a wave for one k-tile
+  constexpr int NM = TM * TN, NR = TM + TN;        // MFMAs and fragment reads of a wave in one k-step
+  static_assert(ROWS % (RPI * WAVES) == 0 && BM % RPI == 0 && NM >= NR, "tile shape");
+  extern __shared__ __attribute__((aligned(16))) bf16 smem[];  // [2][ROWS][64], chunks swizzled as in gemm_direct
+  const int tid = threadIdx.x, lane = tid % SYN_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / SYN_WAVE);   // scalar: LDS addresses of the loads stay scalar
+  const int wm = (wave / WN) * (BM / WM), wn = (wave % WN) * (BN / WN);
+  int tm, tn;
+  if (!tile_of_workgroup(M, N, BM, BN, tm, tn)) return;
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int nk = K / BK;
+
+  // the descriptors begin at the tile's first rows, so a lane's offset stays below 2^32 for any M and N
+  const size_t row_bytes = (size_t)K * sizeof(bf16);
+  const BufferView vx = buffer_view(x + (size_t)m0 * K, (size_t)(M - m0) * row_bytes);
+  const BufferView vw = buffer_view(w + (size_t)n0 * K, (size_t)(N - n0) * row_bytes);
+  // pass p: the wave fills tile rows (p * WAVES + wave) * 8 .. + 8 (x rows first, then W rows; rows beyond M or
+  // N repeat the last valid one and their results are never stored)
+  unsigned src[PASSES];
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    const int row0 = (p * WAVES + wave) * RPI, row = row0 + lane / 8;
+    const int chunk = (lane % 8) ^ direct_swizzle<BK>(row);
+    const int in_tile = row0 < BM ? min(row, M - 1 - m0) : min(row - BM, N - 1 - n0);
+    src[p] = (unsigned)((size_t)in_tile * row_bytes + chunk * 16);
+  }
+  auto fetch_pass = [&](int kt, int buf, int p) {
+    bf16* dst = smem + (size_t)buf * ROWS * BK + (size_t)(p * WAVES + wave) * RPI * BK;
+    buffer_to_lds16((p * WAVES + wave) * RPI < BM ? vx : vw, dst, src[p], kt * (BK * (int)sizeof(bf16)));
+  };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const int fr = lane % 32, fh = lane / 32;
+  int arow[TM], brow[TN], asw[TM], bsw[TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) arow[i] = (wm + i * 32 + fr) * BK, asw[i] = direct_swizzle<BK>(wm + i * 32 + fr);
+#pragma unroll
+  for (int j = 0; j < TN; ++j) brow[j] = (BM + wn + j * 32 + fr) * BK, bsw[j] = direct_swizzle<BK>(BM + wn + j * 32 + fr);
+  bf16x8 a[2][TM], b[2][TN];   // two sets of fragments: one is multiplied while the other is read
+  auto read_one = [&](int buf, int ks, int set, int idx) {
+    const bf16* base = smem + (size_t)buf * ROWS * BK;
+    const int c = 2 * ks + fh;  // the 16-byte chunk of a row that this lane multiplies
+    if (idx < TM) a[set][idx] = *(const bf16x8*)(base + arow[idx] + (c ^ asw[idx]) * 8);
+    else b[set][idx - TM] = *(const bf16x8*)(base + brow[idx - TM] + (c ^ bsw[idx - TM]) * 8);
+  };
+  auto mfmas = [&](int set) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[set][i], b[set][j], acc[i][j], 0, 0, 0);
+  };
+  // one k-tile.  MORE_LOADS: the tile after the next exists; MORE_TILES: a next tile exists.
+  auto tile = [&](int kt, auto more_loads, auto more_tiles) {
+    constexpr int NF = decltype(more_loads)::value ? PASSES : 0, NN = decltype(more_tiles)::value ? NR : 0;
+    const int buf = kt & 1;
+#pragma unroll
+    for (int ks = 0; ks < 3; ++ks) {
+      __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): the fragments read one k-step ago are there
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < NR; ++i) read_one(buf, ks + 1, (ks + 1) & 1, i);
+      mfmas(ks & 1);
+#pragma unroll
+      for (int i = 0; i < NR; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA,
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read behind it
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, NM - NR, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // this wave's loads of the next tile have landed and its reads of this tile are done; behind the
+    // barrier that holds for every wave.  No fence: this is all the barrier has to order.
+    __builtin_amdgcn_s_waitcnt(0x0070);     // vmcnt(0) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    // in program order a load into LDS and a fragment read alternate, so that they can be spread
+#pragma unroll
+    for (int i = 0; i < (NF > NN ? NF : NN); ++i) {
+      if (i < NF) fetch_pass(kt + 2, buf, i);
+      if (i < NN) read_one(buf ^ 1, 0, 0, i);
+    }
+    mfmas(1);
+#pragma unroll
+    for (int i = 0; i < NM; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (i < NF) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);   // one load,
+      if (i < NN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) fetch_pass(0, 0, p);
+  if (nk > 1) {
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) fetch_pass(1, 1, p);
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (PASSES & 15) | ((PASSES >> 4) << 14));   // vmcnt(PASSES): tile 0 is there
+  } else {
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+  }
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int i = 0; i < NR; ++i) read_one(0, 0, 0, i);
+  int kt = 0;
+  for (; kt + 2 < nk; ++kt) tile(kt, std::true_type{}, std::true_type{});
+  if (kt + 1 < nk) tile(kt++, std::false_type{}, std::true_type{});
+  tile(kt, std::false_type{}, std::false_type{});
+  store_tiles<TM, TN, PAIRED>(acc, out, out_is_f32, 0, M, N, m0 + wm, n0 + wn, lane);
+}
+
+template <int BM, int BN, int WM, int WN, bool PAIRED = false>
+static int launch_pipelined(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
+                            hipStream_t stream) {
+  SYN_CHECK(K % 64 == 0, "gemm: K = %d is no multiple of the k-tile 64", K);
+  const size_t lds = (size_t)2 * (BM + BN) * 64 * sizeof(bf16);
+  static bool raised = false;
+  if (lds > 65536 && !raised) {
+    const hipError_t e = hipFuncSetAttribute((const void*)gemm_pipelined_kernel<BM, BN, WM, WN, PAIRED>,
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    SYN_CHECK(e == hipSuccess, "gemm: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
+    raised = true;
+  }
+  gemm_pipelined_kernel<BM, BN, WM, WN, PAIRED>
+      <<<tile_grid(M, N, BM, BN), 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K);
+  return 0;
+}
+
 // M > 64: the tile shape by pick_large_tile; loads straight into LDS where K allows it
 template <bool PAIRED>
 static int launch_large(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
                         hipStream_t stream);
 
-// Which of the large tiles for M > 64: 0 = 256 x 256, 1 = 256 x 192 (both 8 waves, one workgroup a
-// compute unit), 2 = 128 x 128 (4 waves, two workgroups a compute unit, about 15 % less efficient).
+// Which of the large tiles for M > 64: 0 = 256 x 256, 1 = 256 x 192 (one workgroup a compute unit; about
+// 6 % less efficient), 2 = 128 x 128 (two workgroups a compute unit, about 20 % less efficient).
 // The estimate is the number of rounds over the 256 compute units times the work of a tile; it
 // reproduces what was measured at 2048 rows for N = 4096, 6144 and 24576 (a tie goes to the larger tile).
 static int pick_large_tile(int M, int N) {
   auto rounds = [](long tiles, long slots) { return (tiles + slots - 1) / slots; };
   auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   const double cost[3] = {(double)rounds(tiles(256, 256), 256) * 256 * 256,
-                          (double)rounds(tiles(256, 192), 256) * 256 * 192,
-                          (double)rounds(tiles(128, 128), 512) * 2 * 128 * 128 * 1.15};
+                          (double)rounds(tiles(256, 192), 256) * 256 * 192 * 1.06,
+                          (double)rounds(tiles(128, 128), 512) * 2 * 128 * 128 * 1.2};
   int best = 0;
   if (cost[1] < cost[best]) best = 1;
   if (cost[2] < cost[best]) best = 2;
@@ -482,9 +660,9 @@ static int launch_large(const bf16* x, const bf16* w, void* out, int out_is_f32,
                         hipStream_t stream) {
   const int shape = pick_large_tile(M, N);
   if (K % 64 == 0) {
-    if (shape == 0) return launch_direct<256, 256, 64, 2, 4, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
-    if (shape == 1) return launch_direct<256, 192, 64, 4, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
-    return launch_direct<128, 128, 64, 1, 4, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
+    if (shape == 0) return launch_pipelined<256, 256, 2, 4, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
+    if (shape == 1) return launch_pipelined<256, 192, 2, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
+    return launch_pipelined<128, 128, 2, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
   }
   if (shape == 0) return launch_tiled<256, 256, 64, 4, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
   if (shape == 1) return launch_tiled<256, 192, 64, 4, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
