@@ -339,8 +339,31 @@ static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32,
   return 0;
 }
 
+// ------------------------------------------------------------------ loads through a buffer descriptor
+// A base and a size in scalar registers, a 32-bit offset a lane, a further offset as a scalar: a load
+// into LDS is then two instructions (LDS address into M0, the load), where a 64-bit address a lane
+// costs vector adds and takes longer to issue.
+struct BufferView {
+#if defined(__HIP_DEVICE_COMPILE__)   // the host pass of the compiler has no such type
+  __amdgpu_buffer_rsrc_t r;
+#endif
+};
+__device__ __forceinline__ BufferView buffer_view(const void* base, size_t bytes) {
+  BufferView v;
+#if defined(__HIP_DEVICE_COMPILE__)
+  v.r = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)(bytes > 0xffffffffull ? 0xffffffffull : bytes), 0x00020000);
+#endif
+  return v;
+}
+// 16 bytes a lane from base + lane_bytes + uniform_bytes to lds + 16 * lane (lds is the same for all lanes)
+__device__ __forceinline__ void buffer_to_lds16(const BufferView& v, void* lds, unsigned lane_bytes, int uniform_bytes) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(v.r, (__attribute__((address_space(3))) void*)lds, 16, lane_bytes, uniform_bytes, 0, 0);
+#endif
+}
+
 // ------------------------------------------------------------------ tiled, loads straight into LDS
-// The same tiles with global_load_lds_dwordx4: a load writes its 16 bytes a lane into LDS without
+// The same tiles with buffer_load_dwordx4 ... lds: a load writes its 16 bytes a lane into LDS without
 // passing through registers, so a k-tile on its way costs no registers and no LDS store
 // instructions, and the wait for it is the last thing before the barrier.  K (and every slice of
 // it) must be a multiple of BK.  An instruction of a wave fills 1 KB of LDS in lane order: 8 rows of
@@ -367,7 +390,8 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
   constexpr int PASSES = ROWS / (RPI * WAVES);   // instructions of a wave for one k-tile
   static_assert(ROWS % (RPI * WAVES) == 0 && TM >= 1 && TN >= 1, "tile shape");
   extern __shared__ __attribute__((aligned(16))) bf16 smem[];  // [2][ROWS][BK]
-  const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE;
+  const int tid = threadIdx.x, lane = tid % SYN_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / SYN_WAVE);   // scalar: LDS addresses of the loads stay scalar
   const int wm = (wave / WN) * (BM / WM), wn = (wave % WN) * (BN / WN);
   int tm, tn;
   if (!tile_of_workgroup(M, N, BM, BN, tm, tn)) return;
@@ -376,22 +400,26 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
   const int k_begin = (int)blockIdx.y * k_slice, k_end = min(K, k_begin + k_slice);
   const int nk = max(0, (k_end - k_begin) / BK);
 
+  // the descriptors begin at the tile's first rows, so a lane's offset stays below 2^32 for any M and N.
   // pass p: the wave fills tile rows (p * WAVES + wave) * RPI .. + RPI (x rows first, then W rows; rows
   // beyond M or N repeat the last valid one and their results are never stored)
-  const bf16* src[PASSES];
+  static_assert(BM % RPI == 0, "a load lies in x or in W as a whole");
+  const size_t row_bytes = (size_t)K * sizeof(bf16);
+  const BufferView vx = buffer_view(x + (size_t)m0 * K, (size_t)(M - m0) * row_bytes);
+  const BufferView vw = buffer_view(w + (size_t)n0 * K, (size_t)(N - n0) * row_bytes);
+  unsigned src[PASSES];
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
-    const int row = (p * WAVES + wave) * RPI + lane / CPR;
+    const int row0 = (p * WAVES + wave) * RPI, row = row0 + lane / CPR;
     const int chunk = (lane % CPR) ^ direct_swizzle<BK>(row);
-    src[p] = (row < BM ? x + (size_t)min(m0 + row, M - 1) * K : w + (size_t)min(n0 + row - BM, N - 1) * K) +
-             k_begin + chunk * 8;
+    const int in_tile = row0 < BM ? min(row, M - 1 - m0) : min(row - BM, N - 1 - n0);
+    src[p] = (unsigned)((size_t)in_tile * row_bytes + chunk * 16);
   }
   auto fetch = [&](int kt, int buf) {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
       bf16* dst = smem + (size_t)buf * ROWS * BK + (size_t)(p * WAVES + wave) * RPI * BK;  // the same for all lanes
-      __builtin_amdgcn_global_load_lds((const void*)(src[p] + (size_t)kt * BK),
-                                       (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+      buffer_to_lds16((p * WAVES + wave) * RPI < BM ? vx : vw, dst, src[p], (k_begin + kt * BK) * (int)sizeof(bf16));
     }
   };
   // all loads of this wave have written LDS: vmcnt(0), the other counters left alone
@@ -472,25 +500,6 @@ static int launch_direct(const bf16* x, const bf16* w, void* out, int out_is_f32
 // Counters showed the texture addresser busy about 25 cycles for each 1 KB load of 8 rows x 128 bytes,
 // 1,600 of the 2,048 cycles that the MFMAs of a 256x256x64 tile take: loads that arrive in a burst
 // hold up the waves that issue them, so their spread matters more than their number.
-struct BufferView {
-#if defined(__HIP_DEVICE_COMPILE__)   // the host pass of the compiler has no such type
-  __amdgpu_buffer_rsrc_t r;
-#endif
-};
-__device__ __forceinline__ BufferView buffer_view(const void* base, size_t bytes) {
-  BufferView v;
-#if defined(__HIP_DEVICE_COMPILE__)
-  v.r = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)(bytes > 0xffffffffull ? 0xffffffffull : bytes), 0x00020000);
-#endif
-  return v;
-}
-// 16 bytes a lane from base + lane_bytes + uniform_bytes to lds + 16 * lane (lds is the same for all lanes)
-__device__ __forceinline__ void buffer_to_lds16(const BufferView& v, void* lds, unsigned lane_bytes, int uniform_bytes) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(v.r, (__attribute__((address_space(3))) void*)lds, 16, lane_bytes, uniform_bytes, 0, 0);
-#endif
-}
-
 template <int BM, int BN, int WM, int WN, bool PAIRED>
 __global__ void __launch_bounds__(64 * WM * WN)
 gemm_pipelined_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
