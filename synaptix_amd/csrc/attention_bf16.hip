@@ -347,18 +347,20 @@ SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, co
 constexpr int PART = HD + 2;
 constexpr int DEC_MAX_WAVES = HD > 128 ? 4 : 8;  // as many as keep their ~190 registers each without spilling
 
-// Like attn_block for one column block, but every K and V fragment of the block is requested before
-// the first product needs one: a block costs one trip to memory instead of two.
+// The K and V fragments of one block of 64 keys, all requested before the first product needs one.
 struct KvBlock {
   kfrag_t ka[4][KSTEPS];
   bf16x8 va[2][DT];
 };
 
-__device__ __forceinline__ void load_block_decode(KvBlock& b, const bf16* __restrict__ kpage,
-                                                  const bf16* __restrict__ vpage, int lane) {
-  const int r16 = lane % 16, g4 = lane / 16;
+__device__ __forceinline__ void load_k_decode(KvBlock& b, const bf16* __restrict__ kpage, int lane) {
+  const int r16 = lane % 16;
 #pragma unroll
   for (int t = 0; t < 4; ++t) load_row(b.ka[t], kpage + (size_t)tile_row_key(t, r16) * HD, lane);
+}
+
+__device__ __forceinline__ void load_v_decode(KvBlock& b, const bf16* __restrict__ vpage, int lane) {
+  const int r16 = lane % 16, g4 = lane / 16;
 #pragma unroll
   for (int h = 0; h < 2; ++h)
 #pragma unroll
@@ -366,19 +368,86 @@ __device__ __forceinline__ void load_block_decode(KvBlock& b, const bf16* __rest
       b.va[h][dt] = *(const bf16x8*)(vpage + (size_t)(dt * 16 + r16) * SYN_PAGE + h * 32 + 8 * g4);
 }
 
-__device__ __forceinline__ void attn_block_decode(AttnState<1>& st, const QFrag& qf, const KvBlock& blk, int key0,
-                                                  int qpos, int lo, int kv_len, float scale, int lane) {
+// Head sizes that are a power of two from 32 on: a block's K rows (64 x HD) and its V^T rows (HD x 64) are
+// each one contiguous piece of 128 * HD bytes, and a wave brings them into a piece of LDS of its own
+// with loads of 1 KB that write LDS directly, then reads its fragments from there.  Loading the
+// fragments straight from memory asks the first-level cache for 16 rows x 64 bytes with every
+// instruction, which was measured to keep the texture addresser busy about 100 cycles an instruction
+// and to be what bounds the kernel at large batches.
+// In LDS the 16-byte chunk c of row r lies at slot c ^ f(r) of the row, with f chosen so that the 16
+// rows a fragment read touches fall into different banks; the permutation is applied to the address
+// that a lane fetches (the slot it fills is fixed by its number) and again by the reader.
+constexpr bool STAGED = !TAIL16 && (HD & (HD - 1)) == 0;
+constexpr int STAGE_BYTES = STAGED ? 128 * HD : 0;   // one block of K, or of V^T
+constexpr int K_CPR = HD / 8;                        // 16-byte chunks in a K row
+// the rows of a score tile differ in bits 0, 1, 3 and 4 of the key number: those four bits, less as
+// many low ones as rows fit into the 256 bytes that the banks span
+__device__ __forceinline__ int k_swizzle(int row) {
+  constexpr int DROP = HD >= 128 ? 0 : (HD == 64 ? 1 : 2);
+  return ((row & 3) | (((row >> 3) & 3) << 2)) >> DROP;
+}
+__device__ __forceinline__ int v_swizzle(int row) { return (row >> 1) & 7; }  // two rows of 128 bytes span the banks
+
+__device__ __forceinline__ void stage_k(const bf16* __restrict__ kpage, char* stage, int lane) {
+  const BufferView view = buffer_view(kpage, STAGE_BYTES);
+#pragma unroll
+  for (int i = 0; i < HD / 8; ++i) {
+    const int at = 64 * i + lane, row = at / K_CPR, slot = at % K_CPR;
+    buffer_to_lds16(view, stage + 1024 * i, (unsigned)((row * K_CPR + (slot ^ k_swizzle(row))) * 16), 0);
+  }
+}
+__device__ __forceinline__ void stage_v(const bf16* __restrict__ vpage, char* stage, int lane) {
+  const BufferView view = buffer_view(vpage, STAGE_BYTES);
+#pragma unroll
+  for (int i = 0; i < HD / 8; ++i) {
+    const int at = 64 * i + lane, row = at / 8, slot = at % 8;
+    buffer_to_lds16(view, stage + 1024 * i, (unsigned)((row * 8 + (slot ^ v_swizzle(row))) * 16), 0);
+  }
+}
+// the staged piece has landed (this wave's loads are done); nothing that reads it may move above this
+__device__ __forceinline__ void staged_landed() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// this wave's reads of the staged piece have returned: the piece may be filled again
+__device__ __forceinline__ void staged_read() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+__device__ __forceinline__ void read_k_staged(KvBlock& b, const char* stage, int lane) {
+  if constexpr (STAGED) {
+    const int r16 = lane % 16, g4 = lane / 16;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int row = tile_row_key(t, r16), sw = k_swizzle(row);
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) b.ka[t][ks] = *(const kfrag_t*)(stage + (row * K_CPR + ((ks * 4 + g4) ^ sw)) * 16);
+    }
+  }
+}
+__device__ __forceinline__ void read_v_staged(KvBlock& b, const char* stage, int lane) {
+  const int r16 = lane % 16, g4 = lane / 16;
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const int row = dt * 16 + r16;
+      b.va[h][dt] = *(const bf16x8*)(stage + (row * 8 + ((h * 4 + g4) ^ v_swizzle(row))) * 16);
+    }
+}
+
+// One block of 64 keys in two halves, so that the loads of the next block can follow each half at once:
+// the scores and their softmax weights (reads the K fragments), then the weighted values (reads the V fragments).
+__device__ __forceinline__ void decode_scores(AttnState<1>& st, const QFrag& qf, const KvBlock& blk, f32x4 (&s)[4],
+                                              int key0, int qpos, int lo, float scale, int lane) {
   const int g4 = lane / 16;
   const auto& ka = blk.ka;
-  const auto& va = blk.va;
-
-  f32x4 s[4];
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
     s[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) s[t] = mfma_qk(ka[t][ks], qf.k[ks], s[t]);
   }
+}
+
+__device__ __forceinline__ void decode_weights(AttnState<1>& st, f32x4 (&s)[4], int key0, int qpos, int lo, float scale,
+                                               int lane) {
+  const int g4 = lane / 16;
   float mloc = -INFINITY;
 #pragma unroll
   for (int t = 0; t < 4; ++t)
@@ -408,6 +477,12 @@ __device__ __forceinline__ void attn_block_decode(AttnState<1>& st, const QFrag&
   st.l[0] = st.l[0] * alpha + lsum;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) st.o[dt][0] *= alpha;
+}
+
+__device__ __forceinline__ void decode_values(AttnState<1>& st, const KvBlock& blk, const f32x4 (&s)[4], int key0,
+                                              int kv_len, int lane) {
+  const int g4 = lane / 16;
+  const auto& va = blk.va;
   const bool ragged = key0 + SYN_PAGE > kv_len;
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
@@ -458,15 +533,17 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
                          const int* __restrict__ page_table, int table_stride, const int* __restrict__ seq_len,
                          float* __restrict__ partial, bf16* __restrict__ out, float scale, int window, int nh, int nkv,
                          int n_splits, int cols_alloc, QkvIntake in) {
-  // LDS: sm[waves][16] running maxima, sl[waves][16] sums, so[waves][cols_alloc][HD + 4] outputs;
+  // LDS: with STAGED first a piece of STAGE_BYTES for each wave; then
+  //      sm[waves][16] running maxima, sl[waves][16] sums, so[waves][cols_alloc][HD + 4] outputs;
   // FUSED: then xs[waves][HD] floats, snew[16] scores of the new key, qs[cols_alloc][HD], knew[HD], vnew[HD] bf16
-  extern __shared__ float dec_lds[];
+  extern __shared__ __attribute__((aligned(16))) float dec_lds[];
   const int n_waves = blockDim.x / SYN_WAVE;
-  float* sm = dec_lds;
+  float* sm = dec_lds + (size_t)n_waves * (STAGE_BYTES / 4);   // the waves' staging pieces lie first
   float* sl = sm + n_waves * 16;
   float* so = sl + n_waves * 16;
   constexpr int SO_LD = HD + 4;
-  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / SYN_WAVE), lane = threadIdx.x % SYN_WAVE;
+  char* stage = (char*)dec_lds + (size_t)wave * STAGE_BYTES;
   const int seq = blockIdx.x, split = blockIdx.z;
   const int g = nh / nkv, chunks = (g + 15) / 16;
   const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
@@ -486,13 +563,18 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
   const int b_lo = lo / SYN_PAGE, b_hi = n_old > 0 ? (n_old - 1) / SYN_PAGE : b_lo - 1;
   const int per = (b_hi - b_lo + n_splits) / n_splits;  // ceil((b_hi - b_lo + 1) / n_splits)
   const int b0 = b_lo + split * per, b1 = min(b_hi + 1, b0 + per);
-  auto page_of = [&](int kb) {
-    return ((size_t)page_table[(size_t)seq * table_stride + kb] * nkv + kvh) * SYN_PAGE * HD;
+  auto page_of = [&](int kb) {   // the same for all lanes
+    return ((size_t)__builtin_amdgcn_readfirstlane(page_table[(size_t)seq * table_stride + kb]) * nkv + kvh) * SYN_PAGE * HD;
   };
   KvBlock blk;
   if (b0 + wave < b1) {
     const size_t base = page_of(b0 + wave);
-    load_block_decode(blk, k_pages + base, v_pages + base, lane);
+    if constexpr (STAGED) {
+      stage_k(k_pages + base, stage, lane);
+    } else {
+      load_k_decode(blk, k_pages + base, lane);
+      load_v_decode(blk, v_pages + base, lane);
+    }
   }
 
   float* xs = so + (size_t)n_waves * cols_alloc * SO_LD;
@@ -603,13 +685,35 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
     load_q(qf, valid ? q + ((size_t)seq * nh + kvh * g + hg) * HD : nullptr, lane);
   AttnState<1> st;
   attn_init(st);
+  // K and V of a block come one after the other: while the scores and the softmax of block i are computed
+  // its V is on its way, while its values are added the K of block i + 1 is, so a wave always has half a
+  // block in flight (through its staging piece, or without one into the registers that were just used)
   for (int kb = b0 + wave; kb < b1; kb += n_waves) {
-    if (kb != b0 + wave) {  // the first block is already on its way
+    const int next = kb + n_waves;
+    f32x4 s[4];
+    if constexpr (STAGED) {
       const size_t base = page_of(kb);
-      load_block_decode(blk, k_pages + base, v_pages + base, lane);
+      staged_landed();
+      read_k_staged(blk, stage, lane);
+      staged_read();
+      stage_v(v_pages + base, stage, lane);
+      decode_scores(st, qf, blk, s, kb * SYN_PAGE, valid ? q_lim : -1, lo, scale, lane);
+      decode_weights(st, s, kb * SYN_PAGE, valid ? q_lim : -1, lo, scale, lane);
+      staged_landed();
+      read_v_staged(blk, stage, lane);
+      staged_read();
+      if (next < b1) stage_k(k_pages + page_of(next), stage, lane);
+      decode_values(st, blk, s, kb * SYN_PAGE, n_old, lane);
+    } else {
+      const size_t next_base = next < b1 ? page_of(next) : 0;
+      decode_scores(st, qf, blk, s, kb * SYN_PAGE, valid ? q_lim : -1, lo, scale, lane);
+      if (next < b1) load_k_decode(blk, k_pages + next_base, lane);
+      decode_weights(st, s, kb * SYN_PAGE, valid ? q_lim : -1, lo, scale, lane);
+      decode_values(st, blk, s, kb * SYN_PAGE, n_old, lane);
+      if (next < b1) load_v_decode(blk, v_pages + next_base, lane);
     }
-    attn_block_decode(st, qf, blk, kb * SYN_PAGE, valid ? q_lim : -1, lo, n_old, scale, lane);
   }
+  if constexpr (STAGED) staged_landed();   // nothing still on its way into LDS when the wave goes on
   float l = st.l[0];
   l += __shfl_xor(l, 16, SYN_WAVE);
   l += __shfl_xor(l, 32, SYN_WAVE);
@@ -715,15 +819,24 @@ static int launch_decode(const void* q, const QkvIntake* in, void* k_pages, void
   // about 2,048 waves in all: at large batches four waves a workgroup are plenty
   const int cols_alloc = nh / nkv < 16 ? nh / nkv : 16;
   auto lds_for = [&](int waves) {
-    size_t b = (size_t)waves * (32 + (size_t)cols_alloc * (HD + 4)) * sizeof(float);
+    size_t b = (size_t)waves * STAGE_BYTES + (size_t)waves * (32 + (size_t)cols_alloc * (HD + 4)) * sizeof(float);
     if (in) b += ((size_t)waves * HD + 16) * sizeof(float) + (size_t)(cols_alloc + 2) * HD * sizeof(bf16);
     return b;
   };
+  constexpr size_t LDS_MAX = 160 * 1024;
   int waves = DEC_MAX_WAVES;
-  while (waves > 2 && (lds_for(waves) > 64 * 1024 || (long)n_seqs * nkv * chunks * n_splits * waves > 2048)) waves /= 2;
-  if (waves < 4 && lds_for(4) <= 64 * 1024) waves = 4;
+  while (waves > 2 && (lds_for(waves) > LDS_MAX || (long)n_seqs * nkv * chunks * n_splits * waves > 2048)) waves /= 2;
+  if (waves < 4 && lds_for(4) <= LDS_MAX) waves = 4;
   const size_t lds = lds_for(waves);
-  SYN_CHECK(lds <= 64 * 1024, "attention_decode: %zu bytes of LDS for %d heads a group", lds, nh / nkv);
+  SYN_CHECK(lds <= LDS_MAX, "attention_decode: %zu bytes of LDS for %d heads a group", lds, nh / nkv);
+  static bool raised = false;
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)attn_decode_split_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)attn_decode_split_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
+    SYN_CHECK(e == hipSuccess, "attention_decode: %zu bytes of LDS refused: %s", LDS_MAX, hipGetErrorString(e));
+    raised = true;
+  }
   const dim3 grid(n_seqs, nkv * chunks, n_splits);
   if (in)
     attn_decode_split_kernel<true><<<grid, waves * SYN_WAVE, lds, stream>>>(

@@ -84,3 +84,26 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   for (int i = 0; i < nw; ++i) t += red[i];
   return t;
 }
+
+// ---- loads through a buffer descriptor, straight into LDS ----
+// A base and a size in scalar registers, a 32-bit offset a lane, a further offset as a scalar: a load
+// into LDS is then two instructions (LDS address into M0, the load), where a 64-bit address a lane
+// costs vector adds and takes longer to issue.
+struct BufferView {
+#if defined(__HIP_DEVICE_COMPILE__)   // the host pass of the compiler has no such type
+  __amdgpu_buffer_rsrc_t r;
+#endif
+};
+__device__ __forceinline__ BufferView buffer_view(const void* base, size_t bytes) {
+  BufferView v;
+#if defined(__HIP_DEVICE_COMPILE__)
+  v.r = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)(bytes > 0xffffffffull ? 0xffffffffull : bytes), 0x00020000);
+#endif
+  return v;
+}
+// 16 bytes a lane from base + lane_bytes + uniform_bytes to lds + 16 * lane (lds is the same for all lanes)
+__device__ __forceinline__ void buffer_to_lds16(const BufferView& v, void* lds, unsigned lane_bytes, int uniform_bytes) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(v.r, (__attribute__((address_space(3))) void*)lds, 16, lane_bytes, uniform_bytes, 0, 0);
+#endif
+}
