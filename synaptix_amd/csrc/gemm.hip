@@ -354,11 +354,11 @@ __device__ __forceinline__ int direct_swizzle(int row) {
   return BK == 64 ? (row >> 1) & 7 : row & (BK / 8 - 1);
 }
 
-template <int BM, int BN, int BK, int WM, int WN, bool PAIRED>
+template <int BM, int BN, int BK, int WM, int WN, bool PAIRED, int STAGES>
 __global__ void __launch_bounds__(64 * WM * WN)
 gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
                    int M, int N, int K, int k_slice) {
-  static_assert(BK == 64 || BK == 128, "k-tiles of 64 or 128");
+  static_assert((BK == 64 || BK == 128 || BK == 256) && STAGES >= 2, "k-tiles of 64, 128 or 256 in two or more buffers");
   constexpr int WAVES = WM * WN;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   constexpr int ROWS = BM + BN;
@@ -366,7 +366,7 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
   constexpr int RPI = 64 / CPR;                  // rows an instruction of a wave fills
   constexpr int PASSES = ROWS / (RPI * WAVES);   // instructions of a wave for one k-tile
   static_assert(ROWS % (RPI * WAVES) == 0 && TM >= 1 && TN >= 1, "tile shape");
-  extern __shared__ __attribute__((aligned(16))) bf16 smem[];  // [2][ROWS][BK]
+  extern __shared__ __attribute__((aligned(16))) bf16 smem[];  // [STAGES][ROWS][BK]
   const int tid = threadIdx.x, lane = tid % SYN_WAVE;
   const int wave = __builtin_amdgcn_readfirstlane(tid / SYN_WAVE);   // scalar: LDS addresses of the loads stay scalar
   const int wm = (wave / WN) * (BM / WM), wn = (wave % WN) * (BN / WN);
@@ -399,8 +399,15 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
       buffer_to_lds16((p * WAVES + wave) * RPI < BM ? vx : vw, dst, src[p], (k_begin + kt * BK) * (int)sizeof(bf16));
     }
   };
-  // all loads of this wave have written LDS: vmcnt(0), the other counters left alone
-  auto loads_landed = [] { __builtin_amdgcn_s_waitcnt(0x0f70); };
+  // Tile kt lies in buffer kt % STAGES; while it is multiplied the STAGES - 1 tiles after it are on their
+  // way.  Before the barrier that ends a tile a wave waits until its own loads of the next tile have
+  // written LDS (all but the (STAGES - 2) * PASSES youngest have then) and its fragment reads have
+  // returned.  The barrier carries no fence: a fence would wait for every load on its way.
+  constexpr int YOUNGER = (STAGES - 2) * PASSES;
+  auto next_landed = [](bool full_pipeline) {
+    if (full_pipeline) __builtin_amdgcn_s_waitcnt(0x0070 | (YOUNGER & 15) | ((YOUNGER >> 4) << 14));
+    else __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0)
+  };
 
   f32x16 acc[TM][TN];
 #pragma unroll
@@ -411,12 +418,15 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
   const int fr = lane % 32, fh = lane / 32;
-  if (nk > 0) fetch(0, 0);  // a slice beyond the end of K stores zeros
-  loads_landed();
-  __syncthreads();
+#pragma unroll
+  for (int t = 0; t < STAGES - 1; ++t)
+    if (t < nk) fetch(t, t);  // a slice beyond the end of K stores zeros
+  next_landed(nk >= STAGES - 1);
+  __builtin_amdgcn_s_barrier();
   for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < nk) fetch(kt + 1, buf ^ 1);  // the other buffer was last read before the previous barrier
+    const int buf = kt % STAGES;
+    const bool more = kt + STAGES - 1 < nk;
+    if (more) fetch(kt + STAGES - 1, (kt + STAGES - 1) % STAGES);  // that buffer was last read before the previous barrier
     const bf16* xs = smem + (size_t)buf * ROWS * BK;
     const bf16* ws = xs + BM * BK;
 #pragma unroll
@@ -438,27 +448,28 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
     }
-    loads_landed();
-    __syncthreads();
+    next_landed(more);
+    __builtin_amdgcn_s_barrier();
   }
   store_tiles<TM, TN, PAIRED>(acc, out, out_is_f32, blockIdx.y, M, N, m0 + wm, n0 + wn, lane);
 }
 
 // slices > 1 only with a float output [slices, M, N]; K must be a multiple of BK
-template <int BM, int BN, int BK, int WM, int WN, bool PAIRED = false>
+template <int BM, int BN, int BK, int WM, int WN, bool PAIRED = false, int STAGES = 3>
 static int launch_direct(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
                          hipStream_t stream, int slices = 1) {
   SYN_CHECK(K % BK == 0, "gemm: K = %d is no multiple of the k-tile %d", K, BK);
-  const int k_slice = ((K + slices - 1) / slices + 127) / 128 * 128;  // a multiple of BK
-  const size_t lds = (size_t)2 * (BM + BN) * BK * sizeof(bf16);
+  const int step = BK > 128 ? BK : 128;
+  const int k_slice = ((K + slices - 1) / slices + step - 1) / step * step;  // a multiple of BK
+  const size_t lds = (size_t)STAGES * (BM + BN) * BK * sizeof(bf16);
   static bool raised = false;
   if (lds > 65536 && !raised) {
-    const hipError_t e = hipFuncSetAttribute((const void*)gemm_direct_kernel<BM, BN, BK, WM, WN, PAIRED>,
+    const hipError_t e = hipFuncSetAttribute((const void*)gemm_direct_kernel<BM, BN, BK, WM, WN, PAIRED, STAGES>,
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     SYN_CHECK(e == hipSuccess, "gemm: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
     raised = true;
   }
-  gemm_direct_kernel<BM, BN, BK, WM, WN, PAIRED>
+  gemm_direct_kernel<BM, BN, BK, WM, WN, PAIRED, STAGES>
       <<<dim3(tile_grid(M, N, BM, BN), slices), 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
   return 0;
 }
@@ -693,11 +704,12 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   } else if (M <= 32) {
     // few rows: memory-bound; small tiles (many workgroups), deep in K (long pieces of each row);
     // straight into LDS where K allows it (the same speed at 8 rows, a quarter faster at 16 and 32)
-    if (N >= 65536) rc = launch_tiled<32, 32, 256, 1, 1>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
+    if (N >= 65536 && K % 256 == 0) rc = launch_direct<32, 64, 256, 1, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
+    else if (N >= 65536) rc = launch_tiled<32, 32, 256, 1, 1>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
     else if (K % 128 == 0) rc = launch_direct<32, 64, 128, 1, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
     else rc = launch_tiled<32, 64, 128, 1, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
   } else if (M <= 64) {
-    if (K % 128 == 0) rc = launch_direct<64, 64, 128, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
+    if (K % 128 == 0) rc = launch_direct<64, 64, 128, 2, 2, false, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
     else rc = launch_tiled<64, 64, 128, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
   } else {
     rc = launch_large<false>(xb, wb, out, out_is_f32, M, N, K, stream);
@@ -726,7 +738,7 @@ SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, i
     else if (K % 128 == 0) rc = launch_direct<32, 64, 128, 1, 2, true>(xb, wb, out, 0, M, N, K, stream);
     else rc = launch_tiled<32, 64, 128, 1, 2, true>(xb, wb, out, 0, M, N, K, stream);
   } else if (M <= 64) {
-    if (K % 128 == 0) rc = launch_direct<64, 64, 128, 2, 2, true>(xb, wb, out, 0, M, N, K, stream);
+    if (K % 128 == 0) rc = launch_direct<64, 64, 128, 2, 2, true, 2>(xb, wb, out, 0, M, N, K, stream);
     else rc = launch_tiled<64, 64, 128, 2, 2, true>(xb, wb, out, 0, M, N, K, stream);
   } else {
     rc = launch_large<true>(xb, wb, out, 0, M, N, K, stream);

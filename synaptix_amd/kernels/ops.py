@@ -165,13 +165,14 @@ def gemm_swiglu(x, w_paired, out):
 def gemm_slices(M, N, K, dtype):
     """Into how many slices of K a product is cut when its reader can add partial sums.  A product
     with few rows of W has too few workgroups (one for every 64 rows) to pull the weights at speed.
-    The cut aims at one round of workgroups over the 256 compute units, of which each holds three
-    at up to 32 rows of x and two beyond; measured at the shapes of an 8B model (N = 4096 and
-    6144, K = 4096 and 12288) for 1, 8, 32 and 64 rows."""
+    The cut aims at one round of workgroups over the 256 compute units; up to 32 rows of x, where the
+    tiles keep three k-tiles in flight, four slices are enough (and leave the reader fewer partial
+    sums to add); measured at the shapes of an 8B model (N = 4096 and 6144, K = 4096 and 12288) for
+    1, 8, 32 and 64 rows."""
     if dtype != _BF16 or M > 64 or K % 8 != 0 or N > 8192 or K < 2048:
         return 1
     tiles = -(-N // 64)
-    most = min(8, (768 if M <= 32 else 512) // tiles, K // 512)
+    most = min(4 if M <= 32 else 8, (768 if M <= 32 else 512) // tiles, K // 512)
     slices = 1
     while slices * 2 <= most:
         slices *= 2
