@@ -377,9 +377,11 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
   const int k_begin = (int)blockIdx.y * k_slice, k_end = min(K, k_begin + k_slice);
   const int nk = max(0, (k_end - k_begin) / BK);
 
-  // the descriptors begin at the tile's first rows, so a lane's offset stays below 2^32 for any M and N.
-  // pass p: the wave fills tile rows (p * WAVES + wave) * RPI .. + RPI (x rows first, then W rows; rows
-  // beyond M or N repeat the last valid one and their results are never stored)
+  // the descriptors begin at the tile's first rows, so a lane's offset stays below 2^32 for any M and N,
+  // and end with the last row of x and of W: a lane whose row lies beyond reads nothing from memory
+  // (its LDS slot gets zeros, and its results are never stored), which with few rows of x spares
+  // most of the requests for x.
+  // pass p: the wave fills tile rows (p * WAVES + wave) * RPI .. + RPI (x rows first, then W rows)
   static_assert(BM % RPI == 0, "a load lies in x or in W as a whole");
   const size_t row_bytes = (size_t)K * sizeof(bf16);
   const BufferView vx = buffer_view(x + (size_t)m0 * K, (size_t)(M - m0) * row_bytes);
@@ -389,7 +391,7 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
   for (int p = 0; p < PASSES; ++p) {
     const int row0 = (p * WAVES + wave) * RPI, row = row0 + lane / CPR;
     const int chunk = (lane % CPR) ^ direct_swizzle<BK>(row);
-    const int in_tile = row0 < BM ? min(row, M - 1 - m0) : min(row - BM, N - 1 - n0);
+    const int in_tile = row0 < BM ? row : row - BM;
     src[p] = (unsigned)((size_t)in_tile * row_bytes + chunk * 16);
   }
   auto fetch = [&](int kt, int buf) {
