@@ -4,7 +4,8 @@ them, each sequence with its own length, and beside it a fixed-size state for ea
 Layers with the same needs (kv heads, head size, all keys or a window of them) form a group; a
 group has storage and a page pool of its own:
     k_pages [layers, pages, kv_heads, 64, head_dim]
-    v_pages [layers, pages, kv_heads, head_dim, 64]      (transposed inside the page)
+    v_pages [layers, pages, kv_heads, head_dim, 64]      (transposed inside the page; a bf16 page in the
+                                                          order of its kernels, ops.v_pages_to_kernel_order)
 A group that keeps a window gives pages back as soon as every position in them has left the
 window.  Layers with a StateNeed get `state[layer] : [slots, *shape]`, zeroed when a slot is
 taken (the reference keeps such state in the same per-layer vector as the keys and values,

@@ -1,7 +1,9 @@
 // bf16 attention over the paged cache on MFMA, compiled once for each head size (-DSYN_HD=...).
 //
-// Cache pages hold 64 tokens: k_pages[page, kv_head, token, d] and, transposed so that both MFMA
-// operands are contiguous along the contraction, v_pages[page, kv_head, d, token].
+// Cache pages hold 64 tokens: k_pages[page, kv_head, token, d]; the hd x 64 values of a V page of one
+// kv head lie in the order of v_page_offset: transposed, so that both MFMA operands are contiguous
+// along the contraction, and fragment after fragment, so that a decode wave loads each as one
+// contiguous 1 KB.
 //
 // The kernels compute S^T = K . Q^T for a block of 64 keys, so that a lane's accumulator values
 // (4 keys, one query column) are exactly the B operand that O^T += V^T . P^T needs: the
@@ -180,7 +182,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages
       const int c = tid + i * PF_THREADS;
       if (c < 8 * HD) {
         rk[i] = *(const bf16x8*)(kp + (size_t)c * 8);   // K rows are contiguous: chunk c is elements 8c .. 8c+7
-        rv[i] = *(const bf16x8*)(vp + (size_t)c * 8);   // and so are the rows of V^T
+        rv[i] = *(const bf16x8*)(vp + (size_t)c * 8);   // a V page is read as it lies and put in place by stash
       }
     }
   };
@@ -194,7 +196,8 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages
       if (c < 8 * HD) {
         const int key = c / (HD / 8), kcol = c % (HD / 8);
         *(bf16x8*)(ks + tile_slot(key) * LDK + kcol * 8) = rk[i];
-        const int vrow = c / 8, vcol = c % 8;
+        // chunk c of a V page is the fragment c / 64 = h * DT + dt of lane c % 64: dims 16 dt + lane % 16, tokens 32 h + 8 (lane / 16) .. + 8
+        const int vrow = ((c / 64) % DT) * 16 + c % 16, vcol = ((c / 64) / DT) * 4 + (c % 64) / 16;
         bf16x8 v = rv[i];
         if (ragged) {
 #pragma unroll
@@ -359,26 +362,25 @@ __device__ __forceinline__ void load_k_decode(KvBlock& b, const bf16* __restrict
   for (int t = 0; t < 4; ++t) load_row(b.ka[t], kpage + (size_t)tile_row_key(t, r16) * HD, lane);
 }
 
+// a fragment of V is 1 KB of the page, in lane order
 __device__ __forceinline__ void load_v_decode(KvBlock& b, const bf16* __restrict__ vpage, int lane) {
-  const int r16 = lane % 16, g4 = lane / 16;
 #pragma unroll
   for (int h = 0; h < 2; ++h)
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-      b.va[h][dt] = *(const bf16x8*)(vpage + (size_t)(dt * 16 + r16) * SYN_PAGE + h * 32 + 8 * g4);
+    for (int dt = 0; dt < DT; ++dt) b.va[h][dt] = *(const bf16x8*)(vpage + (size_t)((h * DT + dt) * 64 + lane) * 8);
 }
 
-// Head sizes that are a power of two from 32 on: a block's K rows (64 x HD) and its V^T rows (HD x 64) are
-// each one contiguous piece of 128 * HD bytes, and a wave brings them into a piece of LDS of its own
-// with loads of 1 KB that write LDS directly, then reads its fragments from there.  Loading the
-// fragments straight from memory asks the first-level cache for 16 rows x 64 bytes with every
-// instruction, which was measured to keep the texture addresser busy about 100 cycles an instruction
-// and to be what bounds the kernel at large batches.
+// Head sizes that are a power of two from 32 on: a block's K rows (64 x HD) are one contiguous piece of
+// 128 * HD bytes, and a wave brings them into a piece of LDS of its own with loads of 1 KB that write
+// LDS directly, then reads its fragments from there.  Loading K fragments straight from memory asks
+// the first-level cache for 16 rows x 64 bytes with every instruction, which was measured to keep
+// the texture addresser busy about 100 cycles an instruction and to bound the kernel at large
+// batches.  (V needs no such detour: its pages are kept in fragment order.)
 // In LDS the 16-byte chunk c of row r lies at slot c ^ f(r) of the row, with f chosen so that the 16
 // rows a fragment read touches fall into different banks; the permutation is applied to the address
 // that a lane fetches (the slot it fills is fixed by its number) and again by the reader.
 constexpr bool STAGED = !TAIL16 && (HD & (HD - 1)) == 0;
-constexpr int STAGE_BYTES = STAGED ? 128 * HD : 0;   // one block of K, or of V^T
+constexpr int STAGE_BYTES = STAGED ? 128 * HD : 0;   // one block of K
 constexpr int K_CPR = HD / 8;                        // 16-byte chunks in a K row
 // the rows of a score tile differ in bits 0, 1, 3 and 4 of the key number: those four bits, less as
 // many low ones as rows fit into the 256 bytes that the banks span
@@ -386,7 +388,6 @@ __device__ __forceinline__ int k_swizzle(int row) {
   constexpr int DROP = HD >= 128 ? 0 : (HD == 64 ? 1 : 2);
   return ((row & 3) | (((row >> 3) & 3) << 2)) >> DROP;
 }
-__device__ __forceinline__ int v_swizzle(int row) { return (row >> 1) & 7; }  // two rows of 128 bytes span the banks
 
 __device__ __forceinline__ void stage_k(const bf16* __restrict__ kpage, char* stage, int lane) {
   const BufferView view = buffer_view(kpage, STAGE_BYTES);
@@ -396,16 +397,9 @@ __device__ __forceinline__ void stage_k(const bf16* __restrict__ kpage, char* st
     buffer_to_lds16(view, stage + 1024 * i, (unsigned)((row * K_CPR + (slot ^ k_swizzle(row))) * 16), 0);
   }
 }
-__device__ __forceinline__ void stage_v(const bf16* __restrict__ vpage, char* stage, int lane) {
-  const BufferView view = buffer_view(vpage, STAGE_BYTES);
-#pragma unroll
-  for (int i = 0; i < HD / 8; ++i) {
-    const int at = 64 * i + lane, row = at / 8, slot = at % 8;
-    buffer_to_lds16(view, stage + 1024 * i, (unsigned)((row * 8 + (slot ^ v_swizzle(row))) * 16), 0);
-  }
-}
-// the staged piece has landed (this wave's loads are done); nothing that reads it may move above this
-__device__ __forceinline__ void staged_landed() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// The staged K has landed: of this wave's loads at most the V fragments requested after it (2 * DT loads)
+// are still on their way.  Nothing that reads the piece may move above this.
+__device__ __forceinline__ void staged_landed() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * DT) : "memory"); }
 // this wave's reads of the staged piece have returned: the piece may be filled again
 __device__ __forceinline__ void staged_read() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
@@ -420,17 +414,6 @@ __device__ __forceinline__ void read_k_staged(KvBlock& b, const char* stage, int
     }
   }
 }
-__device__ __forceinline__ void read_v_staged(KvBlock& b, const char* stage, int lane) {
-  const int r16 = lane % 16, g4 = lane / 16;
-#pragma unroll
-  for (int h = 0; h < 2; ++h)
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      const int row = dt * 16 + r16;
-      b.va[h][dt] = *(const bf16x8*)(stage + (row * 8 + ((h * 4 + g4) ^ v_swizzle(row))) * 16);
-    }
-}
-
 // One block of 64 keys in two halves, so that the loads of the next block can follow each half at once:
 // the scores and their softmax weights (reads the K fragments), then the weighted values (reads the V fragments).
 __device__ __forceinline__ void decode_scores(AttnState<1>& st, const QFrag& qf, const KvBlock& blk, f32x4 (&s)[4],
@@ -569,12 +552,9 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
   KvBlock blk;
   if (b0 + wave < b1) {
     const size_t base = page_of(b0 + wave);
-    if constexpr (STAGED) {
-      stage_k(k_pages + base, stage, lane);
-    } else {
-      load_k_decode(blk, k_pages + base, lane);
-      load_v_decode(blk, v_pages + base, lane);
-    }
+    if constexpr (STAGED) stage_k(k_pages + base, stage, lane);
+    else load_k_decode(blk, k_pages + base, lane);
+    load_v_decode(blk, v_pages + base, lane);
   }
 
   float* xs = so + (size_t)n_waves * cols_alloc * SO_LD;
@@ -660,8 +640,8 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
             bf16* row = k_pages + page_base + (size_t)(pos % SYN_PAGE) * HD;
             row[d] = o0, row[d + 1] = o1;
           } else if (kind == 2) {
-            bf16* colp = v_pages + page_base + pos % SYN_PAGE;
-            colp[(size_t)d * SYN_PAGE] = o0, colp[(size_t)(d + 1) * SYN_PAGE] = o1;
+            bf16* vpage = v_pages + page_base;
+            vpage[v_page_offset(HD, d, pos % SYN_PAGE)] = o0, vpage[v_page_offset(HD, d + 1, pos % SYN_PAGE)] = o1;
           }
         }
       }
@@ -685,35 +665,27 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
     load_q(qf, valid ? q + ((size_t)seq * nh + kvh * g + hg) * HD : nullptr, lane);
   AttnState<1> st;
   attn_init(st);
-  // K and V of a block come one after the other: while the scores and the softmax of block i are computed
-  // its V is on its way, while its values are added the K of block i + 1 is, so a wave always has half a
-  // block in flight (through its staging piece, or without one into the registers that were just used)
+  // K of the next block is requested as soon as the K fragments of this one are in registers (or have
+  // been used), V of the next block as soon as the V fragments have been used: K is on its way during
+  // the products of this block, V during the scores of the next, without a second set of registers
   for (int kb = b0 + wave; kb < b1; kb += n_waves) {
     const int next = kb + n_waves;
+    const size_t next_base = next < b1 ? page_of(next) : 0;
     f32x4 s[4];
     if constexpr (STAGED) {
-      const size_t base = page_of(kb);
       staged_landed();
       read_k_staged(blk, stage, lane);
       staged_read();
-      stage_v(v_pages + base, stage, lane);
+      if (next < b1) stage_k(k_pages + next_base, stage, lane);
       decode_scores(st, qf, blk, s, kb * SYN_PAGE, valid ? q_lim : -1, lo, scale, lane);
-      decode_weights(st, s, kb * SYN_PAGE, valid ? q_lim : -1, lo, scale, lane);
-      staged_landed();
-      read_v_staged(blk, stage, lane);
-      staged_read();
-      if (next < b1) stage_k(k_pages + page_of(next), stage, lane);
-      decode_values(st, blk, s, kb * SYN_PAGE, n_old, lane);
     } else {
-      const size_t next_base = next < b1 ? page_of(next) : 0;
       decode_scores(st, qf, blk, s, kb * SYN_PAGE, valid ? q_lim : -1, lo, scale, lane);
       if (next < b1) load_k_decode(blk, k_pages + next_base, lane);
-      decode_weights(st, s, kb * SYN_PAGE, valid ? q_lim : -1, lo, scale, lane);
-      decode_values(st, blk, s, kb * SYN_PAGE, n_old, lane);
-      if (next < b1) load_v_decode(blk, v_pages + next_base, lane);
     }
+    decode_weights(st, s, kb * SYN_PAGE, valid ? q_lim : -1, lo, scale, lane);
+    decode_values(st, blk, s, kb * SYN_PAGE, n_old, lane);
+    if (next < b1) load_v_decode(blk, v_pages + next_base, lane);
   }
-  if constexpr (STAGED) staged_landed();   // nothing still on its way into LDS when the wave goes on
   float l = st.l[0];
   l += __shfl_xor(l, 16, SYN_WAVE);
   l += __shfl_xor(l, 32, SYN_WAVE);

@@ -85,6 +85,15 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   return t;
 }
 
+// ---- the order of V inside a bf16 cache page ----
+// A bf16 V page of one kv head holds hd x 64 values (dims x tokens of the page) in the order in which
+// the decode kernel's MFMA takes them: for each half h of the tokens and each 16 dims dt, the 64 lanes'
+// 8 values (lane = 16 * ((token % 32) / 8) + dim % 16, element = token % 8) lie together, so that a
+// fragment is one contiguous 1 KB load.  (A float page is plain [hd][64].)
+__host__ __device__ __forceinline__ int v_page_offset(int hd, int d, int token) {
+  return ((((token >> 5) * (hd >> 4) + (d >> 4)) * 64 + ((token >> 3) & 3) * 16 + (d & 15)) << 3) + (token & 7);
+}
+
 // ---- loads through a buffer descriptor, straight into LDS ----
 // A base and a size in scalar registers, a 32-bit offset a lane, a further offset as a scalar: a load
 // into LDS is then two instructions (LDS address into M0, the load), where a 64-bit address a lane

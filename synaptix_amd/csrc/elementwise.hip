@@ -323,6 +323,7 @@ __global__ void qk_norm_rope_kv_write_kernel(const TIn* __restrict__ qkv, int n_
 
   T* dst;
   size_t dst_stride = 1;
+  bool v_in_mfma_order = false;   // a bf16 V page is kept in the order of v_page_offset
   if (is_q) {
     dst = q_out + ((size_t)tok * nh + head) * hd;
   } else {
@@ -334,6 +335,10 @@ __global__ void qk_norm_rope_kv_write_kernel(const TIn* __restrict__ qkv, int n_
     } else {
       dst = v_pages + base + (pos % SYN_PAGE);
       dst_stride = SYN_PAGE;
+      if (sizeof(T) == 2) {
+        dst = v_pages + base;
+        v_in_mfma_order = true;
+      }
     }
   }
   const bool rotate = (is_q || is_k) && cos_t != nullptr;
@@ -352,8 +357,13 @@ __global__ void qk_norm_rope_kv_write_kernel(const TIn* __restrict__ qkv, int n_
     return o;
   };
   for (int d = 2 * lane; d < hd; d += 2 * SYN_WAVE) {
-    dst[(size_t)d * dst_stride] = from_f32<T>(rotated(d));
-    dst[(size_t)(d + 1) * dst_stride] = from_f32<T>(rotated(d + 1));
+    if (v_in_mfma_order) {
+      dst[v_page_offset(hd, d, pos % SYN_PAGE)] = from_f32<T>(rotated(d));
+      dst[v_page_offset(hd, d + 1, pos % SYN_PAGE)] = from_f32<T>(rotated(d + 1));
+    } else {
+      dst[(size_t)d * dst_stride] = from_f32<T>(rotated(d));
+      dst[(size_t)(d + 1) * dst_stride] = from_f32<T>(rotated(d + 1));
+    }
   }
 }
 
@@ -442,9 +452,9 @@ qk_heads_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ q_out, bf16* __
   }
 }
 
-// The v heads of the same rows: 64 tokens x 32 dims a block go through LDS, so that a transposed row
-// of a page (64 positions of one dim) is written as one 128-byte piece wherever positions are
-// consecutive.
+// The v heads of the same rows: 64 tokens x 32 dims a block go through LDS and are written in the
+// order of v_page_offset, in which 8 consecutive positions of one dim are one 16-byte piece and the
+// 16 dims of a fragment follow each other at 16 bytes.
 #define V_DIMS 32
 __global__ void __launch_bounds__(256)
 v_block_write_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ v_pages, const int* __restrict__ page_table,
@@ -453,6 +463,7 @@ v_block_write_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ v_pages, c
   constexpr int LD = V_DIMS + 2, PAIRS = V_DIMS / 2;
   __shared__ __attribute__((aligned(16))) bf16 vtile[64 * LD];
   __shared__ size_t dst_base[SYN_PAGE];
+  __shared__ int dst_slot[SYN_PAGE];
   const int tid = threadIdx.x, t0 = blockIdx.x * 64, kvh = blockIdx.y, d0 = blockIdx.z * V_DIMS;
   const int heads = nh + 2 * nkv;
   for (int idx = tid; idx < 64 * PAIRS; idx += 256) {
@@ -464,13 +475,14 @@ v_block_write_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ v_pages, c
   if (tid < 64 && t0 + tid < n_tokens) {
     const int tok = t0 + tid, pos = tok_pos[tok];
     const int page = page_table[(size_t)tok_seq[tok] * table_stride + pos / SYN_PAGE];
-    dst_base[tid] = ((size_t)page * nkv + kvh) * SYN_PAGE * hd + pos % SYN_PAGE;
+    dst_base[tid] = ((size_t)page * nkv + kvh) * SYN_PAGE * hd;
+    dst_slot[tid] = pos % SYN_PAGE;
   }
   __syncthreads();
   const int j = tid % 64;
   if (t0 + j < n_tokens)
     for (int d = tid / 64; d < V_DIMS && d0 + d < hd; d += 4)
-      v_pages[dst_base[j] + (size_t)(d0 + d) * SYN_PAGE] = vtile[j * LD + d];
+      v_pages[dst_base[j] + v_page_offset(hd, d0 + d, dst_slot[j])] = vtile[j * LD + d];
 }
 
 SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, int n_parts, void* q_out, void* k_pages, void* v_pages,

@@ -181,6 +181,30 @@ def gemm_slices(M, N, K, dtype):
 
 # ----------------------------------------------------------------------------- attention
 
+def v_pages_to_kernel_order(v):
+    """V pages [..., kv_heads, hd, 64] as plain (dim, token) rows -> the same shape holding each page
+    in the order the bf16 kernels keep it (fragment after fragment of the decode kernel's MFMA: half of
+    the tokens, 16 dims, lane group of 8 tokens, dim, token).  Float pages are plain and stay as they are."""
+    if v.dtype != _BF16:
+        return v
+    lead, hd = v.shape[:-2], v.shape[-2]
+    x = v.reshape(*lead, hd // 16, 16, 2, 4, 8)            # [dt, r, h, g, e]
+    n = len(lead)
+    x = x.permute(*range(n), n + 2, n + 0, n + 3, n + 1, n + 4)   # [h, dt, g, r, e]
+    return x.reshape(*lead, hd, 64).contiguous()
+
+
+def v_pages_from_kernel_order(v):
+    """The inverse of v_pages_to_kernel_order."""
+    if v.dtype != _BF16:
+        return v
+    lead, hd = v.shape[:-2], v.shape[-2]
+    x = v.reshape(*lead, 2, hd // 16, 4, 16, 8)            # [h, dt, g, r, e]
+    n = len(lead)
+    x = x.permute(*range(n), n + 1, n + 3, n + 0, n + 2, n + 4)   # [dt, r, h, g, e]
+    return x.reshape(*lead, hd, 64).contiguous()
+
+
 def _check_pages(k_pages, v_pages, dtype, nkv, hd, name):
     _need(k_pages, name + ".k_pages", dtype, (None, nkv, PAGE_TOKENS, hd))
     _need(v_pages, name + ".v_pages", dtype, (k_pages.shape[0], nkv, hd, PAGE_TOKENS))

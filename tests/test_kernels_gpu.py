@@ -224,6 +224,18 @@ def test_gemm_bf16_paths_agree(ops):
 
 # ----------------------------------------------------------------------------- cache write + attention
 
+def dv(v):
+    """V pages as plain (dim, token) rows on the CPU -> on the device in the kernels' own order."""
+    from synaptix_amd.kernels import ops as real_ops
+    return real_ops.v_pages_to_kernel_order(v).to(DEV)
+
+
+def hv(v):
+    """V pages from the device back to plain (dim, token) rows on the CPU."""
+    from synaptix_amd.kernels import ops as real_ops
+    return real_ops.v_pages_from_kernel_order(v.cpu())
+
+
 def make_cache(n_pages, nkv, hd, dtype, seed, fill="garbage"):
     """Pages filled with large values: whatever a kernel reads beyond a sequence's end shows."""
     k = rnd((n_pages, nkv, 64, hd), seed, dtype, 50.0)
@@ -269,13 +281,13 @@ def test_qk_norm_rope_kv_write(ops, dtype, nh, nkv, hd, rot, norm):
     kw, vw, qw = k0.clone(), v0.clone(), torch.empty((N, nh * hd), dtype=dtype)
     ref.qk_norm_rope_kv_write(qkv, qw, kw, vw, table, tok_seq, tok_pos, qg, kg, 1e-5, cos, sin, nh, nkv, hd)
     d = lambda t: None if t is None else t.to(DEV)
-    kd, vd, qd = k0.to(DEV), v0.to(DEV), torch.empty((N, nh * hd), dtype=dtype, device=DEV)
+    kd, vd, qd = k0.to(DEV), dv(v0), torch.empty((N, nh * hd), dtype=dtype, device=DEV)
     ops.qk_norm_rope_kv_write(d(qkv), qd, kd, vd, d(table), d(tok_seq), d(tok_pos), d(qg), d(kg), 1e-5, d(cos), d(sin),
                               nh, nkv, hd)
     tol = dict(atol=1e-5, rtol=1e-5) if dtype == F32 else dict(atol=3e-2, rtol=1e-2)
     close(qd, qw, what="q", **tol)
     close(kd, kw, what="k pages", **tol)
-    assert torch.equal(vd.cpu(), vw), "v is a copy"
+    assert torch.equal(hv(vd), vw), "v is a copy"
     # untouched places of the pages stay as they were
     untouched = (kw == k0)
     assert torch.equal(kd.cpu()[untouched], k0[untouched])
@@ -283,17 +295,17 @@ def test_qk_norm_rope_kv_write(ops, dtype, nh, nkv, hd, rot, norm):
     if dtype == BF16:
         parts = rnd((3, N, (nh + 2 * nkv) * hd), 24)
         parts[2] = qkv.float() - parts[0] - parts[1]
-        kd3, vd3, qd3 = k0.to(DEV), v0.to(DEV), torch.empty((N, nh * hd), dtype=dtype, device=DEV)
+        kd3, vd3, qd3 = k0.to(DEV), dv(v0), torch.empty((N, nh * hd), dtype=dtype, device=DEV)
         ops.qk_norm_rope_kv_write(d(parts), qd3, kd3, vd3, d(table), d(tok_seq), d(tok_pos), d(qg), d(kg), 1e-5, d(cos),
                                   d(sin), nh, nkv, hd)
         close(qd3, qw, what="q from partial sums", **tol)
         close(kd3, kw, what="k pages from partial sums", **tol)
-        close(vd3, vw, 2e-2, 1e-2, what="v pages from partial sums")
+        close(hv(vd3), vw, 2e-2, 1e-2, what="v pages from partial sums")
     # a reader of another layer's cache writes nothing
-    kd2, vd2 = k0.to(DEV), v0.to(DEV)
+    kd2, vd2 = k0.to(DEV), dv(v0)
     ops.qk_norm_rope_kv_write(d(qkv), qd, kd2, vd2, d(table), d(tok_seq), d(tok_pos), d(qg), d(kg), 1e-5, d(cos), d(sin),
                               nh, nkv, hd, write_kv=False)
-    assert torch.equal(kd2.cpu(), k0) and torch.equal(vd2.cpu(), v0)
+    assert torch.equal(kd2.cpu(), k0) and torch.equal(hv(vd2), v0)
     close(qd, qw, what="q without cache write", **tol)
 
 
@@ -339,10 +351,10 @@ def test_attention_prefill(ops, dtype, nh, nkv, hd, past, new, window):
     d = lambda t: t.to(DEV)
     out = torch.empty((N, nh * hd), dtype=dtype, device=DEV)
     if dtype == F32:
-        ops.attention_f32(d(q), d(k), d(v), d(table), d(tok_seq), d(tok_pos), out, scale, window, nh, nkv, hd)
+        ops.attention_f32(d(q), d(k), dv(v), d(table), d(tok_seq), d(tok_pos), out, scale, window, nh, nkv, hd)
         close(out, want, 1e-4, what="attention f32")
     else:
-        ops.attention_prefill_bf16(d(q), d(k), d(v), d(table), d(starts), d(past_t), out, scale, window, nh, nkv, hd)
+        ops.attention_prefill_bf16(d(q), d(k), dv(v), d(table), d(starts), d(past_t), out, scale, window, nh, nkv, hd)
         close(out, want, 2e-2, 1e-2, what="attention prefill bf16")
 
 
@@ -375,7 +387,7 @@ def test_attention_decode_bf16(ops, nh, nkv, hd, lens, window, splits):
     d = lambda t: t.to(DEV)
     out = torch.empty((B, nh * hd), dtype=BF16, device=DEV)
     work = torch.empty(B * nh * splits * (hd + 2), dtype=F32, device=DEV)
-    ops.attention_decode_bf16(d(q), d(k), d(v), d(table), d(torch.tensor(lens, dtype=I32)), out, work, splits, scale,
+    ops.attention_decode_bf16(d(q), d(k), dv(v), d(table), d(torch.tensor(lens, dtype=I32)), out, work, splits, scale,
                               window, nh, nkv, hd)
     close(out, want, 2e-2, 1e-2, what="attention decode bf16")
 
@@ -419,7 +431,7 @@ def test_attention_decode_with_qkv_intake(ops, nh, nkv, hd, rot, norm, lens, win
     want = torch.empty((B, nh * hd), dtype=F32)
     ref.attention_f32(q_ref.float(), k_ref.float(), v_ref.float(), table, tok_seq, tok_pos, want, scale, window, nh, nkv, hd)
     d = lambda t: None if t is None else t.to(DEV)
-    kd, vd = d(k), d(v)
+    kd, vd = d(k), dv(v)
     out = torch.empty((B, nh * hd), dtype=BF16, device=DEV)
     work = torch.empty(B * nh * splits * (hd + 2), dtype=F32, device=DEV)
     ops.attention_decode_fused_bf16(d(qkv), kd, vd, d(table), d(seq_len), out, work, splits, scale, window, nh, nkv, hd,
@@ -427,9 +439,9 @@ def test_attention_decode_with_qkv_intake(ops, nh, nkv, hd, rot, norm, lens, win
     close(out, want, 2e-2, 1e-2, what="decode attention with q/k/v intake")
     # the cache afterwards: the new rows written (or nothing touched)
     close(kd, k_ref.float(), 2e-2, 1e-2, what="k pages after the step")
-    close(vd, v_ref.float(), 2e-2, 1e-2, what="v pages after the step")
+    close(hv(vd), v_ref.float(), 2e-2, 1e-2, what="v pages after the step")
     if not own:
-        assert torch.equal(kd.cpu(), k) and torch.equal(vd.cpu(), v)
+        assert torch.equal(kd.cpu(), k) and torch.equal(hv(vd), v)
 
 
 def test_attention_far_key_stands_out(ops):
@@ -451,12 +463,12 @@ def test_attention_far_key_stands_out(ops):
         lens = torch.tensor([T], dtype=I32)
         out = torch.empty((1, nh * hd), dtype=BF16, device=DEV)
         work = torch.empty(nh * 6 * (hd + 2), dtype=F32, device=DEV)
-        ops.attention_decode_bf16(d(q), d(k), d(v), d(table), d(lens), out, work, 6, scale, 0, nh, nkv, hd)
+        ops.attention_decode_bf16(d(q), d(k), dv(v), d(table), d(lens), out, work, 6, scale, 0, nh, nkv, hd)
         got = out.cpu().float().view(nh, hd)
         for h in range(nkv):
             close(got[h * 2], want[h], 3e-2, 2e-2, f"decode, far key {far}")
         outp = torch.empty((1, nh * hd), dtype=BF16, device=DEV)
-        ops.attention_prefill_bf16(d(q), d(k), d(v), d(table), d(torch.tensor([0, 1], dtype=I32)),
+        ops.attention_prefill_bf16(d(q), d(k), dv(v), d(table), d(torch.tensor([0, 1], dtype=I32)),
                                    d(torch.tensor([T - 1], dtype=I32)), outp, scale, 0, nh, nkv, hd)
         gotp = outp.cpu().float().view(nh, hd)
         for h in range(nkv):
@@ -489,10 +501,10 @@ def test_attention_window_edge(ops):
     d = lambda t: t.to(DEV)
     out = torch.empty((1, nh * hd), dtype=BF16, device=DEV)
     work = torch.empty(nh * 3 * (hd + 2), dtype=F32, device=DEV)
-    ops.attention_decode_bf16(d(q), d(k), d(v), d(table), d(torch.tensor([T], dtype=I32)), out, work, 3, scale, W, nh,
+    ops.attention_decode_bf16(d(q), d(k), dv(v), d(table), d(torch.tensor([T], dtype=I32)), out, work, 3, scale, W, nh,
                               nkv, hd)
     close(out, want, 2e-2, 1e-2, "decode at the window's edge")
-    ops.attention_prefill_bf16(d(q), d(k), d(v), d(table), d(torch.tensor([0, 1], dtype=I32)),
+    ops.attention_prefill_bf16(d(q), d(k), dv(v), d(table), d(torch.tensor([0, 1], dtype=I32)),
                                d(torch.tensor([T - 1], dtype=I32)), out, scale, W, nh, nkv, hd)
     close(out, want, 2e-2, 1e-2, "prefill at the window's edge")
     o32 = torch.empty((1, nh * hd), dtype=F32, device=DEV)
