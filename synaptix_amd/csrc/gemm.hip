@@ -164,11 +164,13 @@ static void launch_skinny(const bf16* x, const bf16* w, void* out, int out_is_f3
 // Which tile: workgroup b runs on XCD b % 8, and each XCD has an L2 of its own.  Tiles are grouped
 // into panels of PM x PN (m fastest); a panel goes to one XCD, so the workgroups that run there at
 // the same time share rows of x and of W in its L2.  False for the launches that pad the last panels.
+// With slices of K (blockIdx.y) the panels of slice s are handed out s * panels XCDs further on, so
+// that a product of fewer than 8 panels still reaches every XCD.
 __device__ __forceinline__ bool tile_of_workgroup(int M, int N, int BM, int BN, int& tm, int& tn) {
   const int tiles_n = (N + BN - 1) / BN, tiles_m = (M + BM - 1) / BM;
   const int PM = min(8, tiles_m), PN = 4;
-  const int panels_m = (tiles_m + PM - 1) / PM;
-  const int xcd = (int)blockIdx.x % 8, local = (int)blockIdx.x / 8;
+  const int panels_m = (tiles_m + PM - 1) / PM, panels = panels_m * ((tiles_n + PN - 1) / PN);
+  const int xcd = ((int)blockIdx.x + 8 - (int)((blockIdx.y * panels) % 8)) % 8, local = (int)blockIdx.x / 8;
   const int panel = (local / (PM * PN)) * 8 + xcd, in_panel = local % (PM * PN);
   tm = (panel % panels_m) * PM + in_panel % PM;
   tn = (panel / panels_m) * PN + in_panel / PM;
@@ -493,7 +495,7 @@ static int launch_direct(const bf16* x, const bf16* w, void* out, int out_is_f32
 template <int BM, int BN, int WM, int WN, bool PAIRED>
 __global__ void __launch_bounds__(64 * WM * WN)
 gemm_pipelined_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
-                      int M, int N, int K) {
+                      int M, int N, int K, int k_slice) {
   constexpr int BK = 64;
   constexpr int WAVES = WM * WN;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -509,12 +511,15 @@ gemm_pipelined_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, vo
   int tm, tn;
   if (!tile_of_workgroup(M, N, BM, BN, tm, tn)) return;
   const int m0 = tm * BM, n0 = tn * BN;
-  const int nk = K / BK;
+  // blockIdx.y = which slice of K (k_slice elements, a multiple of BK) this workgroup sums; a slice is never empty
+  const int k_begin = (int)blockIdx.y * k_slice;
+  const int nk = (min(K, k_begin + k_slice) - k_begin) / BK;
 
-  // the descriptors begin at the tile's first rows, so a lane's offset stays below 2^32 for any M and N
+  // the descriptors begin at the tile's first rows and the slice's first column, so a lane's offset stays
+  // below 2^32 for any M and N
   const size_t row_bytes = (size_t)K * sizeof(bf16);
-  const BufferView vx = buffer_view(x + (size_t)m0 * K, (size_t)(M - m0) * row_bytes);
-  const BufferView vw = buffer_view(w + (size_t)n0 * K, (size_t)(N - n0) * row_bytes);
+  const BufferView vx = buffer_view(x + (size_t)m0 * K + k_begin, (size_t)(M - m0) * row_bytes - k_begin * sizeof(bf16));
+  const BufferView vw = buffer_view(w + (size_t)n0 * K + k_begin, (size_t)(N - n0) * row_bytes - k_begin * sizeof(bf16));
   // pass p: the wave fills tile rows (p * WAVES + wave) * 8 .. + 8 (x rows first, then W rows; rows beyond M or
   // N repeat the last valid one and their results are never stored)
   unsigned src[PASSES];
@@ -613,13 +618,15 @@ gemm_pipelined_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, vo
   for (; kt + 2 < nk; ++kt) tile(kt, std::true_type{}, std::true_type{});
   if (kt + 1 < nk) tile(kt++, std::false_type{}, std::true_type{});
   tile(kt, std::false_type{}, std::false_type{});
-  store_tiles<TM, TN, PAIRED>(acc, out, out_is_f32, 0, M, N, m0 + wm, n0 + wn, lane);
+  store_tiles<TM, TN, PAIRED>(acc, out, out_is_f32, blockIdx.y, M, N, m0 + wm, n0 + wn, lane);
 }
 
 template <int BM, int BN, int WM, int WN, bool PAIRED = false>
 static int launch_pipelined(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
-                            hipStream_t stream) {
+                            hipStream_t stream, int slices = 1) {
   SYN_CHECK(K % 64 == 0, "gemm: K = %d is no multiple of the k-tile 64", K);
+  const int k_slice = ((K + slices - 1) / slices + 127) / 128 * 128;  // the same cut as the tiles for few rows make
+  SYN_CHECK((long)(slices - 1) * k_slice < K, "gemm: %d slices of %d leave the last one empty (K = %d)", slices, k_slice, K);
   const size_t lds = (size_t)2 * (BM + BN) * 64 * sizeof(bf16);
   static bool raised = false;
   if (lds > 65536 && !raised) {
@@ -629,14 +636,14 @@ static int launch_pipelined(const bf16* x, const bf16* w, void* out, int out_is_
     raised = true;
   }
   gemm_pipelined_kernel<BM, BN, WM, WN, PAIRED>
-      <<<tile_grid(M, N, BM, BN), 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K);
+      <<<dim3(tile_grid(M, N, BM, BN), slices), 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
   return 0;
 }
 
 // M > 64: the tile shape by pick_large_tile; loads straight into LDS where K allows it
 template <bool PAIRED>
 static int launch_large(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
-                        hipStream_t stream);
+                        hipStream_t stream, int slices = 1);
 
 // Which of the large tiles for M > 64: 0 = 256 x 256, 1 = 256 x 192 (one workgroup a compute unit; about
 // 6 % less efficient), 2 = 128 x 128 (two workgroups a compute unit, about 20 % less efficient).
@@ -656,7 +663,9 @@ static int pick_large_tile(int M, int N) {
 
 template <bool PAIRED>
 static int launch_large(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
-                        hipStream_t stream) {
+                        hipStream_t stream, int slices) {
+  // cut along K (the reader adds the partial sums): the largest tile, which the slices multiply
+  if (slices > 1) return launch_pipelined<256, 256, 2, 4, PAIRED>(x, w, out, out_is_f32, M, N, K, stream, slices);
   const int shape = pick_large_tile(M, N);
   if (K % 64 == 0) {
     if (shape == 0) return launch_pipelined<256, 256, 2, 4, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
@@ -670,14 +679,14 @@ static int launch_large(const bf16* x, const bf16* w, void* out, int out_is_f32,
 
 // ------------------------------------------------------------------ entry point
 // dtype: 0 = float in, float out; 1 = bf16 in, bf16 out; 2 = bf16 in, float out.
-// slices > 1 (bf16 in, float out, M <= 64 only): out is [slices, M, N], slice s holds the sum over its
-// part of K; the reader adds the slices.
+// slices > 1 (bf16 in, float out): out is [slices, M, N], slice s holds the sum over its part of K; the
+// reader adds the slices.
 SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int M, int N, int K, int force_simt,
                         int slices, hipStream_t stream) {
   SYN_CHECK(M > 0 && N > 0 && K > 0, "gemm: empty shape M=%d N=%d K=%d", M, N, K);
   SYN_CHECK(dtype >= 0 && dtype <= 2, "gemm: unknown dtype code %d", dtype);
-  SYN_CHECK(slices >= 1 && (slices == 1 || (dtype == 2 && M <= 64 && !force_simt && K % 8 == 0 && slices <= 64)),
-            "gemm: %d slices of K need bf16 operands, a float output and M <= 64 (M = %d)", slices, M);
+  SYN_CHECK(slices >= 1 && (slices == 1 || (dtype == 2 && !force_simt && K % 8 == 0 && slices <= 64 && (M <= 64 || K % 64 == 0))),
+            "gemm: %d slices of K need bf16 operands and a float output (and beyond 64 rows a K that is a multiple of 64; K = %d)", slices, K);
   const dim3 simt_grid((N + SIMT_BN - 1) / SIMT_BN, (M + SIMT_BM - 1) / SIMT_BM);
   if (dtype == 0) {
     gemm_simt_kernel<float, float><<<simt_grid, 256, 0, stream>>>((const float*)x, (const float*)w, (float*)out, M, N, K);
@@ -714,7 +723,7 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
     if (K % 128 == 0) rc = launch_direct<64, 64, 128, 2, 2, false, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
     else rc = launch_tiled<64, 64, 128, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
   } else {
-    rc = launch_large<false>(xb, wb, out, out_is_f32, M, N, K, stream);
+    rc = launch_large<false>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
   }
   if (rc) return rc;
   SYN_LAUNCH_CHECK("gemm");

@@ -115,8 +115,8 @@ def swiglu(gate_up, out):
 def gemm(x, w, out, force_simt=False):
     """out[M, N] = x[M, K] . w[N, K]^T with 32-bit accumulation.
     float x float -> float (plain FMA); bf16 x bf16 -> bf16 or float (MFMA).
-    A float out of shape [S, M, N] (bf16 operands, M <= 64) receives S partial sums over slices
-    of K instead; their sum over S is the product."""
+    A float out of shape [S, M, N] (bf16 operands) receives S partial sums over slices of K
+    instead; their sum over S is the product."""
     _need(x, "gemm.x", (_BF16, _F32), (None, None))
     M, K = x.shape
     _need(w, "gemm.w", x.dtype, (None, K))
@@ -124,8 +124,9 @@ def gemm(x, w, out, force_simt=False):
     slices = 1
     if out.dim() == 3:
         slices = out.shape[0]
-        if x.dtype != _BF16 or M > 64 or force_simt:
-            raise KernelError("gemm: partial sums over slices of K need bf16 operands and M <= 64")
+        if x.dtype != _BF16 or force_simt or (M > 64 and K % 64):
+            raise KernelError("gemm: partial sums over slices of K need bf16 operands (and beyond 64 rows a K "
+                              "that is a multiple of 64)")
         _need(out, "gemm.out", _F32, (slices, M, N))
         code = 2
     elif x.dtype == _F32:
@@ -169,8 +170,16 @@ def gemm_slices(M, N, K, dtype):
     tiles keep three k-tiles in flight, four slices are enough (and leave the reader fewer partial
     sums to add); measured at the shapes of an 8B model (N = 4096 and 6144, K = 4096 and 12288) for
     1, 8, 32 and 64 rows."""
-    if dtype != _BF16 or M > 64 or K % 8 != 0 or N > 8192 or K < 2048:
+    if dtype != _BF16 or K % 8 != 0 or N > 8192 or K < 2048:
         return 1
+    if M > 64:
+        # prompts: 256 x 256 tiles are the most efficient, but a narrow product has too few of them for
+        # the 256 compute units (128 at 2,048 rows and N = 4096); two or four slices of K fill the chip,
+        # at the price of partial sums of M x N floats each
+        if K % 128:
+            return 1
+        tiles = -(-M // 256) * -(-N // 256)
+        return 4 if tiles * 4 <= 256 and K >= 8192 else (2 if tiles * 2 <= 256 else 1)
     tiles = -(-N // 64)
     most = min(4 if M <= 32 else 8, (768 if M <= 32 else 512) // tiles, K // 512)
     slices = 1

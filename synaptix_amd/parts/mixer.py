@@ -88,8 +88,9 @@ class GqaAttention(Mixer):
         cap = self.position.capacity
         if cap is not None and ctx.max_position >= cap:
             raise ValueError(f"position {ctx.max_position} is beyond the position encoding's capacity {cap}")
-        qkv = linear_for_sum(h, self.w_qkv) if ops.gemm_slices(N, self.w_qkv.shape[0], self.hidden, act) > 1 \
-            else linear(h, self.w_qkv, act)             # partial sums over slices of K, or the plain product
+        # single tokens: partial sums over slices of K, which the attention kernel adds; prompts: the plain product
+        qkv = linear_for_sum(h, self.w_qkv) if N <= 64 and ops.gemm_slices(N, self.w_qkv.shape[0], self.hidden, act) > 1 \
+            else linear(h, self.w_qkv, act)
         cos, sin = self.position.tables(h.device)
         table = ctx.page_table(cache.group)
         o = torch.empty((N, nh * hd), dtype=act, device=h.device)

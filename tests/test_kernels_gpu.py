@@ -157,7 +157,8 @@ def test_gemm_bf16(ops, out_dtype, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K,S", [(1, 48, 4096, 4), (8, 4096, 4096, 4), (8, 100, 1000, 3), (16, 64, 12288, 8),
-                                     (40, 70, 2048, 2), (64, 130, 520, 5), (8, 96, 1536, 5), (50, 200, 3072, 7)])
+                                     (40, 70, 2048, 2), (64, 130, 520, 5), (8, 96, 1536, 5), (50, 200, 3072, 7),
+                                     (300, 520, 1024, 2), (130, 260, 640, 3), (65, 33, 4096, 4)])
 def test_gemm_bf16_partial_sums_over_slices_of_k(ops, M, N, K, S):
     """[S, M, N]: slice s holds the sum over its part of K; the slices add up to the product, also
     when K is no multiple of the slice and the last slices are short or empty."""
