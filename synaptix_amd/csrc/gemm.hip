@@ -5,6 +5,8 @@
 //   gemm_skinny    bf16, M == 1: the weight matrix is streamed once from HBM through
 //                  v_mfma_f32_16x16x32_bf16; the waves of a workgroup split K and sum in LDS
 //                  (also over paired gate/up rows, with the gated activation as the epilogue).
+//   gemm_packed    bf16, M <= 16 (used up to 8): the same over a copy of W kept in the order of the MFMA
+//                  fragments, so that every load of a wave is 1 KB of consecutive bytes.
 //   gemm_tiled     bf16: tiles of x and W in LDS, double-buffered, v_mfma_f32_32x32x16_bf16.
 //                  M > 64: 256x256x64, 256x192x64 or 128x128x64 tiles; when K is a multiple of 64 by
 //                  gemm_pipelined, whose loads write LDS without passing through registers and are
@@ -158,6 +160,88 @@ static void launch_skinny(const bf16* x, const bf16* w, void* out, int out_is_f3
   const int rows = TILES * 16;
   gemm_skinny_kernel<TILES, KWAVES, U, PAIRED>
       <<<(N + rows - 1) / rows, TILES * KWAVES * SYN_WAVE, 0, stream>>>(x, w, out, out_is_f32, M, N, K);
+}
+
+// ------------------------------------------------------------------ few rows of x, W in fragment order
+// The same scheme as gemm_skinny (up to 16 rows of x, K split over the waves of a group, partial
+// tiles summed in LDS in a fixed order) over a copy of W that is kept in the order of the MFMA
+// fragments: wp[N / 16][K / 32][64 lanes][8], lane = 16 * (k % 32 / 8) + n % 16.  A wave's load of a
+// fragment is then 1 KB of consecutive bytes, and the fragments of a group of rows follow each other
+// along K: the weight stream is read as a kernel that does nothing else reads it (measured 6.2 to
+// 6.7 TB/s on the wide products, against 4.5 to 5.3 from rows of W).  The fragments of x come from
+// memory for every wave (x stays in the caches); that costs as many requests as W from 16 rows on,
+// so the callers use this kernel up to 8 rows.  Wave kw of a group takes the k-steps kw * U .. + U,
+// then those KWAVES * U further on.
+template <int TILES, int KWAVES, int U, bool PAIRED>
+__global__ void __launch_bounds__(TILES * KWAVES * SYN_WAVE)
+gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void* __restrict__ out, int out_is_f32,
+                   int M, int N, int K) {
+  static_assert(!PAIRED || TILES == 2, "a pair is two tiles");
+  constexpr int WAVES = TILES * KWAVES;
+  __shared__ float part[WAVES][4][64];
+  const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
+  const int tile = wave / KWAVES, kw = wave % KWAVES;
+  const int r16 = lane % 16, kq = (lane / 16) * 8;
+  const int nt = (int)blockIdx.x * TILES + tile, n_tiles = N / 16;   // 16 rows of W
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int nks = K / 32;
+  const bool tile_in = nt < n_tiles;   // the last workgroup may hold a group beyond the end
+  const bf16* wt = wp + ((size_t)min(nt, n_tiles - 1) * nks * 64 + lane) * 8;
+  const bool xok = r16 < M;
+  const bf16* xrow = x + (size_t)min(r16, M - 1) * K + kq;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  if (tile_in) {
+    for (int ks0 = kw * U; ks0 < nks; ks0 += KWAVES * U) {
+      bf16x8 bw[U], ax[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const bool in = ks0 + u < nks;
+        bw[u] = in ? __builtin_nontemporal_load((const bf16x8*)(wt + (size_t)(ks0 + u) * 512)) : zero;
+        ax[u] = (in && xok) ? *(const bf16x8*)(xrow + (ks0 + u) * 32) : zero;
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[u], bw[u], acc, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) part[wave][j][lane] = acc[j];
+  __syncthreads();
+  auto summed = [&](int t, int j, int ln) {
+    float s = 0.f;
+#pragma unroll
+    for (int q = 0; q < KWAVES; ++q) s += part[t * KWAVES + q][j][ln];
+    return s;
+  };
+  if constexpr (PAIRED) {
+    for (int idx = threadIdx.x; idx < 4 * 64; idx += WAVES * SYN_WAVE) {
+      const int j = idx / 64, ln = idx % 64;
+      const int m = 4 * (ln / 16) + j, col = (int)blockIdx.x * 16 + ln % 16;  // N / 2 outputs, 16 a workgroup
+      if (m < M && 2 * col < N) {
+        const float g = summed(0, j, ln), up = summed(1, j, ln);
+        ((bf16*)out)[(size_t)m * (N / 2) + col] = (bf16)(g / (1.f + expf(-g)) * up);
+      }
+    }
+  } else {
+    for (int idx = threadIdx.x; idx < TILES * 4 * 64; idx += WAVES * SYN_WAVE) {
+      const int t = idx / 256, j = (idx / 64) % 4, ln = idx % 64;
+      const int m = 4 * (ln / 16) + j, n = ((int)blockIdx.x * TILES + t) * 16 + ln % 16;
+      if (m < M && n < N) {
+        const float v = summed(t, j, ln);
+        if (out_is_f32)
+          ((float*)out)[(size_t)m * N + n] = v;
+        else
+          ((bf16*)out)[(size_t)m * N + n] = (bf16)v;
+      }
+    }
+  }
+}
+
+template <int TILES, int KWAVES, int U, bool PAIRED = false>
+static void launch_packed(const bf16* x, const bf16* wp, void* out, int out_is_f32, int M, int N, int K,
+                          hipStream_t stream) {
+  const int rows = TILES * 16;
+  gemm_packed_kernel<TILES, KWAVES, U, PAIRED>
+      <<<(N + rows - 1) / rows, TILES * KWAVES * SYN_WAVE, 0, stream>>>(x, wp, out, out_is_f32, M, N, K);
 }
 
 // ------------------------------------------------------------------ shared by the tiled kernels
@@ -756,5 +840,26 @@ SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, i
   }
   if (rc) return rc;
   SYN_LAUNCH_CHECK("gemm_swiglu");
+  return 0;
+}
+
+// The products above for up to 16 rows of x over wp, a copy of W [N, K] in fragment order (see
+// gemm_packed_kernel; N a multiple of 16, K of 32).  out_code: 1 = bf16 [M, N], 2 = float [M, N];
+// paired: W holds gate and up rows in turns of 16 and out is bf16 [M, N / 2] = silu(gate) * up.
+SYN_EXPORT int syn_gemm_packed(const void* x, const void* wp, void* out, int out_code, int M, int N, int K, int paired,
+                               hipStream_t stream) {
+  SYN_CHECK(M > 0 && M <= 16 && N > 0 && K > 0, "gemm_packed: M = %d (1 .. 16), N = %d, K = %d", M, N, K);
+  SYN_CHECK(N % 16 == 0 && K % 32 == 0 && (!paired || N % 32 == 0),
+            "gemm_packed: N = %d must be a multiple of 16 (32 for paired rows), K = %d of 32", N, K);
+  SYN_CHECK(out_code == 1 || out_code == 2, "gemm_packed: unknown output code %d", out_code);
+  SYN_CHECK(!paired || out_code == 1, "gemm_packed: the gated product is stored as bf16");
+  SYN_CHECK((uintptr_t)x % 16 == 0 && (uintptr_t)wp % 16 == 0, "gemm_packed: operands must be 16-byte aligned");
+  const bf16* xb = (const bf16*)x;
+  const bf16* wb = (const bf16*)wp;
+  // from sweeps at N = 4096 .. 151936, K = 4096 and 12288, 1 and 8 rows
+  if (paired) launch_packed<2, 8, 4, true>(xb, wb, out, 0, M, N, K, stream);
+  else if (N <= 8192) launch_packed<1, 16, 2>(xb, wb, out, out_code == 2, M, N, K, stream);
+  else launch_packed<1, 8, 8>(xb, wb, out, out_code == 2, M, N, K, stream);
+  SYN_LAUNCH_CHECK("gemm_packed");
   return 0;
 }

@@ -163,6 +163,44 @@ def gemm_swiglu(x, w_paired, out):
     _call(load_library("core"), "syn_gemm_swiglu", _ptr(x), _ptr(w_paired), _ptr(out), M, N, K, _stream())
 
 
+PACKED_MAX_ROWS = 8   # up to this many rows of x the products over packed weights are the faster ones
+
+
+def pack_weight(w):
+    """A copy of the bf16 weight w [N, K] in the order of the MFMA fragments that the products for few
+    rows take: [N / 16, K / 32, 64, 8] with lane = 16 * (k % 32 // 8) + n % 16 (every load of a wave is then
+    1 KB of consecutive bytes).  None if the shape or the type does not allow it (N a multiple of 16, K of 32)."""
+    if w.dtype != _BF16 or w.dim() != 2 or w.shape[0] % 16 or w.shape[1] % 32:
+        return None
+    N, K = w.shape
+    return w.view(N // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).reshape(N // 16, K // 32, 64, 8).contiguous()
+
+
+def unpack_weight(wp):
+    """The inverse of pack_weight: [N, K]."""
+    nt, nks = wp.shape[:2]
+    return wp.view(nt, nks, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(nt * 16, nks * 32).contiguous()
+
+
+def gemm_packed(x, wp, out, paired=False):
+    """out[M, N] (bf16 or float) = x[M, K] . W^T for M <= 16 with wp = pack_weight(W); paired: W holds gate and
+    up rows in turns of 16 (pair_rows) and out [M, N / 2] bf16 = silu(gate) * up."""
+    _need(x, "gemm_packed.x", _BF16, (None, None))
+    M, K = x.shape
+    if K % 32:
+        raise KernelError(f"gemm_packed: K = {K} is no multiple of 32")
+    _need(wp, "gemm_packed.wp", _BF16, (None, K // 32, 64, 8))
+    N = wp.shape[0] * 16
+    if M > 16 or (paired and N % 32):
+        raise KernelError(f"gemm_packed: M = {M} (at most 16), N = {N}")
+    if paired:
+        _need(out, "gemm_packed.out", _BF16, (M, N // 2))
+    else:
+        _need(out, "gemm_packed.out", (_BF16, _F32), (M, N))
+    _call(load_library("core"), "syn_gemm_packed", _ptr(x), _ptr(wp), _ptr(out), 2 if out.dtype == _F32 else 1,
+          M, N, K, 1 if paired else 0, _stream())
+
+
 def gemm_slices(M, N, K, dtype):
     """Into how many slices of K a product is cut when its reader can add partial sums.  A product
     with few rows of W has too few workgroups (one for every 64 rows) to pull the weights at speed.

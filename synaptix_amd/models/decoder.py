@@ -19,7 +19,7 @@ import torch
 
 from ..kernels import ops
 from ..parts.base import Part
-from ..parts.linear import linear
+from ..parts.linear import linear, packed_copy
 from ..weights.source import TensorSpec
 
 
@@ -54,7 +54,7 @@ class OutputHead(Part):
 
     def __init__(self, name: str, vocab: int, hidden: int, tied_to: TokenEmbedding | None = None):
         self.name, self.vocab, self.hidden, self.tied_to = name, vocab, hidden, tied_to
-        self.weight = None
+        self.weight = self.packed = None
 
     def tensor_specs(self):
         return {} if self.tied_to is not None else {self.name: TensorSpec((self.vocab, self.hidden))}
@@ -65,9 +65,10 @@ class OutputHead(Part):
 
     def load(self, get):
         self.weight = self.tied_to.table if self.tied_to is not None else get(self.name)
+        self.packed = packed_copy(self.weight)   # in fragment order, for single tokens
 
     def forward(self, h):
-        return linear(h, self.weight, torch.float32)
+        return linear(h, self.weight, torch.float32, self.packed)
 
 
 class DecoderModel:

@@ -10,7 +10,7 @@ import torch
 from ..kernels import ops
 from ..weights.source import TensorSpec
 from .base import Part
-from .linear import linear, linear_for_sum
+from .linear import linear, linear_for_sum, packed_copy
 
 
 class FeedForward(Part):
@@ -26,6 +26,7 @@ class GatedMlp(FeedForward):
             raise ValueError(f"activation {activation!r} is not built (silu only)")
         self.prefix, self.hidden, self.intermediate = prefix, hidden, intermediate
         self.w_gate_up = self.w_down = None
+        self.p_gate_up = self.p_down = None   # copies in fragment order for single tokens
         self.paired = False      # gate and up rows in turns of 16: the activation runs inside the product
 
     def tensor_specs(self):
@@ -43,11 +44,16 @@ class GatedMlp(FeedForward):
                        and self.intermediate % ops.PAIR == 0 and self.hidden % 8 == 0)
         self.w_gate_up = ops.pair_rows(gate, up) if self.paired else torch.cat([gate, up], 0)
         self.w_down = get(p + "down_proj.weight")
+        self.p_gate_up = packed_copy(self.w_gate_up) if self.paired and self.intermediate % 16 == 0 else None
+        self.p_down = packed_copy(self.w_down)
 
     def forward(self, h, ctx):
         m = torch.empty((h.shape[0], self.intermediate), dtype=h.dtype, device=h.device)
         if self.paired and h.dtype == torch.bfloat16:
-            ops.gemm_swiglu(h, self.w_gate_up, m)
+            if self.p_gate_up is not None and h.shape[0] <= ops.PACKED_MAX_ROWS:
+                ops.gemm_packed(h, self.p_gate_up, m, paired=True)
+            else:
+                ops.gemm_swiglu(h, self.w_gate_up, m)
         else:
             ops.swiglu(linear(h, self.w_gate_up, h.dtype), m)
-        return linear_for_sum(m, self.w_down)
+        return linear_for_sum(m, self.w_down, self.p_down)

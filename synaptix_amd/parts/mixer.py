@@ -15,7 +15,7 @@ import torch
 from ..kernels import ops
 from ..weights.source import TensorSpec
 from .base import Part, KvNeed
-from .linear import linear, linear_for_sum
+from .linear import linear, linear_for_sum, packed_copy
 from .position import Position, NoPosition
 
 
@@ -68,6 +68,7 @@ class GqaAttention(Mixer):
         # one product for q, k and v: rows of the three matrices one after another
         self.w_qkv = torch.cat([get(p + "q_proj.weight"), get(p + "k_proj.weight"), get(p + "v_proj.weight")], 0)
         self.w_o = get(p + "o_proj.weight")
+        self.p_qkv, self.p_o = packed_copy(self.w_qkv), packed_copy(self.w_o)   # in fragment order, for single tokens
         if self.qk_norm_eps is not None:
             self.q_gain = get(p + "q_norm.weight")
             self.k_gain = get(p + "k_norm.weight").to(self.q_gain.dtype)
@@ -89,8 +90,11 @@ class GqaAttention(Mixer):
         if cap is not None and ctx.max_position >= cap:
             raise ValueError(f"position {ctx.max_position} is beyond the position encoding's capacity {cap}")
         # single tokens: partial sums over slices of K, which the attention kernel adds; prompts: the plain product
-        qkv = linear_for_sum(h, self.w_qkv) if N <= 64 and ops.gemm_slices(N, self.w_qkv.shape[0], self.hidden, act) > 1 \
-            else linear(h, self.w_qkv, act)
+        if self.p_qkv is not None and N <= ops.PACKED_MAX_ROWS and act == torch.bfloat16:
+            qkv = linear(h, self.w_qkv, torch.float32, self.p_qkv).unsqueeze(0)   # one float "partial sum"
+        else:
+            qkv = linear_for_sum(h, self.w_qkv) if N <= 64 and ops.gemm_slices(N, self.w_qkv.shape[0], self.hidden, act) > 1 \
+                else linear(h, self.w_qkv, act)
         cos, sin = self.position.tables(h.device)
         table = ctx.page_table(cache.group)
         o = torch.empty((N, nh * hd), dtype=act, device=h.device)
@@ -102,7 +106,7 @@ class GqaAttention(Mixer):
             ops.attention_decode_fused_bf16(qkv, cache.k_pages, cache.v_pages, table, ctx.seq_len, o, work, splits,
                                             self.scale, window, nh, nkv, hd, self.q_gain, self.k_gain,
                                             self.qk_norm_eps or 0.0, cos, sin, write_kv=owner)
-            return linear_for_sum(o, self.w_o)
+            return linear_for_sum(o, self.w_o, self.p_o)
         q = torch.empty((N, nh * hd), dtype=act, device=h.device)
         ops.qk_norm_rope_kv_write(qkv, q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos,
                                   self.q_gain, self.k_gain, self.qk_norm_eps or 0.0, cos, sin, nh, nkv, hd,
@@ -118,4 +122,4 @@ class GqaAttention(Mixer):
         else:
             ops.attention_prefill_bf16(q, cache.k_pages, cache.v_pages, table, ctx.seq_start, ctx.seq_past, o,
                                        self.scale, window, nh, nkv, hd)
-        return linear_for_sum(o, self.w_o)
+        return linear_for_sum(o, self.w_o, self.p_o)

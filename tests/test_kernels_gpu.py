@@ -212,6 +212,39 @@ def test_gemm_with_the_gated_activation_inside(ops, M, I, K):
         ops.gemm_swiglu(x.to(DEV), paired[:48], torch.empty((M, 24), dtype=BF16, device=DEV))
 
 
+@pytest.mark.parametrize("out_dtype", [BF16, F32])
+@pytest.mark.parametrize("M,N,K", [(1, 16, 32), (1, 4096, 4096), (8, 6144, 4096), (3, 48, 96), (5, 1008, 1120), (8, 16400, 160),
+                                   (16, 64, 12288), (7, 80, 2080)])
+def test_gemm_over_weights_in_fragment_order(ops, out_dtype, M, N, K):
+    """The products for few rows over pack_weight(W): every k-step and every row tile lands where the
+    plain product has it, also where K is no multiple of the waves' turns and N of the workgroup's rows."""
+    x, w = rnd((M, K), 26, BF16), rnd((N, K), 27, BF16)
+    wp = ops.pack_weight(w.to(DEV))
+    assert wp.shape == (N // 16, K // 32, 64, 8)
+    assert torch.equal(ops.unpack_weight(wp).cpu(), w)
+    # lane = 16 * (k % 32 // 8) + n % 16, element k % 8
+    assert wp[N // 16 - 1, K // 32 - 1, 16 * 2 + 5, 3] == w[N - 16 + 5, K - 32 + 2 * 8 + 3]
+    out = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+    ops.gemm_packed(x.to(DEV), wp, out)
+    want = (x.double() @ w.double().T).float()
+    atol = 1e-3 * math.sqrt(K)
+    close(out, want, atol if out_dtype == F32 else atol + 0.02, 0 if out_dtype == F32 else 1e-2, f"packed {M}x{N}x{K}")
+    assert ops.pack_weight(w[:N - 3].to(DEV)) is None and ops.pack_weight(w[:, :K - 8].to(DEV)) is None
+    with pytest.raises(Exception, match="at most 16"):
+        ops.gemm_packed(torch.zeros((17, K), dtype=BF16, device=DEV), wp, torch.empty((17, N), dtype=out_dtype, device=DEV))
+
+
+@pytest.mark.parametrize("M,I,K", [(1, 16, 32), (1, 2560, 4096), (8, 2560, 4096), (7, 112, 992), (4, 16400, 64)])
+def test_gated_product_over_weights_in_fragment_order(ops, M, I, K):
+    x, wg, wu = rnd((M, K), 28, BF16), rnd((I, K), 29, BF16), rnd((I, K), 30, BF16)
+    wp = ops.pack_weight(ops.pair_rows(wg.to(DEV), wu.to(DEV)))
+    out = torch.full((M, I), float("nan"), dtype=BF16, device=DEV)
+    ops.gemm_packed(x.to(DEV), wp, out, paired=True)
+    g, u = x.double() @ wg.double().T, x.double() @ wu.double().T
+    want = (g / (1 + torch.exp(-g)) * u).float()
+    close(out, want, 2e-3 * K + 0.02, 1e-2, f"packed gated product {M}x{I}x{K}")
+
+
 def test_gemm_bf16_paths_agree(ops):
     """The MFMA kernels and the plain kernel compute the same sums."""
     for M in (4, 40, 300):
