@@ -10,11 +10,21 @@ import torch
 from ..kernels import ops
 
 
+_KEEP_PACKED_COPIES = True
+
+
+def keep_packed_copies(flag: bool) -> None:
+    """Whether models loaded from now on keep the second copy of their bf16 weights (packed_copy).
+    Without it single tokens read the plain matrices through the slower kernels."""
+    global _KEEP_PACKED_COPIES
+    _KEEP_PACKED_COPIES = bool(flag)
+
+
 def packed_copy(w):
     """What a part keeps beside a bf16 weight for single tokens: the same matrix in the order of the MFMA
     fragments (ops.pack_weight), or None.  It doubles the memory of the weight; a step of up to
     ops.PACKED_MAX_ROWS rows reads it instead of w."""
-    return ops.pack_weight(w) if w.dtype == torch.bfloat16 else None
+    return ops.pack_weight(w) if _KEEP_PACKED_COPIES and w.dtype == torch.bfloat16 else None
 
 
 def _use_packed(x, packed):

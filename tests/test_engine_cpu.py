@@ -100,3 +100,23 @@ def test_a_head_size_without_a_kernel_is_refused_when_the_engine_is_made(tmp_pat
     eng = cpu_kernels.CpuEngine.load(str(tmp_path), dtype="float32", max_tokens=128, device="cpu")
     s = eng.acquire()
     assert eng.step([(s, [1, 2, 3])], want="last").shape == (1, cfg.vocab_size)
+
+
+def test_single_tokens_give_the_same_logits_with_and_without_packed_weight_copies():
+    """The copy of the weights in fragment order is a layout, not another model."""
+    from synaptix_amd.parts import keep_packed_copies
+    from helpers import random_tokens
+    toks = random_tokens(CONFIGS["A"]["vocab_size"], 12, 77)
+    got = []
+    for keep in (True, False):
+        keep_packed_copies(keep)
+        try:
+            eng = make_engine("A", "bfloat16", 256)
+        finally:
+            keep_packed_copies(True)
+        has = eng.model.blocks[0].mixer.p_o is not None
+        assert has == keep
+        s = eng.acquire()
+        eng.step([(s, toks[:9])], want=None)
+        got.append(torch.cat([eng.step([(s, [t])], want="last") for t in toks[9:]]))
+    assert float((got[0] - got[1]).abs().max()) <= 2e-2
