@@ -348,7 +348,7 @@ SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, co
 //   partial[(seq * nh + head) * n_splits + split] = { m, l, o[HD] }   (float)
 // and a second kernel merges the splits.
 constexpr int PART = HD + 2;
-constexpr int DEC_MAX_WAVES = HD > 128 ? 4 : 8;  // as many as keep their ~190 registers each without spilling
+constexpr int DEC_MAX_WAVES = HD > 128 ? 4 : 8;  // as many as keep their registers (about 220 at 128) without spilling
 
 // The K and V fragments of one block of 64 keys, all requested before the first product needs one.
 struct KvBlock {

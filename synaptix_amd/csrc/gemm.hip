@@ -797,8 +797,8 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
     if (N <= 8192) launch_skinny<1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
     else launch_skinny<1, 8, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
   } else if (M <= 32) {
-    // few rows: memory-bound; small tiles (many workgroups), deep in K (long pieces of each row);
-    // straight into LDS where K allows it (the same speed at 8 rows, a quarter faster at 16 and 32)
+    // few rows: memory-bound; small tiles (many workgroups), deep in K (long pieces of each row), three
+    // k-tiles in flight, straight into LDS where K allows it
     if (N >= 65536 && K % 256 == 0) rc = launch_direct<32, 64, 256, 1, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
     else if (N >= 65536) rc = launch_tiled<32, 32, 256, 1, 1>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
     else if (K % 128 == 0) rc = launch_direct<32, 64, 128, 1, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
