@@ -345,12 +345,20 @@ def attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, seq_past,
 def decode_splits(n_seqs, n_kv_heads, max_pages):
     """How many ways the key blocks of a sequence are split in decode.  A workgroup has up to 8
     waves that take a block each at a time; a wave that takes several blocks one after another
-    pays a trip to memory for each, so the keys are split until about 2,048 waves run (measured
-    at 8 sequences of 2,100 tokens: 4 splits 22 us, 1 split 37 us, 16 splits 30 us), but not so
-    far that waves are left without a block.  One split needs no merge."""
+    pays a trip to memory for each, so the keys are split until about 2,048 waves run, but not so
+    far that a split holds fewer than four blocks.  Contexts from 6K tokens on are split further,
+    up to 1,024 workgroups, while a split keeps eight blocks.  One split needs no merge.
+    Measured inside a graph at 1 to 32 sequences of 512 to 32K tokens (32 heads, 8 kv heads of 128):
+    8 sequences of 2,100 tokens: 4 splits 19 us, 1 split 29 us, 8 splits 23 us; one sequence: 8
+    splits 10.7 us, 4 splits 12.8 us; 8 sequences of 8K tokens: 16 splits 54 us, 4 splits 60 us."""
     groups = max(1, n_seqs * n_kv_heads)
     want = -(-2048 // (groups * 8))
-    return int(max(1, min(want, -(-max_pages // 8), 64)))
+    splits = max(1, min(want, 1 if max_pages <= 8 else max_pages // 4, 64))
+    if max_pages >= 96:
+        more = min(64, 1024 // groups)
+        if more > splits and max_pages // more >= 8:
+            splits = more
+    return int(splits)
 
 
 def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
