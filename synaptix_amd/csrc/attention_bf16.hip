@@ -20,7 +20,7 @@
 // (as crates/synaptix-kernels-cuda/src/cu/fused/attention/flash_splitq.cu:187-600 does); the output
 // is rounded once.
 //
-//   prefill: a workgroup of 8 waves takes 128 query rows of one (sequence, head); a wave 16 of them.
+//   prefill: a workgroup takes 128 query rows of one (sequence, head); a wave 32 of them (16 for heads beyond 128).
 //   decode : a workgroup takes (sequence, kv head, up to 16 heads of its group, one split of the keys);
 //            the heads of a group share every K/V load and the waves share the split's blocks.
 //            A second kernel merges the splits when there is more than one.
@@ -105,16 +105,25 @@ __device__ __forceinline__ void attn_init(AttnState<QB>& st) {
 }
 
 // ------------------------------------------------------------------ prefill
-// A workgroup of 8 waves takes 128 query rows of one (sequence, head), a wave 16 of them; two waves
-// share a SIMD, so that one multiplies while the other waits for LDS or memory.  Blocks of 64 keys go through LDS, double-buffered: while the waves work on one block the
-// next one is on its way from memory into registers.  K lies in LDS as [64 keys, in tile order][HD + 8], V^T as
+// A workgroup takes 128 query rows of one (sequence, head); two or more waves share a SIMD, so that one
+// multiplies while the other waits for LDS or memory.  Blocks of 64 keys go through LDS,
+// double-buffered: while the waves work on one block the next one is on its way from memory into registers.  K lies in LDS as [64 keys, in tile order][HD + 8], V^T as
 // [HD][64 + 8]; the paddings keep the 16-lane fragment reads free of bank conflicts.
 // Softmax runs in the exp2 domain (scores times scale * log2 e); masking is applied only to blocks
 // that reach beyond a row's causal limit, the window's start or the sequence's end.
 // PV takes k-steps of 32 keys (see the key permutation above).
 constexpr float RESCALE_AT = 8.f;
-constexpr int PF_QB = 1;                        // 16-column blocks a wave
-constexpr int PF_WAVES = 8;
+// Up to a head size of 128 a wave takes 32 query rows (two 16-column blocks share every K and V fragment
+// read from LDS, which is what bounds this kernel) and four waves make a workgroup; the kernel is then
+// held to 256 registers so that two workgroups share a compute unit.  Larger heads would spill: they
+// keep 16 rows a wave and eight waves.
+constexpr int PF_QB = HD <= 128 ? 2 : 1;        // 16-column blocks a wave
+constexpr int PF_WAVES = HD <= 128 ? 4 : 8;
+#if SYN_HD <= 128
+#define PF_REGISTERS __attribute__((amdgpu_waves_per_eu(2)))
+#else
+#define PF_REGISTERS
+#endif
 constexpr int PF_THREADS = PF_WAVES * SYN_WAVE;
 constexpr int PF_ROWS = PF_WAVES * PF_QB * 16;  // query rows a workgroup
 constexpr int LDK = HD + 8;
@@ -122,7 +131,7 @@ constexpr int LDV = SYN_PAGE + 8;
 constexpr int PF_TILE = SYN_PAGE * LDK + HD * LDV;          // bf16 elements of one buffer
 constexpr int PF_CHUNKS = (8 * HD + PF_THREADS - 1) / PF_THREADS;  // 16-byte chunks a thread moves for K (and for V)
 
-__global__ void __launch_bounds__(PF_THREADS)
+__global__ void __launch_bounds__(PF_THREADS) PF_REGISTERS
 attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
                     const int* __restrict__ page_table, int table_stride, const int* __restrict__ seq_start,
                     const int* __restrict__ seq_past, int n_seqs, int n_tiles, bf16* __restrict__ out, float scale,
