@@ -113,17 +113,11 @@ __device__ __forceinline__ void attn_init(AttnState<QB>& st) {
 // that reach beyond a row's causal limit, the window's start or the sequence's end.
 // PV takes k-steps of 32 keys (see the key permutation above).
 constexpr float RESCALE_AT = 8.f;
-// Up to a head size of 128 a wave takes 32 query rows (two 16-column blocks share every K and V fragment
-// read from LDS, which is what bounds this kernel) and four waves make a workgroup; the kernel is then
-// held to 256 registers so that two workgroups share a compute unit.  Larger heads would spill: they
-// keep 16 rows a wave and eight waves.
-constexpr int PF_QB = HD <= 128 ? 2 : 1;        // 16-column blocks a wave
-constexpr int PF_WAVES = HD <= 128 ? 4 : 8;
-#if SYN_HD <= 128
-#define PF_REGISTERS __attribute__((amdgpu_waves_per_eu(2)))
-#else
-#define PF_REGISTERS
-#endif
+// A wave takes 16 query rows and eight waves make a workgroup: 126 registers at a head size of 128, so
+// that two workgroups share a compute unit.  (32 rows a wave would share every K and V fragment read
+// from LDS between two column blocks, but need 256 registers: measured slower, 89 against 74 us at 2,048 tokens.)
+constexpr int PF_QB = 1;      // 16-column blocks a wave
+constexpr int PF_WAVES = 8;
 constexpr int PF_THREADS = PF_WAVES * SYN_WAVE;
 constexpr int PF_ROWS = PF_WAVES * PF_QB * 16;  // query rows a workgroup
 constexpr int LDK = HD + 8;
@@ -131,15 +125,22 @@ constexpr int LDV = SYN_PAGE + 8;
 constexpr int PF_TILE = SYN_PAGE * LDK + HD * LDV;          // bf16 elements of one buffer
 constexpr int PF_CHUNKS = (8 * HD + PF_THREADS - 1) / PF_THREADS;  // 16-byte chunks a thread moves for K (and for V)
 
-__global__ void __launch_bounds__(PF_THREADS) PF_REGISTERS
+__global__ void __launch_bounds__(PF_THREADS)
 attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
                     const int* __restrict__ page_table, int table_stride, const int* __restrict__ seq_start,
-                    const int* __restrict__ seq_past, int n_seqs, int n_tiles, bf16* __restrict__ out, float scale,
+                    const int* __restrict__ seq_past, int n_seqs, bf16* __restrict__ out, float scale,
                     int window, int nh, int nkv) {
   extern __shared__ __attribute__((aligned(16))) bf16 lds[];  // [2][PF_TILE]
-  // which sequence and which rows: tiles are numbered sequence by sequence; the grid runs through
-  // them backwards so that the tiles with the most key blocks start first
-  const int tile = n_tiles - 1 - (int)blockIdx.x;
+  // which sequence and which rows: tiles are numbered sequence by sequence.  Heads run fastest through
+  // the grid; workgroups go round the eight dies in turn, and the heads are dealt so that each die gets
+  // neighbouring heads, which share their K and V.  Two workgroups share a compute unit, and a tile's
+  // work grows with its number: the first half of the grid takes the tiles from the last downwards,
+  // the second half from the first upwards, so that the pairs that meet on a unit have about equal work.
+  int total = 0;
+  for (int s = 0; s < n_seqs; ++s) total += (seq_start[s + 1] - seq_start[s] + PF_ROWS - 1) / PF_ROWS;
+  const int y = blockIdx.y, half = (total + 1) / 2;
+  if (y >= total) return;  // the grid is an upper bound
+  const int tile = y < half ? total - 1 - y : y - half;
   int seq = -1, q0 = 0, t_acc = 0;
   for (int s = 0; s < n_seqs; ++s) {
     const int nt = (seq_start[s + 1] - seq_start[s] + PF_ROWS - 1) / PF_ROWS;
@@ -150,10 +151,11 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages
     }
     t_acc += nt;
   }
-  if (seq < 0) return;  // the grid is an upper bound
+  if (seq < 0) return;
   const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE;
   const int r16 = lane % 16, g4 = lane / 16;
-  const int head = blockIdx.y, kvh = head / (nh / nkv);
+  const int hx = blockIdx.x;
+  const int head = nh % 8 == 0 ? (hx % 8) * (nh / 8) + hx / 8 : hx, kvh = head / (nh / nkv);
   const int tok0 = seq_start[seq], n_new = seq_start[seq + 1] - tok0, past = seq_past[seq];
   const int kv_len = past + n_new;
   const int r0 = q0 + wave * PF_QB * 16;
@@ -333,8 +335,8 @@ SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, co
   SYN_CHECK(hd == HD, "attention_prefill: library built for head size %d, called with %d", HD, hd);
   SYN_CHECK(n_seqs > 0 && n_tokens >= n_seqs && nh > 0 && nkv > 0, "attention_prefill: empty input");
   SYN_CHECK(nh % nkv == 0, "attention_prefill: %d heads do not divide into %d kv heads", nh, nkv);
-  SYN_CHECK(nh <= 65535, "attention_prefill: %d heads exceed the grid", nh);
   const int tiles = n_tokens / PF_ROWS + n_seqs;  // an upper bound; surplus workgroups leave at once
+  SYN_CHECK(tiles <= 65535, "attention_prefill: %d tiles of %d rows exceed the grid", tiles, PF_ROWS);
   const size_t lds = (size_t)2 * PF_TILE * sizeof(bf16);
   static bool raised = false;
   if (lds > 65536 && !raised) {
@@ -343,9 +345,9 @@ SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, co
     SYN_CHECK(e == hipSuccess, "attention_prefill: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
     raised = true;
   }
-  attn_prefill_kernel<<<dim3(tiles, nh), PF_THREADS, lds, stream>>>(
+  attn_prefill_kernel<<<dim3(nh, tiles), PF_THREADS, lds, stream>>>(
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, page_table, table_stride, seq_start, seq_past, n_seqs,
-      tiles, (bf16*)out, scale, window, nh, nkv);
+      (bf16*)out, scale, window, nh, nkv);
   SYN_LAUNCH_CHECK("attention_prefill");
   return 0;
 }
