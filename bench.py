@@ -44,6 +44,8 @@ def main() -> int:
                     help="fewer layers than the model has (same layer sizes); both numbers are reported")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
+    ap.add_argument("--no-packed-copies", action="store_true",
+                    help="keep no second copy of the weights in MFMA fragment order: steps of up to 64 rows read the plain matrices")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -53,6 +55,9 @@ def main() -> int:
     from synaptix_amd import Qwen3Config, Engine
     from synaptix_amd.kernels import ops
 
+    if args.no_packed_copies:
+        from synaptix_amd.parts import keep_packed_copies
+        keep_packed_copies(False)
     torch.manual_seed(0)
     cfg = Qwen3Config.from_dict({**QWEN3_8B, "num_hidden_layers": args.layers})
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
