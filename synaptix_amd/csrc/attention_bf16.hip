@@ -38,8 +38,6 @@ static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head sizes in steps of 16 
 constexpr bool TAIL16 = (HD % 32) != 0;
 constexpr int DT = HD / 16;
 
-SYN_EXPORT int syn_attention_head_dim() { return HD; }
-
 // Fragments of Q (or of a K row block) along the head dimension.  Head sizes that are a multiple of
 // 32 take k-steps of 32 (16x16x32); the others take k-steps of 16 throughout (16x16x16): one
 // accumulation chain never mixes the two shapes.
