@@ -42,11 +42,17 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=QWEN3_8B["num_hidden_layers"],
                     help="fewer layers than the model has (same layer sizes); both numbers are reported")
+    ap.add_argument("--prompt", type=int, default=PROMPT,
+                    help="tokens of every prompt (the contract's run has 2,048; the cache holds 8,192 a sequence)")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
     ap.add_argument("--no-packed-copies", action="store_true",
                     help="keep no second copy of the weights in MFMA fragment order: steps of up to 64 rows read the plain matrices")
     args = ap.parse_args()
+    prompt_len = args.prompt
+    if prompt_len < 1 or prompt_len + args.warmup + args.steps + 8 > 8192:
+        print(f"bench.py: --prompt {prompt_len} plus {args.warmup} + {args.steps} + 8 new tokens exceed the context of 8192")
+        return 2
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
@@ -62,12 +68,12 @@ def main() -> int:
     cfg = Qwen3Config.from_dict({**QWEN3_8B, "num_hidden_layers": args.layers})
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
     new_tokens = args.warmup + args.steps + 8
-    per_seq = (PROMPT + new_tokens + 63) // 64 * 64
+    per_seq = (prompt_len + new_tokens + 63) // 64 * 64
     eng = Engine.from_config(cfg, seed=0, dtype="bfloat16", max_tokens=max(batches) * per_seq + 64, max_seq=8192)
     g = torch.Generator().manual_seed(0)
 
     def prompt():
-        return torch.randint(0, cfg.vocab_size, (PROMPT,), generator=g).tolist()
+        return torch.randint(0, cfg.vocab_size, (prompt_len,), generator=g).tolist()
 
     L, H, I, V = cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
     nh, nkv, hd = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
@@ -87,8 +93,8 @@ def main() -> int:
         times.append(time.perf_counter() - t0)
         eng.release(s)
     pre_s = statistics.median(times[2:])
-    pre_flops = 2 * PROMPT * L * layer_params + L * 4 * hd * nh * PROMPT * (PROMPT + 1) // 2 + 2 * V * H
-    prefill = {"value": round(PROMPT / pre_s, 1), "tokens": PROMPT, "ms": round(pre_s * 1e3, 3),
+    pre_flops = 2 * prompt_len * L * layer_params + L * 4 * hd * nh * prompt_len * (prompt_len + 1) // 2 + 2 * V * H
+    prefill = {"value": round(prompt_len / pre_s, 1), "tokens": prompt_len, "ms": round(pre_s * 1e3, 3),
                "frac": round(pre_flops / pre_s / MFMA_PEAK["bf16"], 4)}
 
     # ---- decode
@@ -101,7 +107,7 @@ def main() -> int:
             if lo == 0:
                 tokens = []
             tokens += first
-        longest = PROMPT + warmup + steps + 8
+        longest = prompt_len + warmup + steps + 8
         if not args.no_graph:
             # the captured step is built before anything is timed (with a sequence of its own, one
             # token long; the other rows are padding), so that also a run without warm-up times steps only
@@ -156,7 +162,7 @@ def main() -> int:
         "dtype": "bf16", "data": "synthetic: seeded uniform token ids, random-init weights N(0, 0.02)",
         "config": {"model": "Qwen3-8B shape", "layers": L, "model_layers": QWEN3_8B["num_hidden_layers"],
                    "hidden": H, "heads": nh, "kv_heads": nkv, "head_dim": hd, "intermediate": I, "vocab": V,
-                   "global_batch": args.batch, "seq_len": PROMPT, "context": 8192, "new_tokens": args.steps,
+                   "global_batch": args.batch, "seq_len": prompt_len, "context": 8192, "new_tokens": args.steps,
                    "tie_word_embeddings": False, "rope_theta": 1e6, "rms_norm_eps": 1e-6, "parallelism": "single GPU",
                    "graph": not args.no_graph},
         "prefill": prefill,

@@ -729,15 +729,18 @@ template <bool PAIRED>
 static int launch_large(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
                         hipStream_t stream, int slices = 1);
 
-// Which of the large tiles for M > 64: 0 = 256 x 256, 1 = 256 x 192 (one workgroup a compute unit; about
-// 6 % less efficient), 2 = 128 x 128 (two workgroups a compute unit, about 20 % less efficient).
-// The estimate is the number of rounds over the 256 compute units times the work of a tile; it
-// reproduces what was measured at 2048 rows for N = 4096, 6144 and 24576 (a tie goes to the larger tile).
+// Which of the large tiles for M > 64: 0 = 256 x 256, 1 = 256 x 192 (one workgroup of four waves a compute
+// unit; a fifth less efficient), 2 = 128 x 128 (two workgroups a compute unit, about as much less efficient).
+// The estimate is the number of rounds over the 256 compute units times the work of a tile.  Measured
+// for N = 6144 and 24576 at 1,024 to 8,192 rows: the narrower tile wins where it fills a round that the
+// wide one leaves partly empty (q/k/v at 2,048 and 4,096 rows: 100 against 116 us, 181 against 198) and
+// loses over many rounds (gate+up at 3,072, 5,120 and 7,680 rows: 760 against 638 us, 989 against 900,
+// 1524 against 1349); its factor came out between 1.15 and 1.3.  A tie goes to the larger tile.
 static int pick_large_tile(int M, int N) {
   auto rounds = [](long tiles, long slots) { return (tiles + slots - 1) / slots; };
   auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
   const double cost[3] = {(double)rounds(tiles(256, 256), 256) * 256 * 256,
-                          (double)rounds(tiles(256, 192), 256) * 256 * 192 * 1.06,
+                          (double)rounds(tiles(256, 192), 256) * 256 * 192 * 1.2,
                           (double)rounds(tiles(128, 128), 512) * 2 * 128 * 128 * 1.2};
   int best = 0;
   if (cost[1] < cost[best]) best = 1;
