@@ -270,31 +270,51 @@ static int tile_grid(int M, int N, int BM, int BN) {
 
 // The accumulators of a wave (TM x TN tiles of MFMA 32x32: D[m = 8*(e/4) + 4*(lane/32) + e%4][n = lane%32])
 // to memory.  mw, nw: the first row and column of the wave's part.  PAIRED: columns n % 32 < 16 are
-// gate rows, the 16 after them the up rows of the same outputs (N is a multiple of 32 then): a lane of
-// the first kind gets its partner's value and stores silu(gate) * up, half as wide.
+// gate rows, the 16 after them the up rows of the same outputs (N is a multiple of 32 then, so a tile of
+// 32 columns lies inside or outside as a whole).  Two tiles side by side are stored together: the lanes
+// of the first kind take the first tile (their own gate, the partner's up), the others the second (the
+// partner's gate, their own up), so that a store covers 32 consecutive outputs of a row (64 bytes, not
+// twice 32).  A last tile without a neighbour is stored by the lanes of the first kind alone.
 template <int TM, int TN, bool PAIRED>
 __device__ __forceinline__ void store_tiles(const f32x16 (&acc)[TM][TN], void* __restrict__ out, int out_is_f32,
                                             size_t slice, int M, int N, int mw, int nw, int lane) {
+  if constexpr (PAIRED) {
+    const bool first = lane % 32 < 16;
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+      for (int j = 0; j < TN; j += 2)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int m = mw + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
-        const int n = nw + j * 32 + lane % 32;
-        if constexpr (PAIRED) {
-          const float up = __shfl_xor(acc[i][j][e], 16, SYN_WAVE);
-          const float g = acc[i][j][e];
-          if (m < M && n < N && lane % 32 < 16)
-            ((bf16*)out)[(size_t)m * (N / 2) + (nw + j * 32) / 2 + lane % 16] = (bf16)(g / (1.f + expf(-g)) * up);
-        } else if (m < M && n < N) {
-          if (out_is_f32)
-            ((float*)out)[(slice * M + m) * N + n] = acc[i][j][e];
-          else
-            ((bf16*)out)[(size_t)m * N + n] = (bf16)acc[i][j][e];
+        for (int e = 0; e < 16; ++e) {
+          const int m = mw + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+          const float own0 = acc[i][j][e], other0 = __shfl_xor(own0, 16, SYN_WAVE);
+          if (j + 1 < TN) {   // known once the loop is unrolled
+            const float own1 = acc[i][j + 1 < TN ? j + 1 : j][e], other1 = __shfl_xor(own1, 16, SYN_WAVE);
+            const float g = first ? own0 : other1, up = first ? other0 : own1;
+            if (m < M && nw + (j + (first ? 0 : 1)) * 32 < N)
+              ((bf16*)out)[(size_t)m * (N / 2) + (nw + j * 32) / 2 + lane % 32] = (bf16)(g / (1.f + expf(-g)) * up);
+          } else {
+            if (m < M && nw + j * 32 < N && first)
+              ((bf16*)out)[(size_t)m * (N / 2) + (nw + j * 32) / 2 + lane % 16] = (bf16)(own0 / (1.f + expf(-own0)) * other0);
+          }
         }
-      }
+  } else {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int m = mw + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
+          const int n = nw + j * 32 + lane % 32;
+          if (m < M && n < N) {
+            if (out_is_f32)
+              ((float*)out)[(slice * M + m) * N + n] = acc[i][j][e];
+            else
+              ((bf16*)out)[(size_t)m * N + n] = (bf16)acc[i][j][e];
+          }
+        }
+  }
 }
 
 // ------------------------------------------------------------------ tiled, bf16
