@@ -110,9 +110,12 @@ __device__ __forceinline__ BufferView buffer_view(const void* base, size_t bytes
 #endif
   return v;
 }
-// 16 bytes a lane from base + lane_bytes + uniform_bytes to lds + 16 * lane (lds is the same for all lanes)
+// 16 bytes a lane from base + lane_bytes + uniform_bytes to lds + 16 * lane (lds is the same for all lanes).
+// STREAMED: the load is marked non-temporal, for data that is read once (a decode step's keys).
+template <bool STREAMED = false>
 __device__ __forceinline__ void buffer_to_lds16(const BufferView& v, void* lds, unsigned lane_bytes, int uniform_bytes) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(v.r, (__attribute__((address_space(3))) void*)lds, 16, lane_bytes, uniform_bytes, 0, 0);
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(v.r, (__attribute__((address_space(3))) void*)lds, 16, lane_bytes, uniform_bytes, 0,
+                                           STREAMED ? 2 : 0);
 #endif
 }
