@@ -488,7 +488,7 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
   // (its LDS slot gets zeros, and its results are never stored), which with few rows of x spares
   // most of the requests for x.
   // pass p: the wave fills tile rows (p * WAVES + wave) * RPI .. + RPI (x rows first, then W rows)
-  static_assert(BM % RPI == 0, "a load lies in x or in W as a whole");
+  static_assert(BM % (RPI * WAVES) == 0, "a pass lies in x or in W as a whole, for all waves alike");
   const size_t row_bytes = (size_t)K * sizeof(bf16);
   const BufferView vx = buffer_view(x + (size_t)m0 * K, (size_t)(M - m0) * row_bytes);
   const BufferView vw = buffer_view(w + (size_t)n0 * K, (size_t)(N - n0) * row_bytes);
@@ -504,7 +504,12 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
       bf16* dst = smem + (size_t)buf * ROWS * BK + (size_t)(p * WAVES + wave) * RPI * BK;  // the same for all lanes
-      buffer_to_lds16((p * WAVES + wave) * RPI < BM ? vx : vw, dst, src[p], (k_begin + kt * BK) * (int)sizeof(bf16));
+      // every wave fills rows of x in the first passes and rows of W in the others; up to 64 rows of x a
+      // workgroup is the only reader of its rows of W: their loads are marked non-temporal
+      if (p * WAVES * RPI < BM)
+        buffer_to_lds16(vx, dst, src[p], (k_begin + kt * BK) * (int)sizeof(bf16));
+      else
+        buffer_to_lds16<true>(vw, dst, src[p], (k_begin + kt * BK) * (int)sizeof(bf16));
     }
   };
   // Tile kt lies in buffer kt % STAGES; while it is multiplied the STAGES - 1 tiles after it are on their
