@@ -71,3 +71,31 @@ def test_smoke_entry():
     sys.path.insert(0, ROOT)
     import __graft_entry__
     __graft_entry__.smoke()
+
+
+def test_bench_line_keeps_its_contract():
+    """bench.py with one layer of the named shape and a few steps: one JSON line with the agreed keys;
+    more than one GPU, or a prompt beyond the context, is refused with exit code 2 and one line."""
+    cmd = [sys.executable, f"{ROOT}/bench.py"]
+    proc = subprocess.run(cmd + ["--layers", "1", "--steps", "3", "--warmup", "1", "--batch", "2", "--no-points",
+                                 "--prompt", "256"], capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = [l for l in proc.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    rec = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "prefill", "roofline", "points"):
+        assert key in rec, key
+    assert rec["n_gpus"] == 1 and rec["steps"] == 3 and rec["warmup"] == 1 and rec["dtype"] == "bf16"
+    cfg = rec["config"]
+    assert len(cfg) <= 20 and all(not isinstance(v, (dict, list)) for v in cfg.values())
+    assert cfg["layers"] == 1 and cfg["model_layers"] == 36 and cfg["global_batch"] == 2 and cfg["seq_len"] == 256
+    assert set(rec["prefill"]) == {"value", "tokens", "ms", "frac"} and rec["prefill"]["tokens"] == 256
+    roof = rec["roofline"]
+    assert roof["bound"] == "hbm" and roof["unit"] == "GB/s" and roof["peak"] == 8000.0
+    assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
+    assert rec["value"] > 0 and abs(rec["value"] - 2 / (rec["ms_per_step"] * 1e-3)) < 0.01 * rec["value"]
+    for extra in (["--gpus", "2"], ["--prompt", "9000"]):
+        proc = subprocess.run(cmd + extra, capture_output=True, text=True, timeout=120)
+        assert proc.returncode == 2
+        assert len([l for l in proc.stdout.splitlines() if l.strip()]) == 1
