@@ -504,8 +504,8 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
       bf16* dst = smem + (size_t)buf * ROWS * BK + (size_t)(p * WAVES + wave) * RPI * BK;  // the same for all lanes
-      // every wave fills rows of x in the first passes and rows of W in the others; up to 64 rows of x a
-      // workgroup is the only reader of its rows of W: their loads are marked non-temporal
+      // every wave fills rows of x in the first passes and rows of W in the others; this kernel runs where a
+      // row of W has one reader (up to 64 rows of x) or at most four: its loads are marked non-temporal
       if (p * WAVES * RPI < BM)
         buffer_to_lds16(vx, dst, src[p], (k_begin + kt * BK) * (int)sizeof(bf16));
       else
@@ -819,6 +819,13 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   const bf16* xb = (const bf16*)x;
   const bf16* wb = (const bf16*)w;
   // From sweeps at the shapes of an 8B model (N = 4096 .. 151936, K = 4096 and 12288).
+  // Short prompts (65 to 256 rows) of a narrow product: even the smallest of the large tiles would leave
+  // most compute units without work (q/k/v at 128 rows: 48 tiles of 128 x 128), and the product is still
+  // bound by reading W: the 64 x 64 tiles take it (q/k/v at 128 rows 57 -> 31 us, o_proj in two slices
+  // 52 -> 18, down_proj in four 74 -> 34; at 256 rows 59 -> 36, 57 -> 22, 79 -> 62; from 384 rows on and
+  // for the output head the large tiles win).
+  const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+  const bool few_large_tiles = M > 64 && M <= 256 && K % 128 == 0 && tiles128 * slices <= 256;
   int rc = 0;
   if (M == 1 && slices == 1) {
     // one row: fragments of W straight from memory, K split over the waves
@@ -831,7 +838,7 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
     else if (N >= 65536) rc = launch_tiled<32, 32, 256, 1, 1>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
     else if (K % 128 == 0) rc = launch_direct<32, 64, 128, 1, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
     else rc = launch_tiled<32, 64, 128, 1, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
-  } else if (M <= 64) {
+  } else if (M <= 64 || few_large_tiles) {
     if (K % 128 == 0) rc = launch_direct<64, 64, 128, 2, 2, false, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
     else rc = launch_tiled<64, 64, 128, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
   } else {

@@ -145,6 +145,7 @@ def test_gemm_f32(ops, M, N, K):
     (8, 40000, 256), (40, 33000, 72), (64, 50000, 1000),   # wide
     (1, 9000, 520), (1, 70000, 136),                       # one row: W straight from memory, K over the waves
     (8, 70000, 264), (20, 66000, 72),                      # few rows, very wide: 32-row tiles, 256 deep
+    (100, 300, 1024), (256, 520, 256), (129, 4096, 384), (255, 6144, 128),   # short prompts, narrow: 64-row tiles, several of them along M
 ])
 def test_gemm_bf16(ops, out_dtype, M, N, K):
     x, w = rnd((M, K), 10, BF16), rnd((N, K), 11, BF16)
@@ -158,7 +159,8 @@ def test_gemm_bf16(ops, out_dtype, M, N, K):
 
 @pytest.mark.parametrize("M,N,K,S", [(1, 48, 4096, 4), (8, 4096, 4096, 4), (8, 100, 1000, 3), (16, 64, 12288, 8),
                                      (40, 70, 2048, 2), (64, 130, 520, 5), (8, 96, 1536, 5), (50, 200, 3072, 7),
-                                     (300, 520, 1024, 2), (130, 260, 640, 3), (65, 33, 4096, 4)])
+                                     (300, 520, 1024, 2), (130, 260, 640, 3), (65, 33, 4096, 4),
+                                     (200, 4096, 1024, 2), (256, 1000, 2048, 4)])
 def test_gemm_bf16_partial_sums_over_slices_of_k(ops, M, N, K, S):
     """[S, M, N]: slice s holds the sum over its part of K; the slices add up to the product, also
     when K is no multiple of the slice and the last slices are short or empty."""
