@@ -819,13 +819,13 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   const bf16* xb = (const bf16*)x;
   const bf16* wb = (const bf16*)w;
   // From sweeps at the shapes of an 8B model (N = 4096 .. 151936, K = 4096 and 12288).
-  // Short prompts (65 to 256 rows) of a narrow product: even the smallest of the large tiles would leave
+  // Short prompts (65 to 512 rows) of a narrow product: even the smallest of the large tiles would leave
   // most compute units without work (q/k/v at 128 rows: 48 tiles of 128 x 128), and the product is still
   // bound by reading W: the 64 x 64 tiles take it (q/k/v at 128 rows 57 -> 31 us, o_proj in two slices
-  // 52 -> 18, down_proj in four 74 -> 34; at 256 rows 59 -> 36, 57 -> 22, 79 -> 62; from 384 rows on and
-  // for the output head the large tiles win).
+  // 52 -> 18, down_proj in four 74 -> 34; at 256 rows 59 -> 36, 57 -> 22, 79 -> 62; at 512 rows o_proj
+  // 58 -> 39 and q/k/v 63 -> 67; down_proj from 384 rows on and the output head stay on the large tiles).
   const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-  const bool few_large_tiles = M > 64 && M <= 256 && K % 128 == 0 && tiles128 * slices <= 256;
+  const bool few_large_tiles = M > 64 && M <= 512 && K % 128 == 0 && tiles128 * slices <= 256;
   int rc = 0;
   if (M == 1 && slices == 1) {
     // one row: fragments of W straight from memory, K split over the waves
