@@ -93,8 +93,9 @@ class GqaAttention(Mixer):
         if self.p_qkv is not None and N <= ops.PACKED_MAX_ROWS and act == torch.bfloat16:
             qkv = linear(h, self.w_qkv, torch.float32, self.p_qkv).unsqueeze(0)   # one float "partial sum"
         else:
-            qkv = linear_for_sum(h, self.w_qkv) if N <= 64 and ops.gemm_slices(N, self.w_qkv.shape[0], self.hidden, act) > 1 \
-                else linear(h, self.w_qkv, act)
+            # (the kernels behind single tokens, and behind prompts of up to 64 tokens, add partial sums themselves)
+            sliced = (N <= 64 or ctx.one_token_each) and ops.gemm_slices(N, self.w_qkv.shape[0], self.hidden, act) > 1
+            qkv = linear_for_sum(h, self.w_qkv) if sliced else linear(h, self.w_qkv, act)
         cos, sin = self.position.tables(h.device)
         table = ctx.page_table(cache.group)
         o = torch.empty((N, nh * hd), dtype=act, device=h.device)
