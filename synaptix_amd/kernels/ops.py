@@ -6,7 +6,9 @@ these names: without the built library, or with tensors that are not on the GPU,
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
+import threading
 
 import torch
 
@@ -21,8 +23,26 @@ class KernelError(RuntimeError):
     pass
 
 
+_scope = threading.local()
+
+
 def _stream():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    held = getattr(_scope, "stream", None)
+    return held if held is not None else ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+@contextlib.contextmanager
+def stream_scope():
+    """Within the scope every kernel of this thread is launched on the stream that is current when the scope
+    is entered, asked for once (a model's forward pass launches some 300 kernels and never changes the
+    stream; asking torch each time costs more than the launch).  Scopes nest; code that switches streams
+    inside one opens a new one."""
+    before = getattr(_scope, "stream", None)
+    _scope.stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    try:
+        yield
+    finally:
+        _scope.stream = before
 
 
 def _ptr(t):
@@ -30,19 +50,27 @@ def _ptr(t):
 
 
 def _need(t, name, dtypes, shape=None):
+    # the checks in the order of their cost; the messages are built only when one fails
     if not isinstance(t, torch.Tensor):
         raise KernelError(f"{name}: expected a tensor, got {type(t).__name__}")
-    if t.device.type != "cuda":
+    dt = t.dtype
+    if dt is not dtypes and (dtypes.__class__ is torch.dtype or dt not in dtypes):
+        want = dtypes if isinstance(dtypes, (tuple, list)) else (dtypes,)
+        raise KernelError(f"{name}: dtype {dt}, expected {' or '.join(str(d) for d in want)}")
+    if not t.is_cuda:
         raise KernelError(f"{name}: tensor lies on {t.device}; the kernels of synaptix_amd run on the GPU only")
-    if not isinstance(dtypes, (tuple, list)):
-        dtypes = (dtypes,)
-    if t.dtype not in dtypes:
-        raise KernelError(f"{name}: dtype {t.dtype}, expected {' or '.join(str(d) for d in dtypes)}")
     if not t.is_contiguous():
         raise KernelError(f"{name}: tensor is not contiguous")
     if shape is not None:
-        if len(shape) != t.dim() or any(s is not None and s != g for s, g in zip(shape, t.shape)):
-            raise KernelError(f"{name}: shape {list(t.shape)}, expected {[('*' if s is None else s) for s in shape]}")
+        got = t.shape
+        ok = len(shape) == len(got)
+        if ok:
+            for s, g in zip(shape, got):
+                if s is not None and s != g:
+                    ok = False
+                    break
+        if not ok:
+            raise KernelError(f"{name}: shape {list(got)}, expected {[('*' if s is None else s) for s in shape]}")
 
 
 def _call(lib, fn, *args):

@@ -133,11 +133,12 @@ class DecoderModel:
     # ------------------------------------------------------------------ one step
     def forward(self, ctx, tokens, want_rows, cache) -> torch.Tensor:
         """tokens [N] int32 and want_rows [n] int32 (or None) on the device; returns logits [n, vocab] float."""
-        resid = self.embedding.forward(tokens)
-        pending = None
-        for run, owner in zip(self.schedule, self._owner):
-            pending = self.blocks[run.block].forward(resid, pending, ctx, cache.layer_view(run.cache), owner)
-        if want_rows is None:
-            return None          # nothing is asked for: the cache has been written, that is all
-        h = self.final_norm.add_apply(resid, pending, ctx.act_dtype, rows=want_rows)
-        return self.head.forward(h)
+        with ops.stream_scope():     # one stream for the whole pass, asked for once
+            resid = self.embedding.forward(tokens)
+            pending = None
+            for run, owner in zip(self.schedule, self._owner):
+                pending = self.blocks[run.block].forward(resid, pending, ctx, cache.layer_view(run.cache), owner)
+            if want_rows is None:
+                return None          # nothing is asked for: the cache has been written, that is all
+            h = self.final_norm.add_apply(resid, pending, ctx.act_dtype, rows=want_rows)
+            return self.head.forward(h)

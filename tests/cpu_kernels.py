@@ -79,6 +79,11 @@ def gemm_packed(x, wp, out, paired=False):
         out.copy_((x.to(F32) @ w.to(F32).T).to(out.dtype))
 
 
+def stream_scope():
+    import contextlib
+    return contextlib.nullcontext()
+
+
 def gemm_slices(M, N, K, dtype):
     return 2 if (dtype == torch.bfloat16 and M <= 16 and K >= 64 and K % 8 == 0) else 1
 
@@ -193,7 +198,7 @@ def sample_rows(logits, temperature, uniform, out):
         out[r] = int(hit[0]) if hit.numel() else x.numel() - 1
 
 
-ALL = ["embed", "add_rmsnorm", "rmsnorm_rows", "swiglu", "gemm", "gemm_swiglu", "gemm_packed", "gemm_slices", "qk_norm_rope_kv_write", "attention_f32",
+ALL = ["embed", "add_rmsnorm", "rmsnorm_rows", "swiglu", "gemm", "gemm_swiglu", "gemm_packed", "stream_scope", "gemm_slices", "qk_norm_rope_kv_write", "attention_f32",
        "attention_prefill_bf16", "decode_splits", "attention_decode_bf16", "attention_decode_fused_bf16", "sample_rows"]
 
 
