@@ -194,6 +194,28 @@ def test_trace_run_steps_without_wants_write_no_file(tmp_path):
     assert not os.path.exists(tmp_path / "o" / "0.f32")
 
 
+def test_trace_run_names_the_step_it_cannot_run(tmp_path):
+    """A step that does not fit the cache, or brings a token outside the vocabulary: the steps before it are
+    done, then one line names the step and the reason, exit code 1."""
+    import json
+    import subprocess
+    import sys
+    from helpers import ROOT
+    folder = model_folder("A")
+    for bad, reason in (([1] * 65, "CacheFull"), ([1, 10 ** 6], "vocabulary")):
+        steps = [{"step": 0, "entries": [{"id": "x", "tokens": [1, 2, 3], "want": [2]}], "end": ["x"]},
+                 {"step": 1, "entries": [{"id": "y", "tokens": bad, "want": [0]}], "end": []}]
+        cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+               "--out", str(tmp_path / "o"), "--max-tokens", "64"]
+        proc = subprocess.run(cmd, input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True,
+                              timeout=300)
+        assert proc.returncode == 1
+        assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == ["done 0"]
+        last = [l for l in proc.stderr.splitlines() if l.startswith("trace_run:")]
+        assert len(last) == 1 and "step 1" in last[0] and reason in last[0], proc.stderr[-500:]
+        assert "Traceback" not in proc.stderr
+
+
 # ----------------------------------------------------------------------------- captured decode steps
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_graph_replays_equal_eager_steps(dtype):
