@@ -133,7 +133,11 @@ def main(argv=None) -> int:
     m.add_argument("--dtype", default="bf16", choices=["bf16", "f32"])
     m.set_defaults(fn=cmd_random)
     a = ap.parse_args(argv)
-    return a.fn(a)
+    try:
+        return a.fn(a)
+    except (ValueError, RuntimeError, OSError) as e:     # configuration, weights, cache, kernels, files
+        print(f"synaptix_amd {a.cmd}: {type(e).__name__}: {e}", file=sys.stderr)
+        return 1
 
 
 if __name__ == "__main__":
