@@ -382,8 +382,8 @@ def decode_splits(n_seqs, n_kv_heads, max_pages):
     groups = max(1, n_seqs * n_kv_heads)
     want = -(-2048 // (groups * 8))
     splits = max(1, min(want, 1 if max_pages <= 8 else max_pages // 4, 64))
-    if max_pages >= 96:
-        more = min(64, 1024 // groups)
+    if max_pages >= 96 and groups * splits < 256:    # (with a workgroup for every compute unit more splits only cost merging:
+        more = min(64, 1024 // groups)               # 32 sequences of 8K tokens unsplit 160 us, in 4 splits 166 us)
         if more > splits and max_pages // more >= 8:
             splits = more
     return int(splits)
