@@ -382,7 +382,7 @@ def decode_splits(n_seqs, n_kv_heads, max_pages):
     groups = max(1, n_seqs * n_kv_heads)
     want = -(-2048 // (groups * 8))
     splits = max(1, min(want, 1 if max_pages <= 8 else max_pages // 4, 64))
-    if max_pages >= 96 and groups * splits < 256:    # (with a workgroup for every compute unit more splits only cost merging:
+    if max_pages >= 96 and groups < 256:             # (with a workgroup for every compute unit more splits only cost merging:
         more = min(64, 1024 // groups)               # 32 sequences of 8K tokens unsplit 160 us, in 4 splits 166 us)
         if more > splits and max_pages // more >= 8:
             splits = more
