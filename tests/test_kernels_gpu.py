@@ -601,3 +601,29 @@ def test_measured_ceilings_are_plausible(ops):
     read_gbs, mfma_tflops = ops.measure_ceilings(DEV, read_bytes=1 << 28, repeats=2)
     assert 500 < read_gbs < 8000 * 1.05, read_gbs          # below the HBM peak, far above PCIe
     assert 100 < mfma_tflops < 2500 * 1.05, mfma_tflops    # below the bf16 peak
+
+
+def test_stream_scope_holds_the_stream_that_is_current_when_it_opens(ops):
+    """Inside a scope kernels go to the stream that was current at its start; a scope opened under another
+    stream takes that one; leaving restores what was held before."""
+    def held():
+        return ops._stream().value or 0      # the default stream is the null handle
+
+    main = torch.cuda.current_stream().cuda_stream
+    side = torch.cuda.Stream()
+    assert held() == main
+    with ops.stream_scope():
+        assert held() == main
+        with torch.cuda.stream(side):
+            assert held() == main          # the scope's stream, not torch's current one
+            with ops.stream_scope():
+                assert held() == side.cuda_stream
+                x, gain = rnd((3, 64), 50).to(DEV), torch.ones(64, device=DEV)
+                out = torch.empty((3, 64), device=DEV)
+                ops.rmsnorm_rows(x, gain, 1e-6, out)    # launched on the side stream
+            assert held() == main
+        side.synchronize()
+        want = torch.empty((3, 64))
+        ref.rmsnorm_rows(x.cpu(), gain.cpu(), 1e-6, want)
+        close(out, want, 1e-5, what="launched under a nested scope")
+    assert held() == main

@@ -85,3 +85,25 @@ def test_decode_tables_pad_with_a_spare_page():
     with pytest.raises(CacheError, match="rows"):
         rt.check(rt.lib().syn_decode_fill(c._h, 1, 2, rt.ints([a, b]), rt.ints([9, 8]), 2, rt.ints(widths),
                                           rt.ints(spare), None, None, host.ctypes.data))
+
+
+def test_host_side_rules_of_the_kernels_stay_within_their_kernels_limits():
+    """The numbers of splits and slices that the host picks: pure functions, checked over a grid of sizes."""
+    import torch
+    from synaptix_amd.kernels import ops
+    for n_seqs in (1, 2, 3, 8, 17, 64, 300):
+        for n_kv in (1, 2, 8):
+            for pages in (1, 2, 8, 9, 33, 96, 128, 512, 4096):
+                s = ops.decode_splits(n_seqs, n_kv, pages)
+                assert 1 <= s <= 64 and s <= pages
+                assert s == 1 or pages // s >= 4          # a split keeps at least four blocks
+    assert ops.decode_splits(64, 8, 33) == 1 and ops.decode_splits(1, 8, 33) > 1
+    for M in (1, 8, 9, 32, 33, 64, 65, 128, 512, 2048, 8192):
+        for N, K in ((4096, 4096), (6144, 4096), (4096, 12288), (151936, 4096), (64, 64), (4096, 1000)):
+            s = ops.gemm_slices(M, N, K, torch.bfloat16)
+            assert 1 <= s <= 8
+            if s > 1:
+                step = ((K + s - 1) // s + 127) // 128 * 128
+                assert (s - 1) * step < K, "no slice may be empty"
+                assert K % 8 == 0 and (M <= 64 or K % 128 == 0)
+            assert ops.gemm_slices(M, N, K, torch.float32) == 1
