@@ -11,7 +11,7 @@ import plain_qwen3 as P
 
 
 def lengths_for(name):
-    # the batches of BASELINE's tiny configurations, plus lengths around a page's edge
+    # the batches named for the two tiny configurations (5/17/11 and 1/33/7/64 tokens), plus lengths around a page's edge
     return {"A": [5, 17, 11, 64, 65], "B": [1, 33, 7, 64, 130], "C": [3, 70, 129, 40, 200],
             "E": [2, 66, 9, 130, 31], "F": [4, 65, 20]}[name]
 
@@ -190,7 +190,7 @@ def check_greedy_path(plain, prompt, got, want, margin=2e-2):
 
 
 def sampled_generation(make_engine, name, dtype):
-    """Temperature sampling with per-sequence streams: BASELINE's tiny B case (T = 0.7, seed 1).
+    """Temperature sampling with per-sequence streams: the tiny configuration B at temperature 0.7 and seed 1.
     In float32 the tokens are the plain implementation's.  In bfloat16 a draw may fall on the other
     side of a CDF boundary; then the uniform number must lie at that boundary within the
     probabilities' rounding error, and everything before it must agree."""
