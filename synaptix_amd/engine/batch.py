@@ -40,6 +40,25 @@ class StepLayout:
         self.table_off = [(offsets[len(_NAMES) + g], n_seqs * w) for g, w in enumerate(self.widths)]
 
 
+class ScratchPool:
+    """Named float scratch tensors that grow on demand.  A tensor that grows is replaced and the old
+    one goes back to the allocator, so a pool belongs to one user: the engine's eager steps share
+    one, every captured decode step has its own and freezes it before the capture (a graph holds
+    the addresses it was captured with; growth after that would be a use of freed memory)."""
+
+    def __init__(self, device):
+        self.device, self.tensors, self.frozen = device, {}, False
+
+    def get(self, name: str, numel: int) -> torch.Tensor:
+        t = self.tensors.get(name)
+        if t is None or t.numel() < numel:
+            if self.frozen:
+                raise RuntimeError(f"scratch {name!r} of a captured step would have to grow to {numel} floats")
+            t = torch.empty(max(numel, 1), dtype=torch.float32, device=self.device)
+            self.tensors[name] = t
+        return t
+
+
 class StepContext:
     """What parts see of a step.  Device arrays are views into one buffer."""
 
@@ -62,12 +81,8 @@ class StepContext:
         return ops.decode_splits(self.n_seqs, n_kv_heads, self.layout.widths[group])
 
     def scratch(self, name: str, numel: int) -> torch.Tensor:
-        """Float scratch memory that lives as long as the engine; contents are undefined."""
-        t = self._scratch.get(name)
-        if t is None or t.numel() < numel:
-            t = torch.empty(max(numel, 1), dtype=torch.float32, device=self.device)
-            self._scratch[name] = t
-        return t
+        """Float scratch memory that lives as long as its pool's owner; contents are undefined."""
+        return self._scratch.get(name, numel)
 
 
 def fill_host_buffer(layout: StepLayout, host: np.ndarray, cache, slots, tokens_flat: np.ndarray, counts,

@@ -18,7 +18,7 @@ from ..cache import SequenceCache, CacheError, PAGE_TOKENS, pages_for
 from ..config.registry import load_config, resolve_architecture
 from ..kernels import ops
 from ..weights import FolderSource, RandomSource, load_weights
-from .batch import StepLayout, StepContext, fill_host_buffer
+from .batch import StepLayout, StepContext, ScratchPool, fill_host_buffer
 
 assert ops.PAGE_TOKENS == PAGE_TOKENS
 
@@ -53,7 +53,7 @@ class Engine:
         self.max_positions = max_positions
         self.cache = SequenceCache(model.cache_needs(), max_tokens, max_slots, self.dtype, self.device,
                                    max_positions=max_positions)
-        self._scratch = {}
+        self._scratch = ScratchPool(self.device)      # of the eager steps; captured steps have their own
         self._host = None
         self._dev = None
         self._runners = {}

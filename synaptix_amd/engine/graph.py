@@ -22,7 +22,7 @@ import torch
 
 from ..kernels import ops
 from ..kernels import runtime as rt
-from .batch import StepLayout, StepContext
+from .batch import StepLayout, StepContext, ScratchPool
 
 
 def bucket_for(n: int) -> int:
@@ -52,6 +52,10 @@ class DecodeRunner:
         self.logits = None
         self.graph = None
         self.spare = [g.spare_page for g in engine.cache.groups]
+        # scratch memory of this runner's own: the captured graph holds its addresses, so no later
+        # step or larger runner may ever replace these tensors (row count, table widths and with them
+        # the number of splits are fixed here, so the first pass sizes them for good)
+        self.scratch = ScratchPool(dev)
 
     def _fill(self, host: np.ndarray, slots, tokens, temps, uniforms):
         """The padded tables of the step and, behind them, temperatures and uniform numbers."""
@@ -88,7 +92,7 @@ class DecodeRunner:
         self.copied[i].record()
         if self.graph is None:
             ctx = StepContext(self.layout, self.dev, eng.dtype, [-1] * self.rows, [0] * self.rows, [1] * self.rows,
-                              eng._scratch)
+                              self.scratch)
             ctx.max_position = eng.max_positions - 1 if eng.max_positions else 0   # checked on the host each step
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
@@ -97,6 +101,7 @@ class DecodeRunner:
                     self._forward(ctx)
             torch.cuda.current_stream().wait_stream(side)
             torch.cuda.synchronize()
+            self.scratch.frozen = True
             self.graph = torch.cuda.CUDAGraph()
             with torch.no_grad(), torch.cuda.graph(self.graph):
                 self.logits = self._forward(ctx)

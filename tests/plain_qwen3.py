@@ -133,6 +133,7 @@ class PlainQwen3:
         self.tied = bool(cfg.get("tie_word_embeddings", True))
         self.scale = 1.0 / math.sqrt(self.hd)
         self._tables = None
+        self.table_dtype = F32        # the reference builds its angles in float32 (tests of invariants widen it)
 
     @classmethod
     def from_folder(cls, folder: str, dtype=F32) -> "PlainQwen3":
@@ -146,11 +147,11 @@ class PlainQwen3:
     def tables(self, n_pos: int):
         if self._tables is None or self._tables[0].shape[0] < n_pos:
             # angles in float32 as the reference builds them, then widened if asked
-            cos, sin = rope_tables(self.hd, n_pos, self.theta, F32)
+            cos, sin = rope_tables(self.hd, n_pos, self.theta, self.table_dtype)
             self._tables = (cos.to(self.dtype), sin.to(self.dtype))
         return self._tables
 
-    def attention_block(self, l: int, xn: torch.Tensor, positions) -> torch.Tensor:
+    def attention_block(self, l: int, xn: torch.Tensor, positions, rope_offset: int = 0) -> torch.Tensor:
         """q/k/v projections, per-head q/k norm, rotation, attention, output projection.
 
         crates/synaptix-models/llm/common/src/model.rs:1715-1734 (projections, head split,
@@ -163,30 +164,32 @@ class PlainQwen3:
         v = (xn @ self.w[p + "v_proj.weight"].T).view(S, self.nkv, self.hd)
         q = rms_norm(q, self.w[p + "q_norm.weight"], self.eps)
         k = rms_norm(k, self.w[p + "k_norm.weight"], self.eps)
-        cos, sin = self.tables(int(max(positions)) + 1)
-        q = apply_rope(q, cos, sin, positions)
-        k = apply_rope(k, cos, sin, positions)
+        turned = [p + rope_offset for p in positions]    # rope_offset: every position moved by as much (for invariants)
+        cos, sin = self.tables(int(max(turned)) + 1)
+        q = apply_rope(q, cos, sin, turned)
+        k = apply_rope(k, cos, sin, turned)
         o = attention(q, k, v, self.scale, positions)
         return o.reshape(S, self.nh * self.hd) @ self.w[p + "o_proj.weight"].T
 
-    def hidden(self, ids) -> torch.Tensor:
+    def hidden(self, ids, rope_offset: int = 0) -> torch.Tensor:
         """Residual stream after the last block.  model.rs:1179-1199 (pre-norm wiring)."""
         x = embed(self.w["model.embed_tokens.weight"], ids)
         positions = list(range(len(ids)))
         for l in range(self.L):
             p = f"model.layers.{l}."
-            x = x + self.attention_block(l, rms_norm(x, self.w[p + "input_layernorm.weight"], self.eps), positions)
+            x = x + self.attention_block(l, rms_norm(x, self.w[p + "input_layernorm.weight"], self.eps), positions,
+                                         rope_offset)
             hn = rms_norm(x, self.w[p + "post_attention_layernorm.weight"], self.eps)
             x = x + swiglu_mlp(hn, self.w[p + "mlp.gate_proj.weight"], self.w[p + "mlp.up_proj.weight"],
                                self.w[p + "mlp.down_proj.weight"])
         return x
 
-    def forward(self, ids) -> torch.Tensor:
+    def forward(self, ids, rope_offset: int = 0) -> torch.Tensor:
         """Logits [S, V] at every position of one sequence.
 
         model.rs:1068-1089 (final norm, lm_head; tied -> the embedding matrix, 757-764).
         """
-        h = rms_norm(self.hidden(ids), self.w["model.norm.weight"], self.eps)
+        h = rms_norm(self.hidden(ids, rope_offset), self.w["model.norm.weight"], self.eps)
         w_out = self.w["model.embed_tokens.weight"] if self.tied else self.w["lm_head.weight"]
         return h @ w_out.T
 

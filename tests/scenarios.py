@@ -143,6 +143,114 @@ def long_context(make_engine, dtype, n_prompt=6000, n_decode=4):
     eng.release(s)
 
 
+def decode_beside_fresh_prompt(make_engine, name, dtype, sharp=False):
+    """One step that holds a sequence in its decode phase (tokens cached, one new token) and a
+    prompt that starts; then both decode; then a chunk of several tokens beside a single token."""
+    V = CONFIGS[name]["vocab_size"]
+    old, new = random_tokens(V, 70 + 5, 31), random_tokens(V, 45 + 2, 32)
+    want_old, want_new = plain_logits(name, old, sharp), plain_logits(name, new, sharp)
+    eng = make_engine(name, dtype, 1024, sharp)
+    a, b = eng.acquire(), eng.acquire()
+    got_old = [eng.step([(a, old[:70])], want="all")]
+    lg = eng.step([(a, old[70:71]), (b, new[:45])], want="all")      # decode beside a fresh prompt
+    got_old.append(lg[:1])
+    got_new = [lg[1:]]
+    lg = eng.step([(b, new[45:46]), (a, old[71:72])], want="last")   # both decode, order swapped
+    got_new.append(lg[:1])
+    got_old.append(lg[1:])
+    lg = eng.step([(a, old[72:75]), (b, new[46:47])], want="all")    # a chunk of three beside one token
+    got_old.append(lg[:3])
+    got_new.append(lg[3:])
+    assert_logits_close(torch.cat(got_old), want_old, dtype, f"{name} {dtype} the sequence that was decoding", sharp)
+    assert_logits_close(torch.cat(got_new), want_new, dtype, f"{name} {dtype} the prompt that joined", sharp)
+    eng.release(a)
+    eng.release(b)
+    eng.cache.check()
+
+
+def chunked_prompts(make_engine, name, dtype, chunk, sharp=False):
+    """Prompts fed in chunks of `chunk` tokens, all unfinished prompts in each step (what the
+    generation loop does with prefill_batch): a chunk starts inside a page and may cross pages."""
+    reqs = requests_for(name)
+    eng = make_engine(name, dtype, 1024, sharp)
+    slots = {r: eng.acquire() for r in reqs}
+    fed = {r: 0 for r in reqs}
+    got = {r: [] for r in reqs}
+    while True:
+        batch = [r for r in reqs if fed[r] < len(reqs[r])]
+        if not batch:
+            break
+        lg = eng.step([(slots[r], reqs[r][fed[r]:fed[r] + chunk]) for r in batch], want="all")
+        off = 0
+        for r in batch:
+            n = min(chunk, len(reqs[r]) - fed[r])
+            got[r].append(lg[off:off + n])
+            off += n
+            fed[r] += n
+    for r in reqs:
+        assert_logits_close(torch.cat(got[r]), plain_logits(name, reqs[r], sharp), dtype,
+                            f"{name} {dtype} {r} in chunks of {chunk}", sharp)
+        eng.release(slots[r])
+    eng.cache.check()
+
+
+def generation_with_chunked_prompt(make_engine, name, dtype, n_prompt=200, prefill_batch=64, n_new=6):
+    """The generation loop feeding a prompt in chunks of prefill_batch tokens."""
+    V = CONFIGS[name]["vocab_size"]
+    prompts = [random_tokens(V, n_prompt, 41), random_tokens(V, 70, 42)]
+    plain = plain_model(name)
+    eng = make_engine(name, dtype, 1024, False)
+    outs, _ = generate(eng, prompts, GenerationConfig(max_new_tokens=n_new, prefill_batch=prefill_batch))
+    for p, o in zip(prompts, outs):
+        want = P.generate(plain, p, n_new)
+        if dtype == "float32":
+            assert o.tokens == want
+        else:
+            check_greedy_path(plain, p, o.tokens, want)
+    eng.cache.check()
+
+
+def long_context_through_graphs(make_engine, dtype, n_prompt=6300, n_decode=3):
+    """More than 96 pages a sequence, decoded through captured steps whose page tables are 128
+    and 256 pages wide: with one row the keys are cut into 32 and 64 splits, with 32 rows into
+    16 (the rule for long contexts); a short sequence beside the long one leaves most of its
+    splits empty."""
+    from synaptix_amd.kernels import ops
+    name = "L"
+    V = CONFIGS[name]["vocab_size"]
+    nkv = CONFIGS[name]["num_key_value_heads"]
+    assert ops.decode_splits(1, nkv, 128) == 32 and ops.decode_splits(1, nkv, 256) == 64
+    assert ops.decode_splits(32, nkv, 128) == 16        # the branch for contexts of 96 pages and more
+    long_toks = random_tokens(V, n_prompt + 3 * n_decode, 9)
+    short_toks = random_tokens(V, 20 + 3 * n_decode, 10)
+    want_long, want_short = plain_logits(name, long_toks), plain_logits(name, short_toks)
+    eng = make_engine(name, dtype, n_prompt + 256, False)
+    if not eng.graph_ok:
+        return
+    a, b = eng.acquire(), eng.acquire()
+    eng.step([(a, long_toks[:n_prompt]), (b, short_toks[:20])], want=None)
+    got_long, got_short = [], []
+    at = 0
+    for rows, cap in ((1, 8192), (1, 16384), (32, 8192)):
+        runner = eng.decode_runner(rows, cap)
+        assert runner.widths[0] == (128 if cap == 8192 else 256) and runner.rows == rows
+        for _ in range(n_decode):
+            if rows == 1:                                   # one row: the long sequence alone, the short one eagerly
+                _, lg = runner.step([a], [long_toks[n_prompt + at]])
+                got_long.append(lg[:1].clone())
+                got_short.append(eng.step([(b, [short_toks[20 + at]])], want="last"))
+            else:
+                _, lg = runner.step([b, a], [short_toks[20 + at], long_toks[n_prompt + at]])
+                got_short.append(lg[:1].clone())
+                got_long.append(lg[1:2].clone())
+            at += 1
+    assert_logits_close(torch.cat(got_long), want_long[n_prompt:], dtype, f"{dtype} long sequence through wide graphs")
+    assert_logits_close(torch.cat(got_short), want_short[20:], dtype, f"{dtype} short sequence beside it")
+    eng.release(a)
+    eng.release(b)
+    eng.cache.check()
+
+
 def first_tokens(make_engine, name, dtype):
     """Prompts of one and two tokens; the very first position; a chunk that starts at position 1."""
     V = CONFIGS[name]["vocab_size"]

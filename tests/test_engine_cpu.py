@@ -42,6 +42,12 @@ def test_first_tokens():
     scenarios.first_tokens(make_engine, "B", "float32")
 
 
+def test_decode_beside_a_fresh_prompt_and_prompts_in_chunks():
+    scenarios.decode_beside_fresh_prompt(make_engine, "B", "float32")
+    scenarios.chunked_prompts(make_engine, "C", "float32", 50, sharp=True)
+    scenarios.generation_with_chunked_prompt(make_engine, "A", "float32", n_prompt=150, prefill_batch=64, n_new=3)
+
+
 def test_greedy_and_sampled_generation():
     scenarios.greedy_generation(make_engine, "A", "float32", n_new=5)
     scenarios.sampled_generation(make_engine, "B", "float32")

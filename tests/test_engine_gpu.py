@@ -89,6 +89,28 @@ def test_long_context(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_long_context_through_graphs_of_128_and_256_pages(dtype):
+    scenarios.long_context_through_graphs(make_engine, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,sharp", [("B", False), ("C", True)])
+def test_decode_beside_a_fresh_prompt(name, sharp, dtype):
+    scenarios.decode_beside_fresh_prompt(make_engine, name, dtype, sharp)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("chunk", [2, 50, 64])
+def test_prompts_in_chunks(chunk, dtype):
+    scenarios.chunked_prompts(make_engine, "C", dtype, chunk, sharp=(chunk == 50))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_generation_with_a_prompt_in_chunks_of_64(dtype):
+    scenarios.generation_with_chunked_prompt(make_engine, "B", dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_first_tokens(name, dtype):
     scenarios.first_tokens(make_engine, name, dtype)
@@ -172,8 +194,6 @@ def test_trace_run_whole_one_by_one_and_batched(tmp_path, dtype):
     batches = [["q3", "q0", "q1"], ["q2", "q4", "q1"], ["q4", "q3"]]
     steps, where = batched_trace(reqs, batches, decode=32)
     out = run_trace(folder, dtype, steps, 64 * 6, str(tmp_path / "batched"))
-    for batch in batches:
-        pass
     seen = set()
     for (r, p), (st, row) in where.items():
         seen.add(r)
@@ -250,6 +270,42 @@ def test_graph_replays_equal_eager_steps(dtype):
     assert float((got - want).abs().max()) <= (1e-5 if dtype == "float32" else 2e-2)
     for e in (eager, graph):
         e.cache.check()
+
+
+def test_a_captured_step_keeps_its_own_scratch_memory():
+    """A graph holds the addresses of the scratch memory it was captured with.  Larger steps
+    afterwards (eager ones and larger captured ones) need more of it; the small runner's must stay
+    where it is, and its replays must still give the eager results."""
+    name, dtype = "C", "bfloat16"
+    V = CONFIGS[name]["vocab_size"]
+    eng = make_engine(name, dtype, 64 * 80)
+    eager = make_engine(name, dtype, 1024)
+    prompt = random_tokens(V, 300, 77)
+    s, e = eng.acquire(), eager.acquire()
+    tok = eng.sample(eng.step([(s, prompt)], want="last")).cpu().tolist()
+    eager.step([(e, prompt)], want="last")
+    small = eng.decode_runner(1, 1024)              # 16 pages wide: the keys are cut into 4 splits, merged from scratch memory
+    tok2, _ = small.step([s], tok)
+    want = eager.step([(e, tok)], want="last")
+    before = {k: t.data_ptr() for k, t in small.scratch.tensors.items()}
+    assert before and small.scratch.frozen
+    # larger steps: 40 sequences decoding eagerly, then through a graph of 64 rows
+    many = [eng.acquire() for _ in range(40)]
+    eng.step([(m, random_tokens(V, 70, 80 + i)) for i, m in enumerate(many)], want=None)
+    eng.step([(m, [1]) for m in many], want="last")
+    big = eng.decode_runner(40, 1024)
+    big.step(many, [2] * 40)
+    held = [torch.empty(1 << 20, device="cuda") for _ in range(8)]     # whoever allocates next gets freed blocks
+    for h in held:
+        h.fill_(float("nan"))
+    assert {k: t.data_ptr() for k, t in small.scratch.tensors.items()} == before
+    assert all(small.scratch.tensors[k] is not big.scratch.tensors.get(k) for k in before)
+    assert all(small.scratch.tensors[k] is not eng._scratch.tensors.get(k) for k in before)
+    _, got = small.step([s], tok2)
+    want = eager.step([(e, tok2)], want="last")
+    torch.cuda.synchronize()
+    assert float((got - want).abs().max()) <= 2e-2
+    eng.cache.check()
 
 
 def test_generation_with_and_without_graph_agree():

@@ -48,9 +48,10 @@ def test_pipeline_generate(dtype):
 
 
 def test_command_line_run_and_bench():
-    name = "A"
-    folder = model_folder(name)
-    plain = plain_model(name)
+    # an untied model with peaked attention: the greedy path depends on far keys, not on the last token alone
+    name = "B"
+    folder = model_folder(name, sharp=True)
+    plain = plain_model(name, sharp=True)
     prompt = random_tokens(CONFIGS[name]["vocab_size"], 12, 10)
     want = P.generate(plain, prompt, 7)
     cmd = [sys.executable, "-m", "synaptix_amd", "run", folder, "--prompt-ids", ",".join(map(str, prompt)),
@@ -95,7 +96,23 @@ def test_bench_line_keeps_its_contract():
     assert roof["bound"] == "hbm" and roof["unit"] == "GB/s" and roof["peak"] == 8000.0
     assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
     assert rec["value"] > 0 and abs(rec["value"] - 2 / (rec["ms_per_step"] * 1e-3)) < 0.01 * rec["value"]
-    for extra in (["--gpus", "2"], ["--prompt", "9000"]):
+    # the other shapes: the same keys, the shape's own sizes
+    proc = subprocess.run(cmd + ["--shape", "4b", "--layers", "1", "--steps", "3", "--warmup", "1"], capture_output=True,
+                          text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    rec4 = json.loads([l for l in proc.stdout.splitlines() if l.strip()][-1])
+    assert set(rec4) >= set(rec) - {"measured"}
+    c4 = rec4["config"]
+    assert len(c4) <= 20 and all(not isinstance(v, (dict, list)) for v in c4.values())
+    assert (c4["hidden"], c4["intermediate"], c4["heads"], c4["tie_word_embeddings"]) == (2560, 9728, 32, True)
+    assert c4["global_batch"] == 16 and c4["new_tokens"] == 4 and 64 <= c4["min_prompt"] <= c4["max_prompt"] <= 4096
+    assert abs(rec4["value"] - 16 / (rec4["ms_per_step"] * 1e-3)) < 0.01 * rec4["value"]
+    proc = subprocess.run(cmd + ["--shape", "32b", "--layers", "1", "--steps", "3", "--warmup", "1", "--batch", "2",
+                                 "--no-points", "--prompt", "128"], capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    c32 = json.loads([l for l in proc.stdout.splitlines() if l.strip()][-1])["config"]
+    assert (c32["hidden"], c32["intermediate"], c32["heads"], c32["model_layers"]) == (5120, 25600, 64, 64)
+    for extra in (["--gpus", "2"], ["--prompt", "9000"], ["--shape", "4b", "--gpus", "4"]):
         proc = subprocess.run(cmd + extra, capture_output=True, text=True, timeout=120)
         assert proc.returncode == 2
         assert len([l for l in proc.stdout.splitlines() if l.strip()]) == 1

@@ -247,6 +247,50 @@ def test_gated_product_over_weights_in_fragment_order(ops, M, I, K):
     close(out, want, 2e-3 * K + 0.02, 1e-2, f"packed gated product {M}x{I}x{K}")
 
 
+def _sampled(M, N, n, seed):
+    g = torch.Generator().manual_seed(seed)
+    rows = torch.cat([torch.tensor([0, M - 1, 0, M - 1]), torch.randint(0, M, (n,), generator=g)])
+    cols = torch.cat([torch.tensor([0, 0, N - 1, N - 1]), torch.randint(0, N, (n,), generator=g)])
+    return rows, cols
+
+
+def test_products_of_a_prompt_at_the_sizes_of_an_8b_layer(ops):
+    """The large-tile products at full size: 2,048 rows through gate+up with the activation inside
+    (24,576 paired rows, K = 4096), and through down_proj (N = 4096, K = 12288) in the two slices
+    of K that the engine asks for; some hundred sampled outputs, the corners among them, against
+    64-bit dot products."""
+    M, H, I = 2048, 4096, 12288
+    x = rnd((M, H), 70, BF16)
+    wg, wu = rnd((I, H), 71, BF16, 0.02), rnd((I, H), 72, BF16, 0.02)
+    out = torch.full((M, I), float("nan"), dtype=BF16, device=DEV)
+    ops.gemm_swiglu(x.to(DEV), ops.pair_rows(wg.to(DEV), wu.to(DEV)), out)
+    rows, cols = _sampled(M, I, 400, 73)
+    g = (x[rows].double() * wg[cols].double()).sum(1)
+    u = (x[rows].double() * wu[cols].double()).sum(1)
+    want = (g / (1 + torch.exp(-g)) * u).float()
+    assert torch.isfinite(out).all()
+    close(out[rows.to(DEV), cols.to(DEV)], want, 0.02, 1e-2, "gate+up at 8B sizes")
+    del wg, wu
+    assert ops.gemm_slices(M, H, I, BF16) == 2
+    m = rnd((M, I), 74, BF16)
+    wd = rnd((H, I), 75, BF16, 0.02)
+    parts = torch.full((2, M, H), float("nan"), dtype=F32, device=DEV)
+    ops.gemm(m.to(DEV), wd.to(DEV), parts)
+    rows, cols = _sampled(M, H, 400, 76)
+    want = (m[rows].double() * wd[cols].double()).sum(1).float()
+    assert torch.isfinite(parts).all()
+    close(parts.sum(0)[rows.to(DEV), cols.to(DEV)], want, 2e-3, 1e-4, "down_proj at 8B sizes, two slices")
+    first = (m[rows, :I // 2].double() * wd[cols, :I // 2].double()).sum(1).float()
+    close(parts[0][rows.to(DEV), cols.to(DEV)], first, 2e-3, 1e-4, "its first slice")
+    # and the plain large product, bf16 out (q/k/v of a prompt: N = 6144)
+    wq = rnd((6144, H), 77, BF16, 0.02)
+    q = torch.full((M, 6144), float("nan"), dtype=BF16, device=DEV)
+    ops.gemm(x.to(DEV), wq.to(DEV), q)
+    rows, cols = _sampled(M, 6144, 400, 78)
+    want = (x[rows].double() * wq[cols].double()).sum(1).float()
+    close(q[rows.to(DEV), cols.to(DEV)], want, 0.02, 1e-2, "q/k/v at 8B sizes")
+
+
 def test_gemm_bf16_paths_agree(ops):
     """The MFMA kernels and the plain kernel compute the same sums."""
     for M in (4, 40, 300):
@@ -366,6 +410,9 @@ ATTN_SHAPES = [
     (4, 4, 128, [0, 40], [33, 1], 0),
     (4, 2, 96, [0, 5], [150, 100], 37),          # a window that ends inside pages
     (5, 5, 16, [200], [1], 64),
+    (8, 2, 64, [100, 64, 127], [70, 64, 2], 0),   # chunks of a prompt that start inside a page, at its edge, before its end
+    (32, 8, 128, [100, 1000], [150, 130], 0),     # the same at the head size and group of the large models
+    (6, 2, 48, [33], [300], 50),                  # a chunk over several pages with a window
 ]
 
 
@@ -406,6 +453,9 @@ def test_attention_prefill(ops, dtype, nh, nkv, hd, past, new, window):
     (5, 1, 80, [100, 300], 0, 2),
     (4, 4, 112, [70], 0, 1),
     (8, 2, 256, [130, 700], 0, 4),
+    (32, 8, 128, [7000, 40], 0, 32),            # long contexts: 32 and 64 splits, most of them empty for the short sequence
+    (8, 2, 64, [6500, 130, 7000], 0, 64),
+    (4, 1, 32, [4100], 0, 24),
 ])
 def test_attention_decode_bf16(ops, nh, nkv, hd, lens, window, splits):
     B = len(lens)
@@ -435,6 +485,8 @@ def test_attention_decode_bf16(ops, nh, nkv, hd, lens, window, splits):
     (4, 1, 64, 64, False, [500, 2], 100, 2, 0, True),                # no q/k norm, a window
     (40, 2, 32, 0, True, [90, 300], 0, 2, 2, True),                  # no rotation, 20 heads a group (two chunks)
     (8, 4, 128, 128, True, [257, 1000], 0, 8, 4, False),             # reads a cache that another layer wrote
+    (32, 8, 128, 128, True, [7000, 33], 0, 32, 4, True),             # long contexts: 32 and 64 splits
+    (4, 1, 64, 64, True, [6500, 100, 6401], 0, 64, 0, True),
 ])
 def test_attention_decode_with_qkv_intake(ops, nh, nkv, hd, rot, norm, lens, window, splits, parts, own):
     """Decode attention that makes q, k and v from the fused projection itself equals the q/k kernel

@@ -31,13 +31,13 @@ def tol(dtype):
 def one_sequence_ctx(cache, slot, n_new, dtype):
     """A StepContext for one sequence that brings n_new tokens, as the engine builds it."""
     import numpy as np
-    from synaptix_amd.engine.batch import StepLayout, StepContext, fill_host_buffer
+    from synaptix_amd.engine.batch import StepLayout, StepContext, ScratchPool, fill_host_buffer
     past = cache.length(slot)
     cache.reserve(slot, n_new)
     layout = StepLayout(n_new, 1, 0, [cache.table_width(g, [slot]) for g in range(len(cache.groups))])
     host = np.zeros(layout.total, dtype=np.int32)
     fill_host_buffer(layout, host, cache, [slot], np.zeros(n_new, dtype=np.int32), [n_new], [])
-    return StepContext(layout, torch.from_numpy(host).to(DEV), dtype, [slot], [past], [n_new], {})
+    return StepContext(layout, torch.from_numpy(host).to(DEV), dtype, [slot], [past], [n_new], ScratchPool(DEV))
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])

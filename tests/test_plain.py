@@ -167,16 +167,109 @@ def test_causality_and_prefix(name):
     assert torch.allclose(m.forward(other)[:7], full[:7], atol=1e-5)
 
 
-def test_qk_norm_uses_the_layers_eps_and_sits_before_the_rotation():
-    """Config B has eps 1e-5 and q_norm != k_norm; swapping the two gains, or taking another eps
-    with tiny activations, changes the logits."""
+class NormAfterRotation(P.PlainQwen3):
+    """The mistake that the invariant below is there to catch: q and k rotated first, normed after."""
+
+    def attention_block(self, l, xn, positions, rope_offset=0):
+        p = f"model.layers.{l}.self_attn."
+        S = xn.shape[0]
+        q = (xn @ self.w[p + "q_proj.weight"].T).view(S, self.nh, self.hd)
+        k = (xn @ self.w[p + "k_proj.weight"].T).view(S, self.nkv, self.hd)
+        v = (xn @ self.w[p + "v_proj.weight"].T).view(S, self.nkv, self.hd)
+        turned = [t + rope_offset for t in positions]
+        cos, sin = self.tables(max(turned) + 1)
+        q = P.rms_norm(P.apply_rope(q, cos, sin, turned), self.w[p + "q_norm.weight"], self.eps)
+        k = P.rms_norm(P.apply_rope(k, cos, sin, turned), self.w[p + "k_norm.weight"], self.eps)
+        o = P.attention(q, k, v, self.scale, positions)
+        return o.reshape(S, self.nh * self.hd) @ self.w[p + "o_proj.weight"].T
+
+
+def _uneven_gains(m):
+    """Weights of `m` whose q/k gains differ between the two halves of a head (the partners of a rotation)."""
+    w = dict(m.w)
+    hd = m.hd
+    for l in range(m.L):
+        for n, lo, hi in (("q_norm", 0.5, 2.0), ("k_norm", 1.5, 0.7)):
+            g = torch.cat([torch.full((hd // 2,), lo), torch.full((hd - hd // 2,), hi)])
+            w[f"model.layers.{l}.self_attn.{n}.weight"] = g * (1 + 0.05 * rnd((hd,), 40 + l))
+    return w
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_logits_depend_on_distances_only_which_puts_the_qk_norm_before_the_rotation(name):
+    """Moving every position by the same amount changes no logit: the rotation is the last thing
+    that happens to q and k (crates/synaptix-models/llm/common/src/model.rs:1715-1734).  A gain
+    applied after the rotation scales the two partners of a rotated pair differently, and the
+    score of (m, n) is then no function of m - n: the variant that norms after rotating fails
+    the same check, so the check can tell the two orders apart."""
+    m = plain_model(name)
+    w = _uneven_gains(m)
+    ids = random_tokens(m.cfg["vocab_size"], 9, 4)
+    good = P.PlainQwen3(m.cfg, w, dtype=F64)
+    good.table_dtype = F64                      # exact angles: what is left is the invariant itself
+    base = good.forward(ids)
+    for shift in (1, 37, 200):
+        assert (good.forward(ids, rope_offset=shift) - base).abs().max() < 1e-9
+    bad = NormAfterRotation(m.cfg, w, dtype=F64)
+    bad.table_dtype = F64
+    assert (bad.forward(ids, rope_offset=37) - bad.forward(ids)).abs().max() > 1e-4
+    assert (bad.forward(ids) - base).abs().max() > 1e-4
+
+
+def test_qk_norm_takes_the_layers_eps_and_its_own_gains(monkeypatch):
+    """crates/synaptix-models/llm/qwen3/src/config.rs:89-125: one eps for every norm of the model.
+    Config B has eps 1e-5; with activations so small that eps decides the norm's result, another
+    eps for q and k alone changes the logits; every call of the norm gets the configured value;
+    q_norm and k_norm are two tensors, not one."""
     m = plain_model("B")
     ids = random_tokens(1000, 5, 4)
+    seen = []
+    real = P.rms_norm
+
+    def spy(x, w, eps):
+        seen.append((x.shape[-1], eps))
+        return real(x, w, eps)
+
+    monkeypatch.setattr(P, "rms_norm", spy)
     base = m.forward(ids)
+    assert {e for _, e in seen} == {1e-5} and any(d == m.hd for d, _ in seen) and any(d == 128 for d, _ in seen)
+    # tiny q and k: mean square ~ 1e-10, so the result is x / sqrt(eps) and eps shows in full
     w = dict(m.w)
-    a, b = "model.layers.0.self_attn.q_norm.weight", "model.layers.0.self_attn.k_norm.weight"
-    w[a], w[b] = m.w[b], m.w[a]
+    for l in range(m.L):
+        for n in ("q_proj", "k_proj"):
+            w[f"model.layers.{l}.self_attn.{n}.weight"] = m.w[f"model.layers.{l}.self_attn.{n}.weight"] * 1e-4
+    tiny = P.PlainQwen3(m.cfg, w)
+
+    def other_eps_for_heads(x, w_, eps):
+        return real(x, w_, 1e-6 if x.shape[-1] == m.hd else eps)
+
+    a = tiny.forward(ids)
+    monkeypatch.setattr(P, "rms_norm", other_eps_for_heads)
+    b = tiny.forward(ids)
+    monkeypatch.setattr(P, "rms_norm", real)
+    assert (a - b).abs().max() > 1e-6
+    w = dict(m.w)
+    qn, kn = "model.layers.0.self_attn.q_norm.weight", "model.layers.0.self_attn.k_norm.weight"
+    w[qn], w[kn] = m.w[kn], m.w[qn]
     assert (P.PlainQwen3(m.cfg, w).forward(ids) - base).abs().max() > 1e-5
+
+
+def test_swiglu_vector_of_the_reference():
+    """crates/synaptix-ops/tests/ffn.rs:24-55: x = [1,-1,.5,2], gate/up [2,4], down [4,2]; the
+    activation sits on the gate product.  Expected values worked out by hand below."""
+    x = torch.tensor([[1.0, -1.0, 0.5, 2.0]])
+    wg = torch.tensor([0.1, 0.2, 0.3, 0.4, -0.1, 0.0, 0.5, -0.5]).view(2, 4)
+    wu = torch.tensor([0.5, -0.5, 0.25, 0.0, 0.1, 0.2, -0.3, 0.4]).view(2, 4)
+    wd = torch.tensor([1.0, -1.0, 0.5, 0.25, 0.0, 0.5, -0.5, 1.0]).view(4, 2)
+    gate = [0.1 - 0.2 + 0.15 + 0.8, -0.1 + 0.25 - 1.0]              # 0.85, -0.85
+    up = [0.5 + 0.5 + 0.125, 0.1 - 0.2 - 0.15 + 0.8]                # 1.125, 0.55
+    hid = [g / (1 + math.exp(-g)) * u for g, u in zip(gate, up)]
+    want = [hid[0] - hid[1], 0.5 * hid[0] + 0.25 * hid[1], 0.5 * hid[1], -0.5 * hid[0] + hid[1]]
+    got = P.swiglu_mlp(x, wg, wu, wd)[0]
+    assert torch.allclose(got, torch.tensor(want), atol=1e-6)
+    # the activation on the other product gives other numbers
+    other = [u / (1 + math.exp(-u)) * g for g, u in zip(gate, up)]
+    assert abs(other[0] - hid[0]) > 1e-2
 
 
 def test_float64_agrees_with_float32():
