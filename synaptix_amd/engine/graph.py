@@ -16,6 +16,7 @@ Captured are this package's kernels and torch's allocations only; no memset node
 from __future__ import annotations
 
 import ctypes as C
+import gc
 
 import numpy as np
 import torch
@@ -103,8 +104,19 @@ class DecodeRunner:
             torch.cuda.synchronize()
             self.scratch.frozen = True
             self.graph = torch.cuda.CUDAGraph()
-            with torch.no_grad(), torch.cuda.graph(self.graph):
-                self.logits = self._forward(ctx)
+            # No garbage collection while the stream is being captured: a dead object's finalizer may free
+            # device or pinned memory or destroy another graph (an engine and its runners form a cycle, so
+            # they die in the collector), which the runtime refuses during a capture and torch answers by
+            # ending the process.  Collect what is dead now, then hold the collector off until the capture ends.
+            gc.collect()
+            was_enabled = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.no_grad(), torch.cuda.graph(self.graph):
+                    self.logits = self._forward(ctx)
+            finally:
+                if was_enabled:
+                    gc.enable()
         self.graph.replay()
         out = self.out_tokens[:B].cpu().tolist()      # waits for the step
         for s in slots:
