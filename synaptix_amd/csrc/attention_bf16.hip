@@ -510,6 +510,7 @@ struct QkvIntake {
   const void* q_gain;  // RMSNorm gains of the q and k heads, or nullptr
   const void* k_gain;
   int gain_is_f32;
+  float gain_offset;   // the gain is gain_offset + w[i]
   float eps;
   const float* cos_t;  // rotation tables [positions][rot / 2], or nullptr
   const float* sin_t;
@@ -628,8 +629,8 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
           ss = wave_sum(ss);
           const float inv = rsqrtf(ss / (float)HD + in.eps);
           for (int d = 2 * lane; d < HD; d += 2 * SYN_WAVE) {
-            x[d] = load_gain(gain, in.gain_is_f32, d) * x[d] * inv;
-            x[d + 1] = load_gain(gain, in.gain_is_f32, d + 1) * x[d + 1] * inv;
+            x[d] = load_gain(gain, in.gain_is_f32, d, in.gain_offset) * x[d] * inv;
+            x[d + 1] = load_gain(gain, in.gain_is_f32, d + 1, in.gain_offset) * x[d + 1] * inv;
           }
         }
       }
@@ -855,7 +856,8 @@ SYN_EXPORT int syn_attention_decode_fused_bf16(const void* qkv, int n_parts, voi
                                                const int* page_table, int table_stride, const int* seq_len,
                                                int n_seqs, void* out, float* workspace, int n_splits, float scale,
                                                int window, int nh, int nkv, int hd, const void* q_gain,
-                                               const void* k_gain, int gain_is_f32, float eps, const float* cos_t,
+                                               const void* k_gain, int gain_is_f32, float gain_offset, float eps,
+                                               const float* cos_t,
                                                const float* sin_t, int rot, int own_kv, hipStream_t stream) {
   SYN_CHECK(rot % 2 == 0 && rot >= 0 && rot <= hd, "attention_decode_fused: rotary size %d does not fit head size %d",
             rot, hd);
@@ -865,7 +867,7 @@ SYN_EXPORT int syn_attention_decode_fused_bf16(const void* qkv, int n_parts, voi
   in.qkv = qkv;
   in.n_parts = n_parts;
   in.part_stride = (size_t)n_seqs * (nh + 2 * nkv) * hd;
-  in.q_gain = q_gain, in.k_gain = k_gain, in.gain_is_f32 = gain_is_f32, in.eps = eps;
+  in.q_gain = q_gain, in.k_gain = k_gain, in.gain_is_f32 = gain_is_f32, in.gain_offset = gain_offset, in.eps = eps;
   in.cos_t = cos_t, in.sin_t = sin_t, in.rot = rot, in.own_kv = own_kv;
   return launch_decode(nullptr, &in, k_pages, v_pages, page_table, table_stride, seq_len, n_seqs, out, workspace,
                        n_splits, scale, window, nh, nkv, hd, stream);

@@ -60,6 +60,25 @@ __device__ __forceinline__ float load_gain(const void* w, int is_f32, int i) {
   return is_f32 ? ((const float*)w)[i] : (float)((const bf16*)w)[i];
 }
 
+// the gain of a norm: w[i], or offset + w[i] for checkpoints that store the gain as a difference from one
+__device__ __forceinline__ float load_gain(const void* w, int is_f32, int i, float offset) {
+  return offset + load_gain(w, is_f32, i);
+}
+
+// ---- the activation of a gated feed-forward: act(gate) * up, on 32-bit sums ----
+// One place for every kernel that applies it (the epilogues of the gated products, the activation kernel
+// of the 32-bit path).  `act` is a code that the host checks against SYN_ACT_COUNT before any launch;
+// another activation is another case here and another name in the host's table.
+#define SYN_ACT_SILU 0
+#define SYN_ACT_COUNT 1
+__device__ __forceinline__ float gate_activation(int act, float g) {
+  switch (act) {
+    default:  // SYN_ACT_SILU: z / (1 + e^-z)
+      return g / (1.f + expf(-g));
+  }
+}
+__device__ __forceinline__ float gated(int act, float gate, float up) { return gate_activation(act, gate) * up; }
+
 // ---- reductions over the 64 lanes of a wave ----
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -41,7 +41,7 @@ SYN_EXPORT int syn_embed(const void* table, int table_is_f32, const int* ids, fl
 template <typename TOut>
 __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const float* __restrict__ delta, int n_parts,
                                    size_t part_stride, const int* __restrict__ rows, const void* __restrict__ gain,
-                                   int gain_is_f32, float eps, TOut* __restrict__ out, int H) {
+                                   int gain_is_f32, float gain_offset, float eps, TOut* __restrict__ out, int H) {
   __shared__ float red[16];
   const int r = rows ? rows[blockIdx.x] : blockIdx.x;
   float* x = resid + (size_t)r * H;
@@ -64,7 +64,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const float* __res
   const float inv = rsqrtf(ss / (float)H + eps);
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     const float v = write_back ? x[i] : summed(i);
-    o[i] = from_f32<TOut>(load_gain(gain, gain_is_f32, i) * v * inv);
+    o[i] = from_f32<TOut>(load_gain(gain, gain_is_f32, i, gain_offset) * v * inv);
   }
 }
 
@@ -92,7 +92,7 @@ __device__ inline void store4(bf16* o, int i4, const float4 r) {
 template <typename TOut, int VPT>
 __global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const float* __restrict__ delta, int n_parts,
                                        size_t part_stride, const int* __restrict__ rows,
-                                       const void* __restrict__ gain, int gain_is_f32, float eps,
+                                       const void* __restrict__ gain, int gain_is_f32, float gain_offset, float eps,
                                        TOut* __restrict__ out, int H) {
   __shared__ float red[16];
   const int r = rows ? rows[blockIdx.x] : blockIdx.x;
@@ -110,6 +110,7 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const float* _
     if (i < H4) {
       v[j] = x[i];
       g[j] = load_gain4(gain, gain_is_f32, i);  // fetched here, beside the values, not after the sum
+      g[j].x += gain_offset, g[j].y += gain_offset, g[j].z += gain_offset, g[j].w += gain_offset;
       if (d) {
         for (int p0 = 0; p0 < n_parts; p0 += 8) {
           float4 t[8];
@@ -141,8 +142,8 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ resid, const float* _
 }
 
 SYN_EXPORT int syn_add_rmsnorm(float* resid, const float* delta, int n_parts, int n_rows, const int* rows, int n_out,
-                               const void* gain, int gain_is_f32, float eps, void* out, int out_is_f32, int H,
-                               hipStream_t stream) {
+                               const void* gain, int gain_is_f32, float gain_offset, float eps, void* out,
+                               int out_is_f32, int H, hipStream_t stream) {
   SYN_CHECK(n_out > 0 && H > 0 && n_rows > 0, "add_rmsnorm: empty input (%d rows, width %d)", n_out, H);
   SYN_CHECK(n_parts >= 1 && n_parts <= 64, "add_rmsnorm: %d partial sums", n_parts);
   const size_t stride = (size_t)n_rows * H;
@@ -154,7 +155,7 @@ SYN_EXPORT int syn_add_rmsnorm(float* resid, const float* delta, int n_parts, in
     const int vpt = (H4 + block - 1) / block;  // 1 .. 4
 #define SYN_ARN(T, V)                                                                                          \
   add_rmsnorm_vec_kernel<T, V><<<n_out, block, 0, stream>>>(resid, delta, n_parts, stride, rows, gain, gain_is_f32, \
-                                                            eps, (T*)out, H)
+                                                            gain_offset, eps, (T*)out, H)
     if (out_is_f32) {
       if (vpt == 1) SYN_ARN(float, 1); else if (vpt == 2) SYN_ARN(float, 2); else SYN_ARN(float, 4);
     } else {
@@ -165,10 +166,10 @@ SYN_EXPORT int syn_add_rmsnorm(float* resid, const float* delta, int n_parts, in
     const int block = H >= 4096 ? 1024 : (H >= 1024 ? 512 : 256);
     if (out_is_f32)
       add_rmsnorm_kernel<float><<<n_out, block, 0, stream>>>(resid, delta, n_parts, stride, rows, gain, gain_is_f32,
-                                                            eps, (float*)out, H);
+                                                            gain_offset, eps, (float*)out, H);
     else
       add_rmsnorm_kernel<bf16><<<n_out, block, 0, stream>>>(resid, delta, n_parts, stride, rows, gain, gain_is_f32,
-                                                           eps, (bf16*)out, H);
+                                                           gain_offset, eps, (bf16*)out, H);
   }
   SYN_LAUNCH_CHECK("add_rmsnorm");
   return 0;
@@ -177,8 +178,8 @@ SYN_EXPORT int syn_add_rmsnorm(float* resid, const float* delta, int n_parts, in
 // ------------------------------------------------------------------ RMSNorm of rows of any width
 // One wave a row.
 template <typename T>
-__global__ void rmsnorm_rows_kernel(const T* __restrict__ x, const void* __restrict__ gain, int gain_is_f32, float eps,
-                                    T* __restrict__ out, int n_rows, int width) {
+__global__ void rmsnorm_rows_kernel(const T* __restrict__ x, const void* __restrict__ gain, int gain_is_f32,
+                                    float gain_offset, float eps, T* __restrict__ out, int n_rows, int width) {
   const int row = blockIdx.x * (blockDim.x / SYN_WAVE) + threadIdx.x / SYN_WAVE;
   if (row >= n_rows) return;
   const int lane = threadIdx.x % SYN_WAVE;
@@ -192,40 +193,40 @@ __global__ void rmsnorm_rows_kernel(const T* __restrict__ x, const void* __restr
   ss = wave_sum(ss);
   const float inv = rsqrtf(ss / (float)width + eps);
   for (int i = lane; i < width; i += SYN_WAVE)
-    o[i] = from_f32<T>(load_gain(gain, gain_is_f32, i) * to_f32<T>(xr[i]) * inv);
+    o[i] = from_f32<T>(load_gain(gain, gain_is_f32, i, gain_offset) * to_f32<T>(xr[i]) * inv);
 }
 
-SYN_EXPORT int syn_rmsnorm_rows(const void* x, int is_f32, const void* gain, int gain_is_f32, float eps, void* out,
-                                int n_rows, int width, hipStream_t stream) {
+SYN_EXPORT int syn_rmsnorm_rows(const void* x, int is_f32, const void* gain, int gain_is_f32, float gain_offset,
+                                float eps, void* out, int n_rows, int width, hipStream_t stream) {
   SYN_CHECK(n_rows > 0 && width > 0, "rmsnorm_rows: empty input (%d rows, width %d)", n_rows, width);
   const int wpb = 4;
   const int grid = (n_rows + wpb - 1) / wpb;
   if (is_f32)
-    rmsnorm_rows_kernel<float><<<grid, wpb * SYN_WAVE, 0, stream>>>((const float*)x, gain, gain_is_f32, eps,
-                                                                    (float*)out, n_rows, width);
+    rmsnorm_rows_kernel<float><<<grid, wpb * SYN_WAVE, 0, stream>>>((const float*)x, gain, gain_is_f32, gain_offset,
+                                                                    eps, (float*)out, n_rows, width);
   else
-    rmsnorm_rows_kernel<bf16><<<grid, wpb * SYN_WAVE, 0, stream>>>((const bf16*)x, gain, gain_is_f32, eps,
-                                                                   (bf16*)out, n_rows, width);
+    rmsnorm_rows_kernel<bf16><<<grid, wpb * SYN_WAVE, 0, stream>>>((const bf16*)x, gain, gain_is_f32, gain_offset,
+                                                                   eps, (bf16*)out, n_rows, width);
   SYN_LAUNCH_CHECK("rmsnorm_rows");
   return 0;
 }
 
 // ------------------------------------------------------------------ SwiGLU on a fused [gate | up] row
-// out[n, i] = silu(gu[n, i]) * gu[n, I + i], silu(z) = z / (1 + exp(-z)), in 32-bit.
+// out[n, i] = act(gu[n, i]) * gu[n, I + i] in 32-bit (gate_activation; silu(z) = z / (1 + exp(-z))).
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int n_rows, int I) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int n_rows, int I, int act) {
   const size_t total = (size_t)n_rows * I;
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
     const size_t n = idx / I;
     const int i = (int)(idx - n * I);
     const float g = to_f32<T>(gu[n * 2 * I + i]);
     const float u = to_f32<T>(gu[n * 2 * I + I + i]);
-    out[idx] = from_f32<T>(g / (1.f + expf(-g)) * u);
+    out[idx] = from_f32<T>(gated(act, g, u));
   }
 }
 
 // 8 values a thread with 16-byte loads (bf16, width a multiple of 8)
-__global__ void swiglu_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int n_rows, int I) {
+__global__ void swiglu_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int n_rows, int I, int act) {
   const int I8 = I / 8;
   const size_t total = (size_t)n_rows * I8;
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
@@ -235,21 +236,19 @@ __global__ void swiglu_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict
     const bf16x8 u = *(const bf16x8*)(gu + n * 2 * I + I + i);
     bf16x8 o;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float gf = (float)g[e];
-      o[e] = (bf16)(gf / (1.f + expf(-gf)) * (float)u[e]);
-    }
+    for (int e = 0; e < 8; ++e) o[e] = (bf16)gated(act, (float)g[e], (float)u[e]);
     *(bf16x8*)(out + n * I + i) = o;
   }
 }
 
-SYN_EXPORT int syn_swiglu(const void* gu, void* out, int is_f32, int n_rows, int I, hipStream_t stream) {
+SYN_EXPORT int syn_swiglu(const void* gu, void* out, int is_f32, int n_rows, int I, int act, hipStream_t stream) {
   SYN_CHECK(n_rows > 0 && I > 0, "swiglu: empty input (%d rows, width %d)", n_rows, I);
+  SYN_CHECK(act >= 0 && act < SYN_ACT_COUNT, "swiglu: unknown activation code %d", act);
   if (!is_f32 && I % 8 == 0 && (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0) {
     const size_t total = (size_t)n_rows * (I / 8);
     int grid = (int)((total + 255) / 256);
     if (grid > 65536) grid = 65536;
-    swiglu_vec8_kernel<<<grid, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, n_rows, I);
+    swiglu_vec8_kernel<<<grid, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, n_rows, I, act);
     SYN_LAUNCH_CHECK("swiglu");
     return 0;
   }
@@ -257,9 +256,9 @@ SYN_EXPORT int syn_swiglu(const void* gu, void* out, int is_f32, int n_rows, int
   int grid = (int)((total + 255) / 256);
   if (grid > 65536) grid = 65536;
   if (is_f32)
-    swiglu_kernel<float><<<grid, 256, 0, stream>>>((const float*)gu, (float*)out, n_rows, I);
+    swiglu_kernel<float><<<grid, 256, 0, stream>>>((const float*)gu, (float*)out, n_rows, I, act);
   else
-    swiglu_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, n_rows, I);
+    swiglu_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, n_rows, I, act);
   SYN_LAUNCH_CHECK("swiglu");
   return 0;
 }
@@ -280,9 +279,10 @@ __global__ void qk_norm_rope_kv_write_kernel(const TIn* __restrict__ qkv, int n_
                                              T* __restrict__ v_pages, const int* __restrict__ page_table,
                                              int table_stride, const int* __restrict__ tok_seq,
                                              const int* __restrict__ tok_pos, const void* __restrict__ q_gain,
-                                             const void* __restrict__ k_gain, int gain_is_f32, float eps,
-                                             const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
-                                             int nh, int nkv, int hd, int write_kv) {
+                                             const void* __restrict__ k_gain, int gain_is_f32, float gain_offset,
+                                             float eps, const float* __restrict__ cos_t,
+                                             const float* __restrict__ sin_t, int rot, int nh, int nkv, int hd,
+                                             int write_kv) {
   extern __shared__ float lds[];  // [waves][hd]
   const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
   const int heads = nh + 2 * nkv;
@@ -313,8 +313,8 @@ __global__ void qk_norm_rope_kv_write_kernel(const TIn* __restrict__ qkv, int n_
       ss = wave_sum(ss);
       const float inv = rsqrtf(ss / (float)hd + eps);
       for (int d = 2 * lane; d < hd; d += 2 * SYN_WAVE) {
-        xs[d] = load_gain(gain, gain_is_f32, d) * xs[d] * inv;
-        xs[d + 1] = load_gain(gain, gain_is_f32, d + 1) * xs[d + 1] * inv;
+        xs[d] = load_gain(gain, gain_is_f32, d, gain_offset) * xs[d] * inv;
+        xs[d + 1] = load_gain(gain, gain_is_f32, d + 1, gain_offset) * xs[d + 1] * inv;
       }
     }
   }
@@ -376,8 +376,8 @@ __global__ void __launch_bounds__(256)
 qk_heads_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ q_out, bf16* __restrict__ k_pages,
                 const int* __restrict__ page_table, int table_stride, const int* __restrict__ tok_seq,
                 const int* __restrict__ tok_pos, const void* __restrict__ q_gain, const void* __restrict__ k_gain,
-                int gain_is_f32, float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-                int n_tokens, int nh, int nkv, int n_active) {
+                int gain_is_f32, float gain_offset, float eps, const float* __restrict__ cos_t,
+                const float* __restrict__ sin_t, int n_tokens, int nh, int nkv, int n_active) {
   constexpr int HD = LPH * 8, HPB = 256 / LPH, half = HD / 2;
   constexpr int TPB = 4;  // tokens a block takes, their loads in flight together
   const int head_raw = blockIdx.y * HPB + threadIdx.x / LPH;  // q heads, then k heads
@@ -395,6 +395,8 @@ qk_heads_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ q_out, bf16* __
 #pragma unroll
       for (int e = 0; e < 8; ++e) g[e] = (float)gb[e];
     }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) g[e] += gain_offset;
   }
   bf16x8 raw[TPB];
   int pos[TPB];
@@ -488,8 +490,8 @@ v_block_write_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ v_pages, c
 SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, int n_parts, void* q_out, void* k_pages, void* v_pages,
                                          int is_f32, const int* page_table, int table_stride, const int* tok_seq,
                                          const int* tok_pos, const void* q_gain, const void* k_gain, int gain_is_f32,
-                                         float eps, const float* cos_t, const float* sin_t, int rot, int n_tokens,
-                                         int nh, int nkv, int hd, int write_kv, hipStream_t stream) {
+                                         float gain_offset, float eps, const float* cos_t, const float* sin_t, int rot,
+                                         int n_tokens, int nh, int nkv, int hd, int write_kv, hipStream_t stream) {
   SYN_CHECK(n_tokens > 0 && nh > 0 && nkv > 0 && hd > 0, "qk_norm_rope_kv_write: empty input");
   SYN_CHECK(rot % 2 == 0 && rot >= 0 && rot <= hd, "qk_norm_rope_kv_write: rotary size %d does not fit head size %d",
             rot, hd);
@@ -508,8 +510,8 @@ SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, int n_parts, void* q_o
     const dim3 grid((n_tokens + 3) / 4, (n_active + hpb - 1) / hpb);
 #define SYN_QKH(L)                                                                                                  \
   qk_heads_kernel<L><<<grid, 256, 0, stream>>>((const bf16*)qkv, (bf16*)q_out, (bf16*)k_pages, page_table,          \
-                                               table_stride, tok_seq, tok_pos, q_gain, k_gain, gain_is_f32, eps,     \
-                                               cos_t, sin_t, n_tokens, nh, nkv, n_active)
+                                               table_stride, tok_seq, tok_pos, q_gain, k_gain, gain_is_f32,          \
+                                               gain_offset, eps, cos_t, sin_t, n_tokens, nh, nkv, n_active)
     switch (lph) {
       case 2: SYN_QKH(2); break;
       case 4: SYN_QKH(4); break;
@@ -534,7 +536,8 @@ SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, int n_parts, void* q_o
 #define SYN_QK(T, TIn)                                                                                             \
   qk_norm_rope_kv_write_kernel<T, TIn><<<grid, wpb * SYN_WAVE, lds, stream>>>(                                     \
       (const TIn*)qkv, n_parts > 0 ? n_parts : 1, stride, (T*)q_out, (T*)k_pages, (T*)v_pages, page_table,          \
-      table_stride, tok_seq, tok_pos, q_gain, k_gain, gain_is_f32, eps, cos_t, sin_t, rot, nh, nkv, hd, write_kv)
+      table_stride, tok_seq, tok_pos, q_gain, k_gain, gain_is_f32, gain_offset, eps, cos_t, sin_t, rot, nh, nkv, hd,   \
+      write_kv)
   if (is_f32)
     SYN_QK(float, float);
   else if (n_parts > 0)

@@ -15,7 +15,7 @@
 //                  W arrive as whole 256-byte pieces, which streams them faster than loading MFMA
 //                  fragments (64 bytes a row) straight from memory.  K may be cut into slices
 //                  whose partial sums the reader adds.  With PAIRED, W holds the rows of a gate and of
-//                  an up projection in turns of 16 and the kernel stores silu(gate) * up, half
+//                  an up projection in turns of 16 and the kernel stores act(gate) * up, half
 //                  as wide, without the two products ever being stored.
 //
 // Reference counterparts: crates/synaptix-kernels-cuda/src/best_cu/gemm/gemm_bf16.cu (TN family,
@@ -24,6 +24,13 @@
 #include <type_traits>
 
 #include "common.h"
+
+// What a kernel does with its 32-bit sums: store them as float or as bf16, or (the kernels over paired
+// gate/up rows) store act(gate) * up as bf16 with the activation `act` of gate_activation.
+struct Epilogue {
+  int out_is_f32;
+  int act;
+};
 
 // ------------------------------------------------------------------ SIMT, any type
 #define SIMT_BM 64
@@ -80,7 +87,7 @@ gemm_simt_kernel(const TIn* __restrict__ x, const TIn* __restrict__ w, TOut* __r
 // rows are gate rows, the second the up rows of the same outputs, and silu(gate) * up is stored.
 template <int TILES, int KWAVES, int U, bool PAIRED>
 __global__ void __launch_bounds__(TILES * KWAVES * SYN_WAVE)
-gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
+gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, Epilogue ep,
                    int M, int N, int K) {
   static_assert(!PAIRED || TILES == 2, "a pair is two tiles");
   constexpr int WAVES = TILES * KWAVES;
@@ -136,7 +143,7 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
       const int m = 4 * (ln / 16) + j, col = (int)blockIdx.x * 16 + ln % 16;  // N / 2 outputs, 16 a workgroup
       if (m < M && 2 * col < N) {
         const float g = summed(0, j, ln), up = summed(1, j, ln);
-        ((bf16*)out)[(size_t)m * (N / 2) + col] = (bf16)(g / (1.f + expf(-g)) * up);
+        ((bf16*)out)[(size_t)m * (N / 2) + col] = (bf16)gated(ep.act, g, up);
       }
     }
   } else {
@@ -145,7 +152,7 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
       const int m = 4 * (ln / 16) + j, n = (blockIdx.x * TILES + t) * 16 + ln % 16;
       if (m < M && n < N) {
         const float v = summed(t, j, ln);
-        if (out_is_f32)
+        if (ep.out_is_f32)
           ((float*)out)[(size_t)m * N + n] = v;
         else
           ((bf16*)out)[(size_t)m * N + n] = (bf16)v;
@@ -155,11 +162,11 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
 }
 
 template <int TILES, int KWAVES, int U, bool PAIRED = false>
-static void launch_skinny(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
+static void launch_skinny(const bf16* x, const bf16* w, void* out, Epilogue ep, int M, int N, int K,
                           hipStream_t stream) {
   const int rows = TILES * 16;
   gemm_skinny_kernel<TILES, KWAVES, U, PAIRED>
-      <<<(N + rows - 1) / rows, TILES * KWAVES * SYN_WAVE, 0, stream>>>(x, w, out, out_is_f32, M, N, K);
+      <<<(N + rows - 1) / rows, TILES * KWAVES * SYN_WAVE, 0, stream>>>(x, w, out, ep, M, N, K);
 }
 
 // ------------------------------------------------------------------ few rows of x, W in fragment order
@@ -174,7 +181,7 @@ static void launch_skinny(const bf16* x, const bf16* w, void* out, int out_is_f3
 // then those KWAVES * U further on.
 template <int TILES, int KWAVES, int U, bool PAIRED>
 __global__ void __launch_bounds__(TILES * KWAVES * SYN_WAVE)
-gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void* __restrict__ out, int out_is_f32,
+gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void* __restrict__ out, Epilogue ep,
                    int M, int N, int K) {
   static_assert(!PAIRED || TILES == 2, "a pair is two tiles");
   constexpr int WAVES = TILES * KWAVES;
@@ -218,7 +225,7 @@ gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void
       const int m = 4 * (ln / 16) + j, col = (int)blockIdx.x * 16 + ln % 16;  // N / 2 outputs, 16 a workgroup
       if (m < M && 2 * col < N) {
         const float g = summed(0, j, ln), up = summed(1, j, ln);
-        ((bf16*)out)[(size_t)m * (N / 2) + col] = (bf16)(g / (1.f + expf(-g)) * up);
+        ((bf16*)out)[(size_t)m * (N / 2) + col] = (bf16)gated(ep.act, g, up);
       }
     }
   } else {
@@ -227,7 +234,7 @@ gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void
       const int m = 4 * (ln / 16) + j, n = ((int)blockIdx.x * TILES + t) * 16 + ln % 16;
       if (m < M && n < N) {
         const float v = summed(t, j, ln);
-        if (out_is_f32)
+        if (ep.out_is_f32)
           ((float*)out)[(size_t)m * N + n] = v;
         else
           ((bf16*)out)[(size_t)m * N + n] = (bf16)v;
@@ -237,11 +244,11 @@ gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void
 }
 
 template <int TILES, int KWAVES, int U, bool PAIRED = false>
-static void launch_packed(const bf16* x, const bf16* wp, void* out, int out_is_f32, int M, int N, int K,
+static void launch_packed(const bf16* x, const bf16* wp, void* out, Epilogue ep, int M, int N, int K,
                           hipStream_t stream) {
   const int rows = TILES * 16;
   gemm_packed_kernel<TILES, KWAVES, U, PAIRED>
-      <<<(N + rows - 1) / rows, TILES * KWAVES * SYN_WAVE, 0, stream>>>(x, wp, out, out_is_f32, M, N, K);
+      <<<(N + rows - 1) / rows, TILES * KWAVES * SYN_WAVE, 0, stream>>>(x, wp, out, ep, M, N, K);
 }
 
 // ------------------------------------------------------------------ shared by the tiled kernels
@@ -276,7 +283,7 @@ static int tile_grid(int M, int N, int BM, int BN) {
 // partner's gate, their own up), so that a store covers 32 consecutive outputs of a row (64 bytes, not
 // twice 32).  A last tile without a neighbour is stored by the lanes of the first kind alone.
 template <int TM, int TN, bool PAIRED>
-__device__ __forceinline__ void store_tiles(const f32x16 (&acc)[TM][TN], void* __restrict__ out, int out_is_f32,
+__device__ __forceinline__ void store_tiles(const f32x16 (&acc)[TM][TN], void* __restrict__ out, Epilogue ep,
                                             size_t slice, int M, int N, int mw, int nw, int lane) {
   if constexpr (PAIRED) {
     const bool first = lane % 32 < 16;
@@ -292,10 +299,10 @@ __device__ __forceinline__ void store_tiles(const f32x16 (&acc)[TM][TN], void* _
             const float own1 = acc[i][j + 1 < TN ? j + 1 : j][e], other1 = __shfl_xor(own1, 16, SYN_WAVE);
             const float g = first ? own0 : other1, up = first ? other0 : own1;
             if (m < M && nw + (j + (first ? 0 : 1)) * 32 < N)
-              ((bf16*)out)[(size_t)m * (N / 2) + (nw + j * 32) / 2 + lane % 32] = (bf16)(g / (1.f + expf(-g)) * up);
+              ((bf16*)out)[(size_t)m * (N / 2) + (nw + j * 32) / 2 + lane % 32] = (bf16)gated(ep.act, g, up);
           } else {
             if (m < M && nw + j * 32 < N && first)
-              ((bf16*)out)[(size_t)m * (N / 2) + (nw + j * 32) / 2 + lane % 16] = (bf16)(own0 / (1.f + expf(-own0)) * other0);
+              ((bf16*)out)[(size_t)m * (N / 2) + (nw + j * 32) / 2 + lane % 16] = (bf16)gated(ep.act, own0, other0);
           }
         }
   } else {
@@ -308,7 +315,7 @@ __device__ __forceinline__ void store_tiles(const f32x16 (&acc)[TM][TN], void* _
           const int m = mw + i * 32 + 8 * (e / 4) + 4 * (lane / 32) + e % 4;
           const int n = nw + j * 32 + lane % 32;
           if (m < M && n < N) {
-            if (out_is_f32)
+            if (ep.out_is_f32)
               ((float*)out)[(slice * M + m) * N + n] = acc[i][j][e];
             else
               ((bf16*)out)[(size_t)m * N + n] = (bf16)acc[i][j][e];
@@ -325,7 +332,7 @@ __device__ __forceinline__ void store_tiles(const f32x16 (&acc)[TM][TN], void* _
 // into registers, and is stored into the other buffer before the barrier.
 template <int BM, int BN, int BK, int WM, int WN, bool KTAIL, bool PAIRED>
 __global__ void __launch_bounds__(64 * WM * WN)
-gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
+gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, Epilogue ep,
                   int M, int N, int K, int k_slice) {
   constexpr bool FEW = BM <= 64;                     // the variants for few rows of x: slices of K, absent rows
   constexpr int THREADS = 64 * WM * WN;              // WM x WN waves
@@ -415,11 +422,11 @@ gemm_tiled_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* 
     __syncthreads();
   }
 
-  store_tiles<TM, TN, PAIRED>(acc, out, out_is_f32, FEW ? blockIdx.y : 0, M, N, m0 + wm, n0 + wn, lane);
+  store_tiles<TM, TN, PAIRED>(acc, out, ep, FEW ? blockIdx.y : 0, M, N, m0 + wm, n0 + wn, lane);
 }
 
 template <int BM, int BN, int BK, int WM, int WN, bool PAIRED = false>
-static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
+static int launch_tiled(const bf16* x, const bf16* w, void* out, Epilogue ep, int M, int N, int K,
                         hipStream_t stream, int slices = 1) {
   SYN_CHECK(slices == 1 || BM <= 64, "gemm: slices of K only with the tiles for few rows");
   const int k_slice = ((K + slices - 1) / slices + 127) / 128 * 128;  // the same cut as launch_direct makes
@@ -438,10 +445,10 @@ static int launch_tiled(const bf16* x, const bf16* w, void* out, int out_is_f32,
   // whole k-tiles only, and no slice that begins at or beyond the end of K: then no chunk needs a check
   if (K % BK == 0 && k_slice % BK == 0 && (long)(slices - 1) * k_slice < K)
     gemm_tiled_kernel<BM, BN, BK, WM, WN, false, PAIRED>
-        <<<dim3(grid, slices), 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
+        <<<dim3(grid, slices), 64 * WM * WN, lds, stream>>>(x, w, out, ep, M, N, K, k_slice);
   else
     gemm_tiled_kernel<BM, BN, BK, WM, WN, true, PAIRED>
-        <<<dim3(grid, slices), 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
+        <<<dim3(grid, slices), 64 * WM * WN, lds, stream>>>(x, w, out, ep, M, N, K, k_slice);
   return 0;
 }
 
@@ -462,7 +469,7 @@ __device__ __forceinline__ int direct_swizzle(int row) {
 
 template <int BM, int BN, int BK, int WM, int WN, bool PAIRED, int STAGES>
 __global__ void __launch_bounds__(64 * WM * WN)
-gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
+gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, Epilogue ep,
                    int M, int N, int K, int k_slice) {
   static_assert((BK == 64 || BK == 128 || BK == 256) && STAGES >= 2, "k-tiles of 64, 128 or 256 in two or more buffers");
   constexpr int WAVES = WM * WN;
@@ -564,12 +571,12 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
     next_landed(more);
     __builtin_amdgcn_s_barrier();
   }
-  store_tiles<TM, TN, PAIRED>(acc, out, out_is_f32, blockIdx.y, M, N, m0 + wm, n0 + wn, lane);
+  store_tiles<TM, TN, PAIRED>(acc, out, ep, blockIdx.y, M, N, m0 + wm, n0 + wn, lane);
 }
 
 // slices > 1 only with a float output [slices, M, N]; K must be a multiple of BK
 template <int BM, int BN, int BK, int WM, int WN, bool PAIRED = false, int STAGES = 3>
-static int launch_direct(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
+static int launch_direct(const bf16* x, const bf16* w, void* out, Epilogue ep, int M, int N, int K,
                          hipStream_t stream, int slices = 1) {
   SYN_CHECK(K % BK == 0, "gemm: K = %d is no multiple of the k-tile %d", K, BK);
   const int step = BK > 128 ? BK : 128;
@@ -583,7 +590,7 @@ static int launch_direct(const bf16* x, const bf16* w, void* out, int out_is_f32
     raised = true;
   }
   gemm_direct_kernel<BM, BN, BK, WM, WN, PAIRED, STAGES>
-      <<<dim3(tile_grid(M, N, BM, BN), slices), 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
+      <<<dim3(tile_grid(M, N, BM, BN), slices), 64 * WM * WN, lds, stream>>>(x, w, out, ep, M, N, K, k_slice);
   return 0;
 }
 
@@ -603,7 +610,7 @@ static int launch_direct(const bf16* x, const bf16* w, void* out, int out_is_f32
 // hold up the waves that issue them, so their spread matters more than their number.
 template <int BM, int BN, int WM, int WN, bool PAIRED>
 __global__ void __launch_bounds__(64 * WM * WN)
-gemm_pipelined_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, int out_is_f32,
+gemm_pipelined_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, Epilogue ep,
                       int M, int N, int K, int k_slice) {
   constexpr int BK = 64;
   constexpr int WAVES = WM * WN;
@@ -727,11 +734,11 @@ gemm_pipelined_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, vo
   for (; kt + 2 < nk; ++kt) tile(kt, std::true_type{}, std::true_type{});
   if (kt + 1 < nk) tile(kt++, std::false_type{}, std::true_type{});
   tile(kt, std::false_type{}, std::false_type{});
-  store_tiles<TM, TN, PAIRED>(acc, out, out_is_f32, blockIdx.y, M, N, m0 + wm, n0 + wn, lane);
+  store_tiles<TM, TN, PAIRED>(acc, out, ep, blockIdx.y, M, N, m0 + wm, n0 + wn, lane);
 }
 
 template <int BM, int BN, int WM, int WN, bool PAIRED = false>
-static int launch_pipelined(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
+static int launch_pipelined(const bf16* x, const bf16* w, void* out, Epilogue ep, int M, int N, int K,
                             hipStream_t stream, int slices = 1) {
   SYN_CHECK(K % 64 == 0, "gemm: K = %d is no multiple of the k-tile 64", K);
   const int k_slice = ((K + slices - 1) / slices + 127) / 128 * 128;  // the same cut as the tiles for few rows make
@@ -745,13 +752,13 @@ static int launch_pipelined(const bf16* x, const bf16* w, void* out, int out_is_
     raised = true;
   }
   gemm_pipelined_kernel<BM, BN, WM, WN, PAIRED>
-      <<<dim3(tile_grid(M, N, BM, BN), slices), 64 * WM * WN, lds, stream>>>(x, w, out, out_is_f32, M, N, K, k_slice);
+      <<<dim3(tile_grid(M, N, BM, BN), slices), 64 * WM * WN, lds, stream>>>(x, w, out, ep, M, N, K, k_slice);
   return 0;
 }
 
 // M > 64: the tile shape by pick_large_tile; loads straight into LDS where K allows it
 template <bool PAIRED>
-static int launch_large(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
+static int launch_large(const bf16* x, const bf16* w, void* out, Epilogue ep, int M, int N, int K,
                         hipStream_t stream, int slices = 1);
 
 // Which of the large tiles for M > 64: 0 = 256 x 256, 1 = 256 x 192 (one workgroup of four waves a compute
@@ -774,19 +781,19 @@ static int pick_large_tile(int M, int N) {
 }
 
 template <bool PAIRED>
-static int launch_large(const bf16* x, const bf16* w, void* out, int out_is_f32, int M, int N, int K,
+static int launch_large(const bf16* x, const bf16* w, void* out, Epilogue ep, int M, int N, int K,
                         hipStream_t stream, int slices) {
   // cut along K (the reader adds the partial sums): the largest tile, which the slices multiply
-  if (slices > 1) return launch_pipelined<256, 256, 2, 4, PAIRED>(x, w, out, out_is_f32, M, N, K, stream, slices);
+  if (slices > 1) return launch_pipelined<256, 256, 2, 4, PAIRED>(x, w, out, ep, M, N, K, stream, slices);
   const int shape = pick_large_tile(M, N);
   if (K % 64 == 0) {
-    if (shape == 0) return launch_pipelined<256, 256, 2, 4, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
-    if (shape == 1) return launch_pipelined<256, 192, 2, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
-    return launch_pipelined<128, 128, 2, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
+    if (shape == 0) return launch_pipelined<256, 256, 2, 4, PAIRED>(x, w, out, ep, M, N, K, stream);
+    if (shape == 1) return launch_pipelined<256, 192, 2, 2, PAIRED>(x, w, out, ep, M, N, K, stream);
+    return launch_pipelined<128, 128, 2, 2, PAIRED>(x, w, out, ep, M, N, K, stream);
   }
-  if (shape == 0) return launch_tiled<256, 256, 64, 4, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
-  if (shape == 1) return launch_tiled<256, 192, 64, 4, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
-  return launch_tiled<128, 128, 64, 2, 2, PAIRED>(x, w, out, out_is_f32, M, N, K, stream);
+  if (shape == 0) return launch_tiled<256, 256, 64, 4, 2, PAIRED>(x, w, out, ep, M, N, K, stream);
+  if (shape == 1) return launch_tiled<256, 192, 64, 4, 2, PAIRED>(x, w, out, ep, M, N, K, stream);
+  return launch_tiled<128, 128, 64, 2, 2, PAIRED>(x, w, out, ep, M, N, K, stream);
 }
 
 // ------------------------------------------------------------------ entry point
@@ -806,6 +813,7 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
     return 0;
   }
   const int out_is_f32 = dtype == 2;
+  const Epilogue ep = {out_is_f32, SYN_ACT_SILU};   // (no activation in a plain product)
   const bool aligned = (K % 8 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
   SYN_CHECK(slices == 1 || aligned, "gemm: slices of K need 16-byte aligned operands");
   if (force_simt || !aligned) {
@@ -829,20 +837,20 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   int rc = 0;
   if (M == 1 && slices == 1) {
     // one row: fragments of W straight from memory, K split over the waves
-    if (N <= 8192) launch_skinny<1, 16, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
-    else launch_skinny<1, 8, 4>(xb, wb, out, out_is_f32, M, N, K, stream);
+    if (N <= 8192) launch_skinny<1, 16, 4>(xb, wb, out, ep, M, N, K, stream);
+    else launch_skinny<1, 8, 4>(xb, wb, out, ep, M, N, K, stream);
   } else if (M <= 32) {
     // few rows: memory-bound; small tiles (many workgroups), deep in K (long pieces of each row), three
     // k-tiles in flight, straight into LDS where K allows it
-    if (N >= 65536 && K % 256 == 0) rc = launch_direct<32, 64, 256, 1, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
-    else if (N >= 65536) rc = launch_tiled<32, 32, 256, 1, 1>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
-    else if (K % 128 == 0) rc = launch_direct<32, 64, 128, 1, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
-    else rc = launch_tiled<32, 64, 128, 1, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
+    if (N >= 65536 && K % 256 == 0) rc = launch_direct<32, 64, 256, 1, 2>(xb, wb, out, ep, M, N, K, stream, slices);
+    else if (N >= 65536) rc = launch_tiled<32, 32, 256, 1, 1>(xb, wb, out, ep, M, N, K, stream, slices);
+    else if (K % 128 == 0) rc = launch_direct<32, 64, 128, 1, 2>(xb, wb, out, ep, M, N, K, stream, slices);
+    else rc = launch_tiled<32, 64, 128, 1, 2>(xb, wb, out, ep, M, N, K, stream, slices);
   } else if (M <= 64 || few_large_tiles) {
-    if (K % 128 == 0) rc = launch_direct<64, 64, 128, 2, 2, false, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
-    else rc = launch_tiled<64, 64, 128, 2, 2>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
+    if (K % 128 == 0) rc = launch_direct<64, 64, 128, 2, 2, false, 2>(xb, wb, out, ep, M, N, K, stream, slices);
+    else rc = launch_tiled<64, 64, 128, 2, 2>(xb, wb, out, ep, M, N, K, stream, slices);
   } else {
-    rc = launch_large<false>(xb, wb, out, out_is_f32, M, N, K, stream, slices);
+    rc = launch_large<false>(xb, wb, out, ep, M, N, K, stream, slices);
   }
   if (rc) return rc;
   SYN_LAUNCH_CHECK("gemm");
@@ -852,8 +860,10 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
 // out[M, N/2] = silu(x . Wg^T) * (x . Wu^T), bf16, where w [N, K] holds the rows of Wg and of Wu in
 // turns of 16: rows 32b .. 32b+15 are rows 16b .. 16b+15 of Wg, rows 32b+16 .. 32b+31 those of Wu.
 // The activation is applied to the 32-bit sums and rounded once.
-SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, int N, int K, hipStream_t stream) {
+SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, int N, int K, int act, hipStream_t stream) {
   SYN_CHECK(M > 0 && N > 0 && K > 0, "gemm_swiglu: empty shape M=%d N=%d K=%d", M, N, K);
+  SYN_CHECK(act >= 0 && act < SYN_ACT_COUNT, "gemm_swiglu: unknown activation code %d", act);
+  const Epilogue ep = {0, act};
   SYN_CHECK(N % 32 == 0, "gemm_swiglu: %d paired rows are no multiple of 32", N);
   SYN_CHECK(K % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0,
             "gemm_swiglu: K = %d must be a multiple of 8 and the operands 16-byte aligned", K);
@@ -862,16 +872,16 @@ SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, i
   int rc = 0;
   if (M == 1) {
     // one row: fragments of W straight from memory; eight waves on the gate rows, eight on the up rows
-    launch_skinny<2, 8, 4, true>(xb, wb, out, 0, M, N, K, stream);
+    launch_skinny<2, 8, 4, true>(xb, wb, out, ep, M, N, K, stream);
   } else if (M <= 32) {
-    if (N >= 65536) rc = launch_tiled<32, 32, 256, 1, 1, true>(xb, wb, out, 0, M, N, K, stream);
-    else if (K % 128 == 0) rc = launch_direct<32, 64, 128, 1, 2, true>(xb, wb, out, 0, M, N, K, stream);
-    else rc = launch_tiled<32, 64, 128, 1, 2, true>(xb, wb, out, 0, M, N, K, stream);
+    if (N >= 65536) rc = launch_tiled<32, 32, 256, 1, 1, true>(xb, wb, out, ep, M, N, K, stream);
+    else if (K % 128 == 0) rc = launch_direct<32, 64, 128, 1, 2, true>(xb, wb, out, ep, M, N, K, stream);
+    else rc = launch_tiled<32, 64, 128, 1, 2, true>(xb, wb, out, ep, M, N, K, stream);
   } else if (M <= 64) {
-    if (K % 128 == 0) rc = launch_direct<64, 64, 128, 2, 2, true, 2>(xb, wb, out, 0, M, N, K, stream);
-    else rc = launch_tiled<64, 64, 128, 2, 2, true>(xb, wb, out, 0, M, N, K, stream);
+    if (K % 128 == 0) rc = launch_direct<64, 64, 128, 2, 2, true, 2>(xb, wb, out, ep, M, N, K, stream);
+    else rc = launch_tiled<64, 64, 128, 2, 2, true>(xb, wb, out, ep, M, N, K, stream);
   } else {
-    rc = launch_large<true>(xb, wb, out, 0, M, N, K, stream);
+    rc = launch_large<true>(xb, wb, out, ep, M, N, K, stream);
   }
   if (rc) return rc;
   SYN_LAUNCH_CHECK("gemm_swiglu");
@@ -882,7 +892,9 @@ SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, i
 // gemm_packed_kernel; N a multiple of 16, K of 32).  out_code: 1 = bf16 [M, N], 2 = float [M, N];
 // paired: W holds gate and up rows in turns of 16 and out is bf16 [M, N / 2] = silu(gate) * up.
 SYN_EXPORT int syn_gemm_packed(const void* x, const void* wp, void* out, int out_code, int M, int N, int K, int paired,
-                               hipStream_t stream) {
+                               int act, hipStream_t stream) {
+  SYN_CHECK(act >= 0 && act < SYN_ACT_COUNT, "gemm_packed: unknown activation code %d", act);
+  const Epilogue ep = {out_code == 2, act};
   SYN_CHECK(M > 0 && M <= 16 && N > 0 && K > 0, "gemm_packed: M = %d (1 .. 16), N = %d, K = %d", M, N, K);
   SYN_CHECK(N % 16 == 0 && K % 32 == 0 && (!paired || N % 32 == 0),
             "gemm_packed: N = %d must be a multiple of 16 (32 for paired rows), K = %d of 32", N, K);
@@ -892,9 +904,9 @@ SYN_EXPORT int syn_gemm_packed(const void* x, const void* wp, void* out, int out
   const bf16* xb = (const bf16*)x;
   const bf16* wb = (const bf16*)wp;
   // from sweeps at N = 4096 .. 151936, K = 4096 and 12288, 1 and 8 rows
-  if (paired) launch_packed<2, 8, 4, true>(xb, wb, out, 0, M, N, K, stream);
-  else if (N <= 8192) launch_packed<1, 16, 2>(xb, wb, out, out_code == 2, M, N, K, stream);
-  else launch_packed<1, 8, 8>(xb, wb, out, out_code == 2, M, N, K, stream);
+  if (paired) launch_packed<2, 8, 4, true>(xb, wb, out, ep, M, N, K, stream);
+  else if (N <= 8192) launch_packed<1, 16, 2>(xb, wb, out, ep, M, N, K, stream);
+  else launch_packed<1, 8, 8>(xb, wb, out, ep, M, N, K, stream);
   SYN_LAUNCH_CHECK("gemm_packed");
   return 0;
 }

@@ -83,6 +83,16 @@ def _is_f32(t):
     return 1 if t.dtype == _F32 else 0
 
 
+# The activations of a gated feed-forward that the kernels apply (codes of gate_activation in csrc/common.h).
+ACTIVATIONS = {"silu": 0, "swish": 0}
+
+
+def activation_code(name) -> int:
+    if name not in ACTIVATIONS:
+        raise KernelError(f"activation {name!r}: the kernels apply {sorted(set(ACTIVATIONS))}")
+    return ACTIVATIONS[name]
+
+
 # ----------------------------------------------------------------------------- rows
 
 def embed(table, ids, resid):
@@ -95,8 +105,8 @@ def embed(table, ids, resid):
           ids.shape[0], H, _stream())
 
 
-def add_rmsnorm(resid, delta, gain, eps, out, rows=None):
-    """rows is None:  resid += delta (when given), out = RMSNorm(resid) * gain, for every row.
+def add_rmsnorm(resid, delta, gain, eps, out, rows=None, gain_offset=0.0):
+    """rows is None:  resid += delta (when given), out = RMSNorm(resid) * (gain_offset + gain), for every row.
     rows [n] int32: out[i] = RMSNorm(resid[rows[i]] + delta[rows[i]]) * gain; resid is not written.
     delta may be [S, N, H]: partial sums that are added up on the way."""
     _need(resid, "add_rmsnorm.resid", _F32, (None, None))
@@ -115,27 +125,28 @@ def add_rmsnorm(resid, delta, gain, eps, out, rows=None):
         n_out = rows.shape[0]
     _need(out, "add_rmsnorm.out", (_BF16, _F32), (n_out, H))
     _call(load_library("core"), "syn_add_rmsnorm", _ptr(resid), _ptr(delta), n_parts, N, _ptr(rows), n_out, _ptr(gain),
-          _is_f32(gain), ctypes.c_float(eps), _ptr(out), _is_f32(out), H, _stream())
+          _is_f32(gain), ctypes.c_float(gain_offset), ctypes.c_float(eps), _ptr(out), _is_f32(out), H, _stream())
 
 
-def rmsnorm_rows(x, gain, eps, out):
-    """out = RMSNorm(x) * gain over the last axis; x [..., D] bf16|f32, out like x."""
+def rmsnorm_rows(x, gain, eps, out, gain_offset=0.0):
+    """out = RMSNorm(x) * (gain_offset + gain) over the last axis; x [..., D] bf16|f32, out like x."""
     _need(x, "rmsnorm_rows.x", (_BF16, _F32))
     D = x.shape[-1]
     _need(gain, "rmsnorm_rows.gain", (_BF16, _F32), (D,))
     _need(out, "rmsnorm_rows.out", x.dtype, tuple(x.shape))
     _call(load_library("core"), "syn_rmsnorm_rows", _ptr(x), _is_f32(x), _ptr(gain), _is_f32(gain),
-          ctypes.c_float(eps), _ptr(out), x.numel() // D, D, _stream())
+          ctypes.c_float(gain_offset), ctypes.c_float(eps), _ptr(out), x.numel() // D, D, _stream())
 
 
-def swiglu(gate_up, out):
-    """out[n, i] = silu(gate_up[n, i]) * gate_up[n, I + i]."""
+def swiglu(gate_up, out, activation="silu"):
+    """out[n, i] = act(gate_up[n, i]) * gate_up[n, I + i]."""
     _need(gate_up, "swiglu.gate_up", (_BF16, _F32), (None, None))
     N, I2 = gate_up.shape
     if I2 % 2:
         raise KernelError(f"swiglu: fused width {I2} is odd")
     _need(out, "swiglu.out", gate_up.dtype, (N, I2 // 2))
-    _call(load_library("core"), "syn_swiglu", _ptr(gate_up), _ptr(out), _is_f32(gate_up), N, I2 // 2, _stream())
+    _call(load_library("core"), "syn_swiglu", _ptr(gate_up), _ptr(out), _is_f32(gate_up), N, I2 // 2,
+          activation_code(activation), _stream())
 
 
 # ----------------------------------------------------------------------------- matrix product
@@ -178,8 +189,8 @@ def pair_rows(gate, up):
     return torch.stack([gate.view(I // PAIR, PAIR, K), up.view(I // PAIR, PAIR, K)], 1).reshape(2 * I, K).contiguous()
 
 
-def gemm_swiglu(x, w_paired, out):
-    """out[M, I] = silu(x . Wg^T) * (x . Wu^T) in bf16 with w_paired = pair_rows(Wg, Wu): the
+def gemm_swiglu(x, w_paired, out, activation="silu"):
+    """out[M, I] = act(x . Wg^T) * (x . Wu^T) in bf16 with w_paired = pair_rows(Wg, Wu): the
     activation on the 32-bit sums inside the product, so that the two products are never stored."""
     _need(x, "gemm_swiglu.x", _BF16, (None, None))
     M, K = x.shape
@@ -188,7 +199,8 @@ def gemm_swiglu(x, w_paired, out):
     if N % (2 * PAIR) or K % 8:
         raise KernelError(f"gemm_swiglu: {N} paired rows, K = {K} (multiples of {2 * PAIR} and of 8)")
     _need(out, "gemm_swiglu.out", _BF16, (M, N // 2))
-    _call(load_library("core"), "syn_gemm_swiglu", _ptr(x), _ptr(w_paired), _ptr(out), M, N, K, _stream())
+    _call(load_library("core"), "syn_gemm_swiglu", _ptr(x), _ptr(w_paired), _ptr(out), M, N, K,
+          activation_code(activation), _stream())
 
 
 PACKED_MAX_ROWS = 8   # up to this many rows of x the products over packed weights are the faster ones
@@ -210,9 +222,9 @@ def unpack_weight(wp):
     return wp.view(nt, nks, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(nt * 16, nks * 32).contiguous()
 
 
-def gemm_packed(x, wp, out, paired=False):
+def gemm_packed(x, wp, out, paired=False, activation="silu"):
     """out[M, N] (bf16 or float) = x[M, K] . W^T for M <= 16 with wp = pack_weight(W); paired: W holds gate and
-    up rows in turns of 16 (pair_rows) and out [M, N / 2] bf16 = silu(gate) * up."""
+    up rows in turns of 16 (pair_rows) and out [M, N / 2] bf16 = act(gate) * up."""
     _need(x, "gemm_packed.x", _BF16, (None, None))
     M, K = x.shape
     if K % 32:
@@ -226,7 +238,7 @@ def gemm_packed(x, wp, out, paired=False):
     else:
         _need(out, "gemm_packed.out", (_BF16, _F32), (M, N))
     _call(load_library("core"), "syn_gemm_packed", _ptr(x), _ptr(wp), _ptr(out), 2 if out.dtype == _F32 else 1,
-          M, N, K, 1 if paired else 0, _stream())
+          M, N, K, 1 if paired else 0, activation_code(activation), _stream())
 
 
 def gemm_slices(M, N, K, dtype):
@@ -286,10 +298,10 @@ def _check_pages(k_pages, v_pages, dtype, nkv, hd, name):
 
 
 def qk_norm_rope_kv_write(qkv, q_out, k_pages, v_pages, page_table, tok_seq, tok_pos, q_gain, k_gain, eps,
-                          cos, sin, n_heads, n_kv_heads, head_dim, write_kv=True):
+                          cos, sin, n_heads, n_kv_heads, head_dim, write_kv=True, gain_offset=0.0):
     """qkv [N, width] in the activation type, or float partial sums [S, N, width] that are added first.
     Split a fused [q | k | v] projection row into heads; RMSNorm q and k heads (if gains are
-    given), rotate them at tok_pos (if tables are given; their width is rotary_dim / 2), write q to
+    given; the gain is gain_offset + its tensor), rotate them at tok_pos (if tables are given; their width is rotary_dim / 2), write q to
     q_out [N, nh*hd], k and v into the cache pages of sequence tok_seq[n] at position tok_pos[n]
     (not with write_kv False: a layer that reads a cache which another layer writes)."""
     nh, nkv, hd = n_heads, n_kv_heads, head_dim
@@ -325,7 +337,8 @@ def qk_norm_rope_kv_write(qkv, q_out, k_pages, v_pages, page_table, tok_seq, tok
             raise KernelError(f"qk_norm_rope_kv_write: rotary size {rot} exceeds head size {hd}")
     _call(load_library("core"), "syn_qk_norm_rope_kv_write", _ptr(qkv), n_parts, _ptr(q_out), _ptr(k_pages), _ptr(v_pages),
           _is_f32(q_out), _ptr(page_table), page_table.shape[1], _ptr(tok_seq), _ptr(tok_pos), _ptr(q_gain), _ptr(k_gain),
-          gain_f32, ctypes.c_float(eps), _ptr(cos), _ptr(sin), rot, N, nh, nkv, hd, 1 if write_kv else 0, _stream())
+          gain_f32, ctypes.c_float(gain_offset), ctypes.c_float(eps), _ptr(cos), _ptr(sin), rot, N, nh, nkv, hd,
+          1 if write_kv else 0, _stream())
 
 
 def attention_f32(q, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale, window, n_heads, n_kv_heads,
@@ -411,7 +424,8 @@ def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspa
 
 
 def attention_decode_fused_bf16(qkv, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
-                                n_heads, n_kv_heads, head_dim, q_gain, k_gain, eps, cos, sin, write_kv=True):
+                                n_heads, n_kv_heads, head_dim, q_gain, k_gain, eps, cos, sin, write_kv=True,
+                                gain_offset=0.0):
     """attention_decode_bf16 for one new token a sequence whose q, k and v come straight from the
     fused projection: qkv [B, (nh + 2 nkv) * hd] in bf16, or float partial sums [S, B, ...] that are
     added first.  The q/k RMSNorm (if gains are given), the rotation at position seq_len - 1 (if
@@ -453,7 +467,7 @@ def attention_decode_fused_bf16(qkv, k_pages, v_pages, page_table, seq_len, out,
     _call(_attn_lib(hd), "syn_attention_decode_fused_bf16", _ptr(qkv), n_parts, _ptr(k_pages), _ptr(v_pages),
           _ptr(page_table), page_table.shape[1], _ptr(seq_len), B, _ptr(out), _ptr(workspace), int(n_splits),
           ctypes.c_float(scale), int(window or 0), nh, nkv, hd, _ptr(q_gain), _ptr(k_gain), gain_f32,
-          ctypes.c_float(eps), _ptr(cos), _ptr(sin), rot, 1 if write_kv else 0, _stream())
+          ctypes.c_float(gain_offset), ctypes.c_float(eps), _ptr(cos), _ptr(sin), rot, 1 if write_kv else 0, _stream())
 
 
 # ----------------------------------------------------------------------------- sampling

@@ -22,9 +22,11 @@ class FeedForward(Part):
 
 class GatedMlp(FeedForward):
     def __init__(self, prefix: str, hidden: int, intermediate: int, activation: str = "silu"):
-        if activation not in ("silu", "swish"):
-            raise ValueError(f"activation {activation!r} is not built (silu only)")
-        self.prefix, self.hidden, self.intermediate = prefix, hidden, intermediate
+        try:
+            ops.activation_code(activation)       # the kernels apply it by its code; an unknown name is refused here
+        except ops.KernelError as e:
+            raise ValueError(f"{prefix}: {e}") from None
+        self.prefix, self.hidden, self.intermediate, self.activation = prefix, hidden, intermediate, activation
         self.w_gate_up = self.w_down = None
         self.p_gate_up = self.p_down = None   # copies in fragment order for single tokens
         self.paired = False      # gate and up rows in turns of 16: the activation runs inside the product
@@ -51,9 +53,9 @@ class GatedMlp(FeedForward):
         m = torch.empty((h.shape[0], self.intermediate), dtype=h.dtype, device=h.device)
         if self.paired and h.dtype == torch.bfloat16:
             if self.p_gate_up is not None and h.shape[0] <= ops.PACKED_MAX_ROWS:
-                ops.gemm_packed(h, self.p_gate_up, m, paired=True)
+                ops.gemm_packed(h, self.p_gate_up, m, paired=True, activation=self.activation)
             else:
-                ops.gemm_swiglu(h, self.w_gate_up, m)
+                ops.gemm_swiglu(h, self.w_gate_up, m, self.activation)
         else:
-            ops.swiglu(linear(h, self.w_gate_up, h.dtype), m)
+            ops.swiglu(linear(h, self.w_gate_up, h.dtype), m, self.activation)
         return linear_for_sum(m, self.w_down, self.p_down)

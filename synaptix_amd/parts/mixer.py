@@ -39,13 +39,14 @@ class Mixer(Part):
 class GqaAttention(Mixer):
     def __init__(self, prefix: str, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, *,
                  position: Position | None = None, qk_norm_eps: float | None = None, scale: float | None = None,
-                 window: int | None = None):
+                 window: int | None = None, qk_gain_offset: float = 0.0):
         if n_kv_heads <= 0 or n_heads % n_kv_heads:
             raise ValueError(f"{n_heads} heads do not divide into {n_kv_heads} kv heads")
         self.prefix = prefix
         self.hidden, self.nh, self.nkv, self.hd = hidden, n_heads, n_kv_heads, head_dim
         self.position = position or NoPosition()
         self.qk_norm_eps = qk_norm_eps
+        self.qk_gain_offset = float(qk_gain_offset)     # the q/k gains are this + their tensors
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
         self.window = window
         self.w_qkv = self.w_o = self.q_gain = self.k_gain = None
@@ -106,12 +107,13 @@ class GqaAttention(Mixer):
             work = ctx.scratch("attention_decode", N * nh * splits * (hd + 2))
             ops.attention_decode_fused_bf16(qkv, cache.k_pages, cache.v_pages, table, ctx.seq_len, o, work, splits,
                                             self.scale, window, nh, nkv, hd, self.q_gain, self.k_gain,
-                                            self.qk_norm_eps or 0.0, cos, sin, write_kv=owner)
+                                            self.qk_norm_eps or 0.0, cos, sin, write_kv=owner,
+                                            gain_offset=self.qk_gain_offset)
             return linear_for_sum(o, self.w_o, self.p_o)
         q = torch.empty((N, nh * hd), dtype=act, device=h.device)
         ops.qk_norm_rope_kv_write(qkv, q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos,
                                   self.q_gain, self.k_gain, self.qk_norm_eps or 0.0, cos, sin, nh, nkv, hd,
-                                  write_kv=owner)
+                                  write_kv=owner, gain_offset=self.qk_gain_offset)
         if act == torch.float32:
             ops.attention_f32(q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos, o, self.scale, window,
                               nh, nkv, hd)

@@ -16,10 +16,13 @@ from .base import Part
 
 
 class RmsNorm(Part):
-    def __init__(self, name: str, dim: int, eps: float):
+    def __init__(self, name: str, dim: int, eps: float, gain_offset: float = 0.0):
+        """gain_offset: the gain is gain_offset + the stored tensor (0 here; 1 for checkpoints that store
+        the gain as a difference from one, crates/synaptix-models/llm/common/src/config.rs:1-5)."""
         self.name = name          # full tensor name of the gain
         self.dim = dim
         self.eps = float(eps)
+        self.gain_offset = float(gain_offset)
         self.gain = None
 
     def tensor_specs(self):
@@ -33,11 +36,11 @@ class RmsNorm(Part):
         normed; with rows [n] int32 only those rows of resid + delta are normed and resid is kept."""
         n = resid.shape[0] if rows is None else rows.shape[0]
         out = torch.empty((n, self.dim), dtype=out_dtype, device=resid.device)
-        ops.add_rmsnorm(resid, delta, self.gain, self.eps, out, rows)
+        ops.add_rmsnorm(resid, delta, self.gain, self.eps, out, rows, self.gain_offset)
         return out
 
     def apply(self, x):
         """Norm over the last axis of a tensor in the activation type."""
         out = torch.empty_like(x)
-        ops.rmsnorm_rows(x, self.gain, self.eps, out)
+        ops.rmsnorm_rows(x, self.gain, self.eps, out, self.gain_offset)
         return out

@@ -22,7 +22,7 @@ def embed(table, ids, resid):
     resid.copy_(table[ids.long()].to(F32))
 
 
-def add_rmsnorm(resid, delta, gain, eps, out, rows=None):
+def add_rmsnorm(resid, delta, gain, eps, out, rows=None, gain_offset=0.0):
     if delta is not None and delta.dim() == 3:
         delta = delta.sum(0)
     if rows is None:
@@ -34,16 +34,17 @@ def add_rmsnorm(resid, delta, gain, eps, out, rows=None):
         if delta is not None:
             x = x + delta[rows.long()]
     inv = torch.rsqrt((x * x).mean(-1, keepdim=True) + eps)
-    out.copy_((gain.to(F32) * x * inv).to(out.dtype))
+    out.copy_(((gain_offset + gain.to(F32)) * x * inv).to(out.dtype))
 
 
-def rmsnorm_rows(x, gain, eps, out):
+def rmsnorm_rows(x, gain, eps, out, gain_offset=0.0):
     xf = x.to(F32)
     inv = torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps)
-    out.copy_((gain.to(F32) * xf * inv).to(out.dtype))
+    out.copy_(((gain_offset + gain.to(F32)) * xf * inv).to(out.dtype))
 
 
-def swiglu(gate_up, out):
+def swiglu(gate_up, out, activation="silu"):
+    assert activation in ("silu", "swish")
     I = gate_up.shape[1] // 2
     g, u = gate_up[:, :I].to(F32), gate_up[:, I:].to(F32)
     out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
@@ -62,7 +63,8 @@ def gemm(x, w, out, force_simt=False):
 PAIR = 16
 
 
-def gemm_swiglu(x, w_paired, out):
+def gemm_swiglu(x, w_paired, out, activation="silu"):
+    assert activation in ("silu", "swish")
     N, K = w_paired.shape
     w = w_paired.view(N // (2 * PAIR), 2, PAIR, K)
     g = x.to(F32) @ w[:, 0].reshape(N // 2, K).to(F32).T
@@ -70,7 +72,7 @@ def gemm_swiglu(x, w_paired, out):
     out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
 
 
-def gemm_packed(x, wp, out, paired=False):
+def gemm_packed(x, wp, out, paired=False, activation="silu"):
     from synaptix_amd.kernels import ops
     w = ops.unpack_weight(wp)
     if paired:
@@ -89,7 +91,7 @@ def gemm_slices(M, N, K, dtype):
 
 
 def qk_norm_rope_kv_write(qkv, q_out, k_pages, v_pages, page_table, tok_seq, tok_pos, q_gain, k_gain, eps,
-                          cos, sin, n_heads, n_kv_heads, head_dim, write_kv=True):
+                          cos, sin, n_heads, n_kv_heads, head_dim, write_kv=True, gain_offset=0.0):
     nh, nkv, hd = n_heads, n_kv_heads, head_dim
     if qkv.dim() == 3:                      # partial sums over slices of K
         qkv = qkv.sum(0)
@@ -100,7 +102,7 @@ def qk_norm_rope_kv_write(qkv, q_out, k_pages, v_pages, page_table, tok_seq, tok
     def norm(t, g):
         if g is None:
             return t
-        return g.to(F32) * t * torch.rsqrt((t * t).mean(-1, keepdim=True) + eps)
+        return (gain_offset + g.to(F32)) * t * torch.rsqrt((t * t).mean(-1, keepdim=True) + eps)
 
     def rope(t):
         if cos is None:
@@ -172,13 +174,14 @@ def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspa
 
 
 def attention_decode_fused_bf16(qkv, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
-                                n_heads, n_kv_heads, head_dim, q_gain, k_gain, eps, cos, sin, write_kv=True):
+                                n_heads, n_kv_heads, head_dim, q_gain, k_gain, eps, cos, sin, write_kv=True,
+                                gain_offset=0.0):
     B = qkv.shape[-2]
     q = torch.empty((B, n_heads * head_dim), dtype=torch.bfloat16)
     tok_seq = torch.arange(B, dtype=torch.int32)
     tok_pos = (seq_len - 1).to(torch.int32)
     qk_norm_rope_kv_write(qkv, q, k_pages, v_pages, page_table, tok_seq, tok_pos, q_gain, k_gain, eps, cos, sin,
-                          n_heads, n_kv_heads, head_dim, write_kv=write_kv)
+                          n_heads, n_kv_heads, head_dim, write_kv=write_kv, gain_offset=gain_offset)
     attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
                           n_heads, n_kv_heads, head_dim)
 

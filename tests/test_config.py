@@ -78,3 +78,10 @@ def test_eps_and_theta_are_held_as_32_bit():
     import numpy as np
     cfg = Qwen3Config.from_dict({**TINY_A, "rms_norm_eps": 1e-6})
     assert cfg.eps_f32 == float(np.float32(1e-6)) != 1e-6
+
+
+def test_a_feed_forward_names_its_activation_and_refuses_one_without_a_kernel():
+    from synaptix_amd.parts import GatedMlp
+    assert GatedMlp("x.", 64, 128, "silu").activation == "silu"
+    with pytest.raises(ValueError, match="activation 'gelu_pytorch_tanh'"):
+        GatedMlp("x.", 64, 128, "gelu_pytorch_tanh")

@@ -278,7 +278,7 @@ def test_a_captured_step_keeps_its_own_scratch_memory():
     where it is, and its replays must still give the eager results."""
     name, dtype = "C", "bfloat16"
     V = CONFIGS[name]["vocab_size"]
-    eng = make_engine(name, dtype, 64 * 80)
+    eng = make_engine(name, dtype, 64 * 100)
     eager = make_engine(name, dtype, 1024)
     prompt = random_tokens(V, 300, 77)
     s, e = eng.acquire(), eager.acquire()

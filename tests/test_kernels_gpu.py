@@ -76,6 +76,72 @@ def test_add_rmsnorm(ops, out_dtype, gain_dtype, N, H):
     close(out2, want2, 1e-5 if out_dtype == F32 else 2e-2, 1e-5 if out_dtype == F32 else 1e-2, "gathered rows")
 
 
+def test_norm_gains_stored_as_a_difference_from_one(ops):
+    """gain_offset = 1: the gain is 1 + w in every kernel that norms (rows with the residual sum, rows of any
+    width, the q/k heads of prompts in both of their kernels, the q/k heads inside decode attention)."""
+    eps = 1e-5
+    for H, dt in ((72, F32), (4096, BF16)):
+        resid, delta = rnd((3, H), 2), rnd((3, H), 3)
+        w = (0.1 * rnd((H,), 4)).to(dt)
+        want = torch.empty((3, H), dtype=F32)
+        ref.add_rmsnorm(resid.clone(), delta, 1 + w.float(), eps, want)
+        got = torch.empty((3, H), dtype=F32, device=DEV)
+        ops.add_rmsnorm(resid.to(DEV), delta.to(DEV), w.to(DEV), eps, got, gain_offset=1.0)
+        close(got, want, 1e-5, 1e-5, "add_rmsnorm with 1 + w")
+        x = rnd((5, H), 5)
+        ref.rmsnorm_rows(x, 1 + w.float(), eps, want2 := torch.empty((5, H)))
+        got2 = torch.empty((5, H), dtype=F32, device=DEV)
+        ops.rmsnorm_rows(x.to(DEV), w.to(DEV), eps, got2, gain_offset=1.0)
+        close(got2, want2, 1e-5, 1e-5, "rmsnorm_rows with 1 + w")
+    # q/k heads: head size 128 takes the 16-byte kernel, 48 the general one
+    for nh, nkv, hd in ((4, 2, 128), (6, 2, 48)):
+        N, width = 5, (nh + 2 * nkv) * hd
+        table = torch.arange(2, dtype=I32).view(1, 2)
+        tok_seq, tok_pos = torch.zeros(N, dtype=I32), torch.arange(60, 60 + N, dtype=I32)
+        qkv = rnd((N, width), 6, BF16)
+        qg, kg = (0.2 * rnd((hd,), 7)).to(BF16), (0.2 * rnd((hd,), 8)).to(BF16)
+        ang = torch.arange(80, dtype=F32)[:, None] * (0.3 / (1 + torch.arange(hd // 2, dtype=F32)))[None, :]
+        cos, sin = torch.cos(ang), torch.sin(ang)
+        k_ref, v_ref = torch.zeros((2, nkv, 64, hd), dtype=BF16), torch.zeros((2, nkv, hd, 64), dtype=BF16)
+        q_ref = torch.empty((N, nh * hd), dtype=BF16)
+        ref.qk_norm_rope_kv_write(qkv, q_ref, k_ref, v_ref, table, tok_seq, tok_pos, (1 + qg.float()), (1 + kg.float()),
+                                  eps, cos, sin, nh, nkv, hd)
+        d = lambda t: t.to(DEV)
+        kd, vd = torch.zeros_like(k_ref).to(DEV), dv(torch.zeros_like(v_ref))
+        q = torch.empty((N, nh * hd), dtype=BF16, device=DEV)
+        ops.qk_norm_rope_kv_write(d(qkv), q, kd, vd, d(table), d(tok_seq), d(tok_pos), d(qg), d(kg), eps, d(cos), d(sin),
+                                  nh, nkv, hd, gain_offset=1.0)
+        close(q, q_ref.float(), 2e-2, 1e-2, f"q heads of size {hd} with 1 + w")
+        close(kd, k_ref.float(), 2e-2, 1e-2, f"k heads of size {hd} with 1 + w")
+        # one more token through decode attention with the q/k/v intake
+        one = rnd((1, width), 9, BF16)
+        seq_len = torch.tensor([66], dtype=I32)
+        q1 = torch.empty((1, nh * hd), dtype=BF16)
+        ref.qk_norm_rope_kv_write(one, q1, k_ref, v_ref, table, torch.zeros(1, dtype=I32), seq_len - 1, 1 + qg.float(),
+                                  1 + kg.float(), eps, cos, sin, nh, nkv, hd)
+        want = torch.empty((1, nh * hd), dtype=F32)
+        ref.attention_f32(q1.float(), k_ref.float(), v_ref.float(), table, torch.zeros(1, dtype=I32), seq_len - 1, want,
+                          0.1, 0, nh, nkv, hd)
+        # positions 0..59 of the pages hold zeros: they take part in the softmax on both sides alike
+        out = torch.empty((1, nh * hd), dtype=BF16, device=DEV)
+        work = torch.empty(nh * 2 * (hd + 2), dtype=F32, device=DEV)
+        ops.attention_decode_fused_bf16(d(one), kd, vd, d(table), d(seq_len), out, work, 2, 0.1, 0, nh, nkv, hd, d(qg),
+                                        d(kg), eps, d(cos), d(sin), gain_offset=1.0)
+        close(out, want, 2e-2, 1e-2, f"decode attention, head size {hd}, gains 1 + w")
+
+
+def test_an_unknown_activation_is_refused_before_any_launch(ops):
+    x = torch.zeros((2, 64), dtype=BF16, device=DEV)
+    out = torch.zeros((2, 32), dtype=BF16, device=DEV)
+    with pytest.raises(Exception, match="activation 'gelu'"):
+        ops.swiglu(x, out, "gelu")
+    with pytest.raises(Exception, match="activation 'relu'"):
+        ops.gemm_swiglu(x, torch.zeros((64, 64), dtype=BF16, device=DEV), out, "relu")
+    from synaptix_amd.kernels.build import load_library
+    lib = load_library("core")
+    assert lib.syn_swiglu(None, None, 0, 2, 32, 7, None) != 0 and b"activation code 7" in lib.syn_last_error()
+
+
 def test_rmsnorm_eps_sits_inside_the_root(ops):
     # tiny x: sqrt(mean + eps) and sqrt(mean) + eps differ by orders of magnitude
     x = torch.full((1, 64), 1e-4)
