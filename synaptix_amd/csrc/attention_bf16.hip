@@ -26,7 +26,10 @@
 //            A second kernel merges the splits when there is more than one.
 // Reference counterparts: flash_splitq.cu (prefill), flash_decode.cu:92-205,340-387 (split + merge,
 // one block a q-head there, scalar dot products).
+#include <mutex>
+
 #include "common.h"
+#include "no_alloc.h"
 
 #ifndef SYN_HD
 #error "compile with -DSYN_HD=<head size>"
@@ -845,6 +848,45 @@ SYN_EXPORT int syn_attention_decode_bf16(const void* q, const void* k_pages, con
                                          int nkv, int hd, hipStream_t stream) {
   return launch_decode(q, nullptr, (void*)k_pages, (void*)v_pages, page_table, table_stride, seq_len, n_seqs, out,
                        workspace, n_splits, scale, window, nh, nkv, hd, stream);
+}
+
+// ---- the same without a workspace argument: see no_alloc.h ----
+// `scratch` is a device array; in host code its name is only a handle for hipGetSymbolAddress, never
+// an address to hand to a kernel.  Each GPU holds its own copy at its own address: the address is
+// looked up once per device, with that device current, and kept.
+static __device__ __align__(256) unsigned char scratch[SYN_NOALLOC_SCRATCH_BYTES];
+#define SYN_NOALLOC_MAX_DEVICES 64
+static float* scratch_of_device[SYN_NOALLOC_MAX_DEVICES];
+static std::mutex scratch_lock;
+
+SYN_EXPORT int syn_attention_decode_bf16_noalloc(const void* q, const void* k_pages, const void* v_pages,
+                                                 const int* page_table, int table_stride, const int* seq_len,
+                                                 int n_seqs, void* out, int n_splits, float scale, int window, int nh,
+                                                 int nkv, int hd, hipStream_t stream) {
+  SYN_CHECK(n_seqs > 0 && nh > 0 && n_splits > 0 && hd > 0, "attention_decode_noalloc: empty input");
+  const unsigned long long need = (unsigned long long)n_seqs * nh * n_splits * (hd + 2) * sizeof(float);
+  SYN_CHECK(need <= SYN_NOALLOC_SCRATCH_BYTES,
+            "attention_decode_noalloc: %d sequences x %d heads x %d splits need %llu bytes of partial results, the "
+            "library keeps %u; use fewer splits or the entry point with a workspace argument",
+            n_seqs, nh, n_splits, need, (unsigned)SYN_NOALLOC_SCRATCH_BYTES);
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  SYN_CHECK(e == hipSuccess && dev >= 0 && dev < SYN_NOALLOC_MAX_DEVICES, "attention_decode_noalloc: no current device (%s)",
+            hipGetErrorString(e));
+  float* ws;
+  {
+    std::lock_guard<std::mutex> hold(scratch_lock);
+    if (scratch_of_device[dev] == nullptr) {
+      void* p = nullptr;
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      SYN_CHECK(e == hipSuccess && p != nullptr, "attention_decode_noalloc: the scratch array has no address on device %d: %s",
+                dev, hipGetErrorString(e));
+      scratch_of_device[dev] = (float*)p;
+    }
+    ws = scratch_of_device[dev];
+  }
+  return launch_decode(q, nullptr, (void*)k_pages, (void*)v_pages, page_table, table_stride, seq_len, n_seqs, out, ws,
+                       n_splits, scale, window, nh, nkv, hd, stream);
 }
 
 // The same for one new token a sequence whose q, k and v come straight from the fused projection:

@@ -31,7 +31,7 @@ HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden"]
 CORE_SOURCES = ["elementwise.hip", "sampling.hip", "gemm.hip", "attention_f32.hip", "probes.hip"]
 RUNTIME_SOURCES = ["runtime.cpp"]
 ATTN_SOURCE = "attention_bf16.hip"
-HEADERS = ["common.h"]
+HEADERS = ["common.h", "no_alloc.h"]
 
 
 class KernelBuildError(RuntimeError):
