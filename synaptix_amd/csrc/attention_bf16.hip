@@ -126,33 +126,39 @@ constexpr int LDV = SYN_PAGE + 8;
 constexpr int PF_TILE = SYN_PAGE * LDK + HD * LDV;          // bf16 elements of one buffer
 constexpr int PF_CHUNKS = (8 * HD + PF_THREADS - 1) / PF_THREADS;  // 16-byte chunks a thread moves for K (and for V)
 
+// Which sequence and which 128 query rows workgroup blockIdx.y takes: tiles are numbered sequence by
+// sequence.  Two workgroups share a compute unit, and a tile's work grows with its number: the first
+// half of the grid takes the tiles from the last downwards, the second half from the first upwards,
+// so that the pairs that meet on a unit have about equal work.  False: the grid is an upper bound.
+__device__ __forceinline__ bool prefill_tile(const int* __restrict__ seq_start, int n_seqs, int& seq, int& q0) {
+  int total = 0;
+  for (int s = 0; s < n_seqs; ++s) total += (seq_start[s + 1] - seq_start[s] + PF_ROWS - 1) / PF_ROWS;
+  const int y = blockIdx.y, half = (total + 1) / 2;
+  if (y >= total) return false;
+  const int tile = y < half ? total - 1 - y : y - half;
+  int t_acc = 0;
+  for (int s = 0; s < n_seqs; ++s) {
+    const int nt = (seq_start[s + 1] - seq_start[s] + PF_ROWS - 1) / PF_ROWS;
+    if (tile < t_acc + nt) {
+      seq = s;
+      q0 = (tile - t_acc) * PF_ROWS;
+      return true;
+    }
+    t_acc += nt;
+  }
+  return false;
+}
+
 __global__ void __launch_bounds__(PF_THREADS)
 attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
                     const int* __restrict__ page_table, int table_stride, const int* __restrict__ seq_start,
                     const int* __restrict__ seq_past, int n_seqs, bf16* __restrict__ out, float scale,
                     int window, int nh, int nkv) {
   extern __shared__ __attribute__((aligned(16))) bf16 lds[];  // [2][PF_TILE]
-  // which sequence and which rows: tiles are numbered sequence by sequence.  Heads run fastest through
-  // the grid; workgroups go round the eight dies in turn, and the heads are dealt so that each die gets
-  // neighbouring heads, which share their K and V.  Two workgroups share a compute unit, and a tile's
-  // work grows with its number: the first half of the grid takes the tiles from the last downwards,
-  // the second half from the first upwards, so that the pairs that meet on a unit have about equal work.
-  int total = 0;
-  for (int s = 0; s < n_seqs; ++s) total += (seq_start[s + 1] - seq_start[s] + PF_ROWS - 1) / PF_ROWS;
-  const int y = blockIdx.y, half = (total + 1) / 2;
-  if (y >= total) return;  // the grid is an upper bound
-  const int tile = y < half ? total - 1 - y : y - half;
-  int seq = -1, q0 = 0, t_acc = 0;
-  for (int s = 0; s < n_seqs; ++s) {
-    const int nt = (seq_start[s + 1] - seq_start[s] + PF_ROWS - 1) / PF_ROWS;
-    if (tile < t_acc + nt) {
-      seq = s;
-      q0 = (tile - t_acc) * PF_ROWS;
-      break;
-    }
-    t_acc += nt;
-  }
-  if (seq < 0) return;
+  // Heads run fastest through the grid; workgroups go round the eight dies in turn, and the heads are
+  // dealt so that each die gets neighbouring heads, which share their K and V.
+  int seq, q0;
+  if (!prefill_tile(seq_start, n_seqs, seq, q0)) return;
   const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE;
   const int r16 = lane % 16, g4 = lane / 16;
   const int hx = blockIdx.x;
@@ -329,10 +335,230 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages
   }
 }
 
+// ------------------------------------------------------------------ prefill, 32 query rows a wave
+// The same tiles of 128 query rows with v_mfma_f32_32x32x16_bf16 for both products, for head sizes 64
+// and 128: a workgroup of four waves, each with 32 query rows.  A fragment of K or V read from LDS (1 KB)
+// then feeds a product of 32 x 32 x 16 instead of 16 x 16 x 32: half the LDS reads for the same work,
+// which is what bounded the waves of 16 rows (one fragment read for every MFMA).
+//   A[i = lane % 32][k = 8 (lane / 32) + e], B[k = 8 (lane / 32) + e][n = lane % 32],
+//   D[i = 8 (e / 4) + 4 (lane / 32) + e % 4][n = lane % 32], e = 0 .. 15
+// S^T = K . Q^T in two tiles of 32 keys; row m of a tile stands for key pf2_row_key(m), chosen so that a
+// lane's accumulator values e = 8j .. 8j + 7 are the 8 consecutive keys 16 j + 8 (lane / 32) .. + 7: they
+// are, rounded to bf16, the B operand of O^T += V^T . P^T for k-step j, and the matching V^T fragment is
+// one 16-byte piece of the page as it lies in memory.  Both K and V blocks therefore go into LDS as they
+// are, by loads that write LDS directly (no registers, no store instructions): V verbatim (a fragment
+// read covers runs of 256 consecutive bytes), K with the 16-byte chunks of each row swizzled, since its
+// fragment reads touch 32 rows at the same column.
+constexpr bool PF2_OK = HD == 64 || HD == 128;
+constexpr int PF2_WAVES = 4;
+constexpr int PF2_THREADS = PF2_WAVES * SYN_WAVE;
+constexpr int PF2_KBYTES = SYN_PAGE * HD * 2;   // a block of K; a block of V is as large
+constexpr int PF2_BUF = 2 * PF2_KBYTES;         // one buffer: K, then V
+constexpr int PF2_CPR = HD / 8;                 // 16-byte chunks in a row of K
+constexpr int PF2_KS = HD / 16;                 // k-steps of the scores
+constexpr int PF2_AHEAD = 6;                    // fragment reads on their way ahead of the MFMA that takes them
+constexpr int PF2_DT = HD >= 32 ? HD / 32 : 1;  // tiles of 32 output dims (the kernel is compiled for every head size, launched for two)
+static_assert(PF_ROWS == PF2_WAVES * 32, "both prefill kernels take tiles of the same number of rows");
+
+__device__ __forceinline__ int pf2_swizzle(int row) { return PF2_CPR == 16 ? (row & 15) : ((row >> 1) & 7); }
+__device__ __forceinline__ int pf2_row_key(int m) { return 16 * (m / 16) + 8 * ((m % 8) / 4) + 4 * ((m % 16) / 8) + m % 4; }
+
+__global__ void __launch_bounds__(PF2_THREADS, 2)
+attn_prefill32_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
+                      const int* __restrict__ page_table, int table_stride, const int* __restrict__ seq_start,
+                      const int* __restrict__ seq_past, int n_seqs, bf16* __restrict__ out, float scale,
+                      int window, int nh, int nkv) {
+  extern __shared__ __attribute__((aligned(16))) char lds2[];  // [2][K block | V block]
+  int seq, q0;
+  if (!prefill_tile(seq_start, n_seqs, seq, q0)) return;
+  const int tid = threadIdx.x, lane = tid % SYN_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / SYN_WAVE);
+  const int n32 = lane % 32, hh = lane / 32;
+  const int hx = blockIdx.x;
+  const int head = nh % 8 == 0 ? (hx % 8) * (nh / 8) + hx / 8 : hx, kvh = head / (nh / nkv);
+  const int tok0 = seq_start[seq], n_new = seq_start[seq + 1] - tok0, past = seq_past[seq];
+  const int kv_len = past + n_new;
+  const int r0 = q0 + wave * 32;
+  const bool wave_on = r0 < n_new;
+  const int row = r0 + n32;
+  const bool valid = row < n_new;
+  const int qpos = valid ? past + row : -1;
+  const int lo = (window > 0 && valid) ? max(0, qpos - window + 1) : 0;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  bf16x8 qf[PF2_KS];
+#pragma unroll
+  for (int ks = 0; ks < PF2_KS; ++ks)
+    qf[ks] = valid ? *(const bf16x8*)(q + ((size_t)(tok0 + row) * nh + head) * HD + 16 * ks + 8 * hh) : zero8;
+  // visible keys of this wave, and of the whole workgroup
+  const int w_kmax = past + min(r0 + 31, n_new - 1);
+  const int w_qmin = past + r0;
+  const int w_kmin = window > 0 ? max(0, w_qmin - window + 1) : 0;
+  const int g_kmax = past + min(q0 + PF_ROWS - 1, n_new - 1);
+  const int g_kmin = window > 0 ? max(0, past + q0 - window + 1) : 0;
+  const int kb_lo = g_kmin / SYN_PAGE, kb_hi = g_kmax / SYN_PAGE;
+  const float scale2 = scale * 1.44269504088896340736f;   // > 0: the host sends other scales to the other kernel
+
+  f32x16 o[PF2_DT];
+#pragma unroll
+  for (int d = 0; d < PF2_DT; ++d)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o[d][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  auto fetch = [&](int kb, int buf) {
+    const size_t base =
+        ((size_t)__builtin_amdgcn_readfirstlane(page_table[(size_t)seq * table_stride + kb]) * nkv + kvh) * SYN_PAGE * HD;
+    const BufferView vk = buffer_view(k_pages + base, PF2_KBYTES), vv = buffer_view(v_pages + base, PF2_KBYTES);
+    char* dst = lds2 + buf * PF2_BUF;
+#pragma unroll
+    for (int it = 0; it < PF2_KBYTES / 1024 / PF2_WAVES; ++it) {
+      const int i = it * PF2_WAVES + wave;                 // which 1 KB of the block this wave's load fills
+      const int at = 64 * i + lane, krow = at / PF2_CPR, slot = at % PF2_CPR;
+      buffer_to_lds16(vk, dst + 1024 * i, (unsigned)((krow * PF2_CPR + (slot ^ pf2_swizzle(krow))) * 16), 0);
+      buffer_to_lds16(vv, dst + PF2_KBYTES + 1024 * i, (unsigned)(at * 16), 0);
+    }
+  };
+  auto landed = [&]() {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's loads have written LDS; behind the barrier all have
+    __syncthreads();
+  };
+
+  fetch(kb_lo, 0);
+  landed();
+  for (int kb = kb_lo; kb <= kb_hi; ++kb) {
+    const int buf = (kb - kb_lo) & 1;
+    if (kb < kb_hi) fetch(kb + 1, buf ^ 1);   // that buffer was last read before the previous barrier
+    const int key0 = kb * SYN_PAGE;
+    char* ks_ = lds2 + buf * PF2_BUF;
+    char* vs_ = ks_ + PF2_KBYTES;
+    if (key0 + SYN_PAGE > kv_len) {
+      // the sequence ends inside this block: whatever lies behind its end in the page is made zero, so
+      // that 0 * (that) is 0.  Chunk c holds tokens 32 h + 8 g .. + 7 of one dim, c = (h * DT + dt) * 64 + 16 g + r.
+      for (int c = tid; c < 8 * HD; c += PF2_THREADS) {
+        const int tok = 32 * (c / (64 * DT)) + 8 * ((c % 64) / 16);
+        if (key0 + tok + 8 > kv_len) {
+          bf16x8 v = *(bf16x8*)(vs_ + c * 16);
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (key0 + tok + e >= kv_len) v[e] = (bf16)0.f;
+          *(bf16x8*)(vs_ + c * 16) = v;
+        }
+      }
+      __syncthreads();
+    }
+    if (wave_on && key0 <= w_kmax && key0 + SYN_PAGE > w_kmin) {
+      // Fragment reads from LDS take longer than an MFMA: PF2_AHEAD of them are on their way before the
+      // first product needs one, then one read follows each MFMA.  The first V fragments are requested
+      // before the softmax, so that they arrive while its maxima are taken.
+      constexpr int NQK = 2 * PF2_KS, NPV = 4 * PF2_DT;
+      constexpr int AHEAD = NQK < PF2_AHEAD ? NQK : PF2_AHEAD, VAHEAD = NPV < PF2_AHEAD ? NPV : PF2_AHEAD;
+      f32x16 s[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s[t][e] = 0.f;
+      const int krow0 = pf2_row_key(n32), sw0 = pf2_swizzle(krow0), sw1 = pf2_swizzle(32 + krow0);
+      auto k_frag = [&](int i) {   // read i: k-step i / 2 of score tile i % 2
+        const int t = i % 2, ks = i / 2;
+        return *(const bf16x8*)(ks_ + ((32 * t + krow0) * PF2_CPR + ((2 * ks + hh) ^ (t ? sw1 : sw0))) * 16);
+      };
+      auto v_frag = [&](int i) {   // read i: output tile i % PF2_DT of k-step i / PF2_DT = 2 t + j
+        const int d = i % PF2_DT, tj = i / PF2_DT, t = tj / 2, j = tj % 2;
+        return *(const bf16x8*)(vs_ + (((t * DT + 2 * d + n32 / 16) * 64 + (2 * j + hh) * 16 + n32 % 16)) * 16);
+      };
+      bf16x8 kf[NQK], vf[NPV];
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < AHEAD; ++i) kf[i] = k_frag(i);
+#pragma unroll
+      for (int i = 0; i < NQK; ++i) {
+        s[i % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], qf[i / 2], s[i % 2], 0, 0, 0);
+        if (i + AHEAD < NQK) kf[i + AHEAD] = k_frag(i + AHEAD);
+        else if (i + AHEAD - NQK < VAHEAD) vf[i + AHEAD - NQK] = v_frag(i + AHEAD - NQK);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
+#pragma unroll
+      for (int i = 0; i < NQK; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA,
+        if (i + AHEAD < NQK || i + AHEAD - NQK < VAHEAD) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one read behind it
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // a block needs masking if some row of the wave does not see all of it
+      const bool need_mask = key0 + SYN_PAGE - 1 > w_qmin || (window > 0 && key0 < w_kmax - window + 1) || r0 + 32 > n_new;
+      if (need_mask) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int key = key0 + 32 * t + 16 * (e / 8) + 8 * hh + e % 8;
+            if (key > qpos || key < lo) s[t][e] = -INFINITY;
+          }
+      }
+      float mloc = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mloc = fmaxf(mloc, s[t][e]);
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 32, SYN_WAVE)) * scale2;
+      // m_run is the reference of the exponents, not the exact maximum: it is only raised when a block
+      // exceeds it by more than RESCALE_AT (in log2 units), so that the accumulators are rescaled in few blocks
+      const bool raise = mloc > m_run + RESCALE_AT || (m_run == -INFINITY && mloc > -INFINITY);
+      if (__any(raise)) {
+        const float m_new = raise ? mloc : m_run;
+        const float alpha = raise ? __builtin_amdgcn_exp2f(m_run - m_new) : 1.f;  // from -inf: 0
+        m_run = m_new;
+        l_run *= alpha;
+#pragma unroll
+        for (int d = 0; d < PF2_DT; ++d) o[d] *= alpha;
+      }
+      const float neg_m = m_run == -INFINITY ? 0.f : -m_run;  // a column that has seen no key yet
+      float lsum = 0.f;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int tj = 0; tj < 4; ++tj) {
+        bf16x8 pb;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float p = __builtin_amdgcn_exp2f(fmaf(s[tj / 2][8 * (tj % 2) + e], scale2, neg_m));   // a masked score: 2^-inf = 0
+          lsum += p;
+          pb[e] = (bf16)p;
+        }
+#pragma unroll
+        for (int d = 0; d < PF2_DT; ++d) {
+          const int i = tj * PF2_DT + d;
+          o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[i], pb, o[d], 0, 0, 0);
+          if (i + VAHEAD < NPV) vf[i + VAHEAD] = v_frag(i + VAHEAD);
+        }
+      }
+      l_run += lsum;
+    }
+    landed();
+  }
+  if (!wave_on) return;
+  float l = l_run + __shfl_xor(l_run, 32, SYN_WAVE);
+  if (!valid) return;
+  const float inv = 1.f / l;
+  bf16* orow = out + ((size_t)(tok0 + row) * nh + head) * HD + 4 * hh;
+#pragma unroll
+  for (int d = 0; d < PF2_DT; ++d)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      bf16x4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = (bf16)(o[d][4 * b + e] * inv);
+      *(bf16x4*)(orow + 32 * d + 8 * b) = v;
+    }
+}
+
 SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, const void* v_pages,
                                           const int* page_table, int table_stride, const int* seq_start,
                                           const int* seq_past, int n_seqs, int n_tokens, void* out, float scale,
-                                          int window, int nh, int nkv, int hd, hipStream_t stream) {
+                                          int window, int nh, int nkv, int hd, int variant, hipStream_t stream) {
+  // variant: 0 = whichever is faster for this head size, 1 = waves of 16 query rows (every head size),
+  // 2 = waves of 32 query rows (head sizes 64 and 128, a positive scale)
+  SYN_CHECK(variant >= 0 && variant <= 2, "attention_prefill: unknown variant %d", variant);
+  SYN_CHECK(variant != 2 || (PF2_OK && scale > 0.f), "attention_prefill: waves of 32 rows take head sizes 64 and 128 and "
+            "a positive scale (head size %d, scale %g)", HD, (double)scale);
   SYN_CHECK(hd == HD, "attention_prefill: library built for head size %d, called with %d", HD, hd);
   SYN_CHECK(n_seqs > 0 && n_tokens >= n_seqs && nh > 0 && nkv > 0, "attention_prefill: empty input");
   SYN_CHECK(nh % nkv == 0, "attention_prefill: %d heads do not divide into %d kv heads", nh, nkv);
@@ -345,6 +571,15 @@ SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, co
                                        (int)lds);
     SYN_CHECK(e == hipSuccess, "attention_prefill: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
     raised = true;
+  }
+  if constexpr (PF2_OK) {
+    if (variant == 2 || (variant == 0 && scale > 0.f)) {
+      attn_prefill32_kernel<<<dim3(nh, tiles), PF2_THREADS, 2 * PF2_BUF, stream>>>(
+          (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, page_table, table_stride, seq_start, seq_past,
+          n_seqs, (bf16*)out, scale, window, nh, nkv);
+      SYN_LAUNCH_CHECK("attention_prefill32");
+      return 0;
+    }
   }
   attn_prefill_kernel<<<dim3(nh, tiles), PF_THREADS, lds, stream>>>(
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, page_table, table_stride, seq_start, seq_past, n_seqs,

@@ -364,9 +364,11 @@ def _attn_lib(hd):
 
 
 def attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, seq_past, out, scale, window, n_heads,
-                           n_kv_heads, head_dim):
+                           n_kv_heads, head_dim, variant=0):
     """Causal attention of the new tokens of each sequence over its cache (which already holds them).
-    seq_start [B+1]: offsets of the sequences' new tokens in q; seq_past [B]: tokens cached before."""
+    seq_start [B+1]: offsets of the sequences' new tokens in q; seq_past [B]: tokens cached before.
+    variant: 0 = the kernel's own choice, 1 = waves of 16 query rows (every head size), 2 = waves of 32
+    query rows (head sizes 64 and 128); for comparisons."""
     nh, nkv, hd = n_heads, n_kv_heads, head_dim
     _need(q, "attention_prefill.q", _BF16, (None, nh * hd))
     N = q.shape[0]
@@ -380,7 +382,7 @@ def attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, seq_past,
     _need(out, "attention_prefill.out", _BF16, (N, nh * hd))
     _call(_attn_lib(hd), "syn_attention_prefill_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
           page_table.shape[1], _ptr(seq_start), _ptr(seq_past), B, N, _ptr(out), ctypes.c_float(scale),
-          int(window or 0), nh, nkv, hd, _stream())
+          int(window or 0), nh, nkv, hd, int(variant), _stream())
 
 
 def decode_splits(n_seqs, n_kv_heads, max_pages):

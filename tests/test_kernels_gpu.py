@@ -479,6 +479,8 @@ ATTN_SHAPES = [
     (8, 2, 64, [100, 64, 127], [70, 64, 2], 0),   # chunks of a prompt that start inside a page, at its edge, before its end
     (32, 8, 128, [100, 1000], [150, 130], 0),     # the same at the head size and group of the large models
     (6, 2, 48, [33], [300], 50),                  # a chunk over several pages with a window
+    (8, 4, 64, [5, 0, 190], [260, 129, 3], 70),   # head size 64 with a window, sequences that end inside pages
+    (16, 2, 128, [0, 77], [513, 200], 0),         # eight heads a group, several tiles of 128 rows
 ]
 
 
@@ -489,14 +491,15 @@ def test_attention_prefill(ops, dtype, nh, nkv, hd, past, new, window):
     lens = [p + n for p, n in zip(past, new)]
     width = max((T + 63) // 64 for T in lens) + 1
     table = shuffled_table(B, width, 3)
-    k, v = make_cache(B * width, nkv, hd, dtype, 30)
+    k, v = make_cache(B * width, nkv, hd, dtype, 30, fill="nan" if (hd == 64 and dtype == BF16) else "garbage")
     fill_sequences(k, v, table, lens, nkv, hd, dtype, 31)
     tok_seq, tok_pos, starts, past_t, len_t = step_arrays(past, new)
     N = len(tok_seq)
     q = rnd((N, nh * hd), 32, dtype)
     scale = 1 / math.sqrt(hd)
     want = torch.empty((N, nh * hd), dtype=F32)
-    ref.attention_f32(q.float(), k.float(), v.float(), table, tok_seq, tok_pos, want, scale, window, nh, nkv, hd)
+    ref.attention_f32(q.float(), torch.nan_to_num(k.float()), torch.nan_to_num(v.float()), table, tok_seq, tok_pos, want,
+                      scale, window, nh, nkv, hd)
     d = lambda t: t.to(DEV)
     out = torch.empty((N, nh * hd), dtype=dtype, device=DEV)
     if dtype == F32:
@@ -505,6 +508,17 @@ def test_attention_prefill(ops, dtype, nh, nkv, hd, past, new, window):
     else:
         ops.attention_prefill_bf16(d(q), d(k), dv(v), d(table), d(starts), d(past_t), out, scale, window, nh, nkv, hd)
         close(out, want, 2e-2, 1e-2, what="attention prefill bf16")
+        # both kernels where the head size allows both: waves of 16 and of 32 query rows
+        for variant in (1, 2):
+            out.fill_(float("nan"))
+            if variant == 2 and hd not in (64, 128):
+                with pytest.raises(Exception, match="waves of 32 rows"):
+                    ops.attention_prefill_bf16(d(q), d(k), dv(v), d(table), d(starts), d(past_t), out, scale, window,
+                                               nh, nkv, hd, variant=variant)
+                continue
+            ops.attention_prefill_bf16(d(q), d(k), dv(v), d(table), d(starts), d(past_t), out, scale, window, nh, nkv,
+                                       hd, variant=variant)
+            close(out, want, 2e-2, 1e-2, what=f"attention prefill bf16, variant {variant}")
 
 
 @pytest.mark.parametrize("nh,nkv,hd,lens,window,splits", [
