@@ -182,7 +182,7 @@ static void launch_skinny(const bf16* x, const bf16* w, void* out, Epilogue ep, 
 template <int TILES, int KWAVES, int U, bool PAIRED>
 __global__ void __launch_bounds__(TILES * KWAVES * SYN_WAVE)
 gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void* __restrict__ out, Epilogue ep,
-                   int M, int N, int K) {
+                   int M, int N, int K, int ks_slice) {
   static_assert(!PAIRED || TILES == 2, "a pair is two tiles");
   constexpr int WAVES = TILES * KWAVES;
   __shared__ float part[WAVES][4][64];
@@ -197,12 +197,15 @@ gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void
   const bool xok = r16 < M;
   const bf16* xrow = x + (size_t)min(r16, M - 1) * K + kq;
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  // blockIdx.y = which slice of K (ks_slice k-steps of 32) this workgroup sums; its output is slice blockIdx.y
+  // of a float [slices, M, N] that the reader adds up (a product with few rows of W gets more workgroups so)
+  const int ks_begin = (int)blockIdx.y * ks_slice, ks_end = min(nks, ks_begin + ks_slice);
   if (tile_in) {
-    for (int ks0 = kw * U; ks0 < nks; ks0 += KWAVES * U) {
+    for (int ks0 = ks_begin + kw * U; ks0 < ks_end; ks0 += KWAVES * U) {
       bf16x8 bw[U], ax[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const bool in = ks0 + u < nks;
+        const bool in = ks0 + u < ks_end;
         bw[u] = in ? __builtin_nontemporal_load((const bf16x8*)(wt + (size_t)(ks0 + u) * 512)) : zero;
         ax[u] = (in && xok) ? *(const bf16x8*)(xrow + (ks0 + u) * 32) : zero;
       }
@@ -235,7 +238,7 @@ gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void
       if (m < M && n < N) {
         const float v = summed(t, j, ln);
         if (ep.out_is_f32)
-          ((float*)out)[(size_t)m * N + n] = v;
+          ((float*)out)[((size_t)blockIdx.y * M + m) * N + n] = v;
         else
           ((bf16*)out)[(size_t)m * N + n] = (bf16)v;
       }
@@ -245,10 +248,11 @@ gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void
 
 template <int TILES, int KWAVES, int U, bool PAIRED = false>
 static void launch_packed(const bf16* x, const bf16* wp, void* out, Epilogue ep, int M, int N, int K,
-                          hipStream_t stream) {
+                          hipStream_t stream, int slices = 1) {
   const int rows = TILES * 16;
+  const int ks_slice = (K / 32 + slices - 1) / slices;
   gemm_packed_kernel<TILES, KWAVES, U, PAIRED>
-      <<<(N + rows - 1) / rows, TILES * KWAVES * SYN_WAVE, 0, stream>>>(x, wp, out, ep, M, N, K);
+      <<<dim3((N + rows - 1) / rows, slices), TILES * KWAVES * SYN_WAVE, 0, stream>>>(x, wp, out, ep, M, N, K, ks_slice);
 }
 
 // ------------------------------------------------------------------ shared by the tiled kernels
@@ -890,10 +894,13 @@ SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, i
 
 // The products above for up to 16 rows of x over wp, a copy of W [N, K] in fragment order (see
 // gemm_packed_kernel; N a multiple of 16, K of 32).  out_code: 1 = bf16 [M, N], 2 = float [M, N];
-// paired: W holds gate and up rows in turns of 16 and out is bf16 [M, N / 2] = silu(gate) * up.
+// paired: W holds gate and up rows in turns of 16 and out is bf16 [M, N / 2] = act(gate) * up.
+// slices > 1 (float out, not paired): out is [slices, M, N], slice s holds the sum over its part of K.
 SYN_EXPORT int syn_gemm_packed(const void* x, const void* wp, void* out, int out_code, int M, int N, int K, int paired,
-                               int act, hipStream_t stream) {
+                               int act, int slices, hipStream_t stream) {
   SYN_CHECK(act >= 0 && act < SYN_ACT_COUNT, "gemm_packed: unknown activation code %d", act);
+  SYN_CHECK(slices >= 1 && slices <= 64 && (slices == 1 || (out_code == 2 && !paired)),
+            "gemm_packed: %d slices of K need a float output [slices, M, N] and no activation", slices);
   const Epilogue ep = {out_code == 2, act};
   SYN_CHECK(M > 0 && M <= 16 && N > 0 && K > 0, "gemm_packed: M = %d (1 .. 16), N = %d, K = %d", M, N, K);
   SYN_CHECK(N % 16 == 0 && K % 32 == 0 && (!paired || N % 32 == 0),
@@ -905,8 +912,8 @@ SYN_EXPORT int syn_gemm_packed(const void* x, const void* wp, void* out, int out
   const bf16* wb = (const bf16*)wp;
   // from sweeps at N = 4096 .. 151936, K = 4096 and 12288, 1 and 8 rows
   if (paired) launch_packed<2, 8, 4, true>(xb, wb, out, ep, M, N, K, stream);
-  else if (N <= 8192) launch_packed<1, 16, 2>(xb, wb, out, ep, M, N, K, stream);
-  else launch_packed<1, 8, 8>(xb, wb, out, ep, M, N, K, stream);
+  else if (N <= 8192) launch_packed<1, 16, 2>(xb, wb, out, ep, M, N, K, stream, slices);
+  else launch_packed<1, 8, 8>(xb, wb, out, ep, M, N, K, stream, slices);
   SYN_LAUNCH_CHECK("gemm_packed");
   return 0;
 }

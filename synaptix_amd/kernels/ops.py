@@ -224,7 +224,8 @@ def unpack_weight(wp):
 
 def gemm_packed(x, wp, out, paired=False, activation="silu"):
     """out[M, N] (bf16 or float) = x[M, K] . W^T for M <= 16 with wp = pack_weight(W); paired: W holds gate and
-    up rows in turns of 16 (pair_rows) and out [M, N / 2] bf16 = act(gate) * up."""
+    up rows in turns of 16 (pair_rows) and out [M, N / 2] bf16 = act(gate) * up.  A float out of shape
+    [S, M, N] receives S partial sums over slices of K instead."""
     _need(x, "gemm_packed.x", _BF16, (None, None))
     M, K = x.shape
     if K % 32:
@@ -233,12 +234,42 @@ def gemm_packed(x, wp, out, paired=False, activation="silu"):
     N = wp.shape[0] * 16
     if M > 16 or (paired and N % 32):
         raise KernelError(f"gemm_packed: M = {M} (at most 16), N = {N}")
+    slices = 1
     if paired:
         _need(out, "gemm_packed.out", _BF16, (M, N // 2))
+    elif out.dim() == 3:          # float partial sums over slices of K, which the reader adds
+        slices = out.shape[0]
+        _need(out, "gemm_packed.out", _F32, (slices, M, N))
     else:
         _need(out, "gemm_packed.out", (_BF16, _F32), (M, N))
     _call(load_library("core"), "syn_gemm_packed", _ptr(x), _ptr(wp), _ptr(out), 2 if out.dtype == _F32 else 1,
-          M, N, K, 1 if paired else 0, activation_code(activation), _stream())
+          M, N, K, 1 if paired else 0, activation_code(activation), slices, _stream())
+
+
+N_COMPUTE_UNITS = 256     # of the MI355X: what the rules below fill
+
+
+def packed_slices(N, K):
+    """Into how many slices of K gemm_packed is cut when its reader can add partial sums.  It has a workgroup
+    for every 16 rows of W, each with a fixed share of the weight stream; when their number is no
+    multiple of the compute units the last round runs half empty (N = 5120: 320 workgroups, two rounds for
+    the work of 1.25; N = 2560: 160 compute units of 256).  The smallest cut that fills its rounds to 90 %
+    is taken, if one exists among up to 8 slices of at least 1,024."""
+    groups = -(-N // 16)
+
+    def fill(s):
+        work = groups * s / N_COMPUTE_UNITS
+        return work / -(-groups * s // N_COMPUTE_UNITS)
+
+    best = 1
+    for s in (1, 2, 3, 4, 5, 6, 8):
+        if s > 1 and K // s < 1024:
+            break
+        if fill(s) >= 0.9:
+            return s
+        if fill(s) > fill(best) + 0.05:
+            best = s
+    return best
 
 
 def gemm_slices(M, N, K, dtype):

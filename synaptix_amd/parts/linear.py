@@ -54,7 +54,12 @@ def linear_for_sum(x, w, packed=None):
     into the next norm): [S, M, N] when cutting K into S slices gives a small product more
     workgroups, else [M, N]."""
     if _use_packed(x, packed):
-        return linear(x, w, torch.float32, packed)
+        slices = ops.packed_slices(w.shape[0], w.shape[1])
+        if slices <= 1:
+            return linear(x, w, torch.float32, packed)
+        out = torch.empty((slices, x.shape[0], w.shape[0]), dtype=torch.float32, device=x.device)
+        ops.gemm_packed(x, packed, out)
+        return out
     M, K = x.shape
     N = w.shape[0]
     slices = ops.gemm_slices(M, N, K, x.dtype) if w.dtype == x.dtype else 1

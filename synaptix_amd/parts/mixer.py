@@ -92,7 +92,9 @@ class GqaAttention(Mixer):
             raise ValueError(f"position {ctx.max_position} is beyond the position encoding's capacity {cap}")
         # single tokens: partial sums over slices of K, which the attention kernel adds; prompts: the plain product
         if self.p_qkv is not None and N <= ops.PACKED_MAX_ROWS and act == torch.bfloat16:
-            qkv = linear(h, self.w_qkv, torch.float32, self.p_qkv).unsqueeze(0)   # one float "partial sum"
+            qkv = linear_for_sum(h, self.w_qkv, self.p_qkv)       # float partial sums [S, N, width]
+            if qkv.dim() == 2:
+                qkv = qkv.unsqueeze(0)
         else:
             # (the kernels behind single tokens, and behind prompts of up to 64 tokens, add partial sums themselves)
             sliced = (N <= 64 or ctx.one_token_each) and ops.gemm_slices(N, self.w_qkv.shape[0], self.hidden, act) > 1

@@ -77,6 +77,11 @@ def gemm_packed(x, wp, out, paired=False, activation="silu"):
     w = ops.unpack_weight(wp)
     if paired:
         gemm_swiglu(x, w, out)
+    elif out.dim() == 3:                    # partial sums over slices of K (whole k-steps of 32)
+        S, K = out.shape[0], w.shape[1]
+        step = -(-(K // 32) // S) * 32
+        for i in range(S):
+            out[i] = x[:, i * step:(i + 1) * step].to(F32) @ w[:, i * step:(i + 1) * step].to(F32).T
     else:
         out.copy_((x.to(F32) @ w.to(F32).T).to(out.dtype))
 

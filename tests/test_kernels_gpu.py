@@ -297,6 +297,15 @@ def test_gemm_over_weights_in_fragment_order(ops, out_dtype, M, N, K):
     want = (x.double() @ w.double().T).float()
     atol = 1e-3 * math.sqrt(K)
     close(out, want, atol if out_dtype == F32 else atol + 0.02, 0 if out_dtype == F32 else 1e-2, f"packed {M}x{N}x{K}")
+    if out_dtype == F32:
+        # partial sums over slices of K: each slice its own part, the slices add up, also when the last ones are short or empty
+        for S in (2, 3, 7):
+            parts = torch.full((S, M, N), float("nan"), dtype=F32, device=DEV)
+            ops.gemm_packed(x.to(DEV), wp, parts)
+            close(parts.sum(0), want, atol, what=f"packed {M}x{N}x{K} in {S} slices")
+            step = -(-(K // 32) // S) * 32
+            first = (x[:, :step].double() @ w[:, :step].double().T).float()
+            close(parts[0], first, atol, what=f"first of {S} slices")
     assert ops.pack_weight(w[:N - 3].to(DEV)) is None and ops.pack_weight(w[:, :K - 8].to(DEV)) is None
     with pytest.raises(Exception, match="at most 16"):
         ops.gemm_packed(torch.zeros((17, K), dtype=BF16, device=DEV), wp, torch.empty((17, N), dtype=out_dtype, device=DEV))
@@ -355,6 +364,18 @@ def test_products_of_a_prompt_at_the_sizes_of_an_8b_layer(ops):
     rows, cols = _sampled(M, 6144, 400, 78)
     want = (x[rows].double() * wq[cols].double()).sum(1).float()
     close(q[rows.to(DEV), cols.to(DEV)], want, 0.02, 1e-2, "q/k/v at 8B sizes")
+
+
+def test_slices_fill_the_compute_units(ops):
+    """The host-side rule for the products over packed weights: one slice where the workgroups fill their
+    rounds, more where they would leave the last round half empty."""
+    assert ops.packed_slices(4096, 4096) == 1 and ops.packed_slices(151936, 4096) == 1
+    assert ops.packed_slices(5120, 25600) == 3 and ops.packed_slices(6144, 4096) == 2
+    assert ops.packed_slices(2560, 4096) == 3
+    assert ops.packed_slices(2560, 1024) == 1          # no slice shorter than 1,024
+    for N in range(16, 12000, 16):
+        s = ops.packed_slices(N, 8192)
+        assert 1 <= s <= 8
 
 
 def test_gemm_bf16_paths_agree(ops):
