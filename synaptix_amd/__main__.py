@@ -4,7 +4,7 @@ the same option names and meanings where this engine has the feature.
 
     python -m synaptix_amd run MODEL [PROMPT] [--prompt-file F | --prompt-ids 1,2,3 | --prompt-ids-file F]
            [--max-tokens 128] [--temperature 1.0] [--seed 0] [--device cuda] [--max-seq N]
-           [--compute-dtype bf16|f32] [--no-graph] [--warmup]
+           [--compute-dtype bf16|f32] [--no-graph] [--warmup] [--op-times]
     python -m synaptix_amd bench MODEL [--n-tokens 128] [--prompt-tokens 32] [--batch-size 1] [--warmup 3] [--dtype bf16]
     python -m synaptix_amd random CONFIG_JSON OUT_DIR [--seed 0] [--dtype bf16|f32]
 
@@ -48,7 +48,13 @@ def cmd_run(a) -> int:
         import dataclasses
         pipe.generate(prompt, dataclasses.replace(cfg, max_new_tokens=4, temperature=0.0), use_graph=not a.no_graph)
     t0 = time.perf_counter()
-    ids, st = pipe.generate(prompt, cfg, use_graph=not a.no_graph)
+    if a.op_times:      # the reference's per-op profile (model.rs:22-99): every op synchronised and timed, eager steps
+        from .kernels import ops
+        with ops.op_timing() as times:
+            ids, st = pipe.generate(prompt, cfg, use_graph=False)
+        print(times.report(), file=sys.stderr)
+    else:
+        ids, st = pipe.generate(prompt, cfg, use_graph=not a.no_graph)
     ms = (time.perf_counter() - t0) * 1e3
     print(pipe.decode(ids) if as_text else " ".join(str(t) for t in ids))
     # the reference's line: crates/synaptix-cli/src/commands/run.rs:234
@@ -109,6 +115,8 @@ def main(argv=None) -> int:
     r.add_argument("--compute-dtype", default="bf16", choices=["bf16", "f32"])
     r.add_argument("--no-graph", action="store_true")
     r.add_argument("--warmup", action="store_true")
+    r.add_argument("--op-times", action="store_true",
+                   help="time every kernel entry point with the device synchronised around it (eager steps) and print the table")
     r.add_argument("--top-k", type=int, default=0)
     r.add_argument("--top-p", type=float, default=1.0)
     r.add_argument("--min-p", type=float, default=0.0)

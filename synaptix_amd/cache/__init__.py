@@ -1,5 +1,5 @@
-from .pages import PAGE_TOKENS, PagePool, CacheFull, CacheError, pages_for
+from .pages import PAGE_TOKENS, CacheFull, CacheError, pages_for
 from .sequence_cache import SequenceCache, KvLayerView, StateLayerView, Snapshot
 
-__all__ = ["PAGE_TOKENS", "PagePool", "CacheFull", "CacheError", "pages_for", "SequenceCache", "Snapshot", "KvLayerView",
+__all__ = ["PAGE_TOKENS", "CacheFull", "CacheError", "pages_for", "SequenceCache", "Snapshot", "KvLayerView",
            "StateLayerView"]

@@ -182,20 +182,6 @@ int fill_table(Cache* c, int group, const int* sids, int n, int width, int fill,
 RT_API const char* syn_rt_last_error() { return g_error; }
 RT_API int syn_rt_page_tokens() { return PAGE_TOKENS; }
 
-// ------------------------------------------------------------------ page pool on its own
-RT_API void* syn_pool_new(int n_pages) {
-  if (n_pages <= 0) {
-    fail(MISUSE, "a page pool needs at least one page");
-    return nullptr;
-  }
-  return new PagePool(n_pages);
-}
-RT_API void syn_pool_delete(void* h) { delete (PagePool*)h; }
-RT_API int syn_pool_free_pages(void* h) { return ((PagePool*)h)->free_pages(); }
-RT_API int syn_pool_take(void* h, int n, int* out) { return ((PagePool*)h)->take(n, out); }
-RT_API int syn_pool_give_back(void* h, const int* pages, int n) { return ((PagePool*)h)->give_back(pages, n); }
-RT_API int syn_pool_check(void* h) { return ((PagePool*)h)->check(); }
-
 // ------------------------------------------------------------------ cache bookkeeping
 RT_API void* syn_cache_new(int n_groups, const long* windows, int n_pages, int max_slots, long max_positions) {
   if (n_groups < 0 || n_pages <= 0 || max_slots <= 0) {

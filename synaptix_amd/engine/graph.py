@@ -79,6 +79,8 @@ class DecodeRunner:
         """One token for each of `slots`; returns (sampled tokens as a host list, logits [B, V]).
         temps None: greedy for every row."""
         eng, B = self.engine, len(slots)
+        if ops.timing_active():
+            raise ops.KernelError("op_timing: per-op times need eager steps; a captured decode step cannot be timed op by op")
         if B > self.rows:
             raise ValueError(f"{B} sequences for a graph of {self.rows} rows")
         for s in slots:

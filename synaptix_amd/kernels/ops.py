@@ -74,9 +74,64 @@ def _need(t, name, dtypes, shape=None):
 
 
 def _call(lib, fn, *args):
+    if _timing is not None:
+        return _timed_call(lib, fn, args)
     rc = getattr(lib, fn)(*args)
     if rc != 0:
         raise KernelError(lib.syn_last_error().decode(errors="replace"))
+
+
+# ----------------------------------------------------------------------------- per-op times
+# The reference can time every op of a forward pass by synchronising the device around it
+# (crates/synaptix-models/llm/common/src/model.rs:22-99: prof(name, f), a table of (ms, calls) by name,
+# sorted by time, switched on for prefill or decode; off during graph capture).  Here the ops are the
+# kernel entry points; op_timing() switches the same thing on for the code inside it.
+
+_timing = None      # None, or {entry point: [milliseconds, calls]}
+
+
+def _timed_call(lib, fn, args):
+    import time
+    if torch.cuda.is_current_stream_capturing():
+        raise KernelError("op_timing: per-op times need eager steps (synchronising is not allowed while a graph is captured)")
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    rc = getattr(lib, fn)(*args)
+    torch.cuda.synchronize()
+    slot = _timing.setdefault(fn, [0.0, 0])
+    slot[0] += (time.perf_counter() - t0) * 1e3
+    slot[1] += 1
+    if rc != 0:
+        raise KernelError(lib.syn_last_error().decode(errors="replace"))
+
+
+def timing_active() -> bool:
+    return _timing is not None
+
+
+class OpTimes(dict):
+    """{entry point: [milliseconds, calls]} with the reference's report: sorted by time, with shares."""
+
+    def report(self) -> str:
+        total = sum(v[0] for v in self.values()) or 1.0
+        lines = [f"{'op':34s} {'ms':>10s} {'calls':>7s} {'share':>7s}"]
+        for name, (ms, calls) in sorted(self.items(), key=lambda kv: -kv[1][0]):
+            lines.append(f"{name:34s} {ms:10.3f} {calls:7d} {100 * ms / total:6.1f}%")
+        lines.append(f"{'total':34s} {total:10.3f}")
+        return "\n".join(lines)
+
+
+@contextlib.contextmanager
+def op_timing():
+    """Within the scope every kernel entry point is timed with the device synchronised before and after it
+    (so the times include each launch's latency and nothing overlaps); yields the table that fills up.
+    Steps inside the scope must be eager: captured steps are refused."""
+    global _timing
+    before, _timing = _timing, OpTimes()
+    try:
+        yield _timing
+    finally:
+        _timing = before
 
 
 def _is_f32(t):

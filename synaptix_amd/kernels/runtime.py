@@ -21,12 +21,6 @@ _IP, _LP, _FP, _UP = C.POINTER(C.c_int), C.POINTER(C.c_long), C.POINTER(C.c_floa
 
 _SIGNATURES = {
     "syn_rt_page_tokens": (_I, []),
-    "syn_pool_new": (_P, [_I]),
-    "syn_pool_delete": (None, [_P]),
-    "syn_pool_free_pages": (_I, [_P]),
-    "syn_pool_take": (_I, [_P, _I, _IP]),
-    "syn_pool_give_back": (_I, [_P, _IP, _I]),
-    "syn_pool_check": (_I, [_P]),
     "syn_cache_new": (_P, [_I, _LP, _I, _I, _L]),
     "syn_cache_delete": (None, [_P]),
     "syn_cache_free_slots": (_I, [_P]),

@@ -4,30 +4,13 @@ import random
 import pytest
 import torch
 
-from synaptix_amd.cache import SequenceCache, PagePool, CacheFull, CacheError, pages_for
+from synaptix_amd.cache import SequenceCache, CacheFull, CacheError, pages_for
 from synaptix_amd.parts import KvNeed, StateNeed
 
 
 def make(max_tokens=640, max_slots=None, needs=None, max_positions=None):
     needs = needs if needs is not None else [KvNeed(2, 16)] * 3
     return SequenceCache(needs, max_tokens, max_slots, torch.float32, "cpu", max_positions=max_positions)
-
-
-def test_page_pool():
-    p = PagePool(4)
-    a = p.take(3)
-    assert a == [0, 1, 2] and p.free_pages == 1
-    with pytest.raises(CacheFull):
-        p.take(2)
-    assert p.free_pages == 1                        # nothing was taken
-    p.give_back([1])
-    with pytest.raises(CacheError, match="not held"):
-        p.give_back([1])                            # freed twice
-    with pytest.raises(CacheError):
-        p.give_back([9])
-    p.check()
-    assert sorted(p.take(2)) == [1, 3]
-    p.check()
 
 
 def test_groups_and_storage():

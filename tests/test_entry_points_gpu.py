@@ -68,6 +68,36 @@ def test_command_line_run_and_bench():
     assert line["new_tokens"] == 48 and line["prompt_tokens"] == 27 and line["decode_tok_s"] > 0
 
 
+def test_per_op_times_of_eager_steps_and_their_refusal_under_capture():
+    from synaptix_amd import Engine
+    from synaptix_amd.kernels import ops
+    eng = Engine.load(model_folder("B"), dtype="bfloat16", max_tokens=512)
+    s = eng.acquire()
+    plain = eng.step([(s, [1, 2, 3, 4, 5])], want="last").clone()
+    eng.release(s)
+    s = eng.acquire()
+    with ops.op_timing() as times:
+        timed = eng.step([(s, [1, 2, 3, 4, 5])], want="last")
+        eng.step([(s, [6])], want="last")
+    assert torch.equal(timed, plain)                       # timing changes no result
+    L = CONFIGS["B"]["num_hidden_layers"]
+    assert times["syn_add_rmsnorm"][1] == 2 * (2 * L + 1) and times["syn_embed"][1] == 2
+    assert times["syn_attention_prefill_bf16"][1] == L and times["syn_attention_decode_fused_bf16"][1] == L
+    assert all(ms > 0 for ms, _ in times.values())
+    text = times.report()
+    assert text.splitlines()[0].split() == ["op", "ms", "calls", "share"] and "total" in text
+    with ops.op_timing():
+        with pytest.raises(Exception, match="per-op times need eager steps"):
+            eng.decode_runner(1, 256).step([s], [7])
+    eng.release(s)
+    # the command line's switch
+    cmd = [sys.executable, "-m", "synaptix_amd", "run", model_folder("A"), "--prompt-ids", "1,2,3", "--max-tokens", "3",
+           "--temperature", "0", "--op-times"]
+    proc = subprocess.run(cmd, capture_output=True, text=True, cwd=ROOT, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "syn_gemm" in proc.stderr and "share" in proc.stderr
+
+
 def test_smoke_entry():
     sys.path.insert(0, ROOT)
     import __graft_entry__
