@@ -1,10 +1,11 @@
 """Compile the native sources and load them through ctypes.
 
-Three kinds of library:
+Four kinds of library:
   core            every kernel whose sizes are run-time parameters (hipcc, gfx950)
   attn_hd<N>      the bf16 MFMA attention kernels, compiled for one head size (hipcc, gfx950)
   runtime         host code only: cache bookkeeping, step tables, the sampler's random stream
                   (the host C++ compiler)
+  ref             host code only: the kernels' plain C++ twins, the oracle of the kernel tests
 
 A library is built at its first use if no built file matches the sources, which is how the
 reference treats its kernels too (compiled at first use; crates/synaptix-kernels-cuda/src/kernels/compile.rs).
@@ -30,6 +31,7 @@ FLAGS = ["-O3", f"--offload-arch={ARCH}", "-std=c++17", "-fPIC", "-shared", "-fv
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden"]
 CORE_SOURCES = ["elementwise.hip", "sampling.hip", "gemm.hip", "attention_f32.hip", "probes.hip"]
 RUNTIME_SOURCES = ["runtime.cpp"]
+REF_SOURCES = ["ref/ref_kernels.cpp"]          # the kernels' plain C++ twins (host code)
 ATTN_SOURCE = "attention_bf16.hip"
 HEADERS = ["common.h", "no_alloc.h"]
 
@@ -79,7 +81,7 @@ def _writable_dir() -> str:
 
 
 def _digest(sources, defines) -> str:
-    host = list(sources) == RUNTIME_SOURCES
+    host = list(sources) in (RUNTIME_SOURCES, REF_SOURCES)
     h = hashlib.sha256()
     for name in list(sources) + ([] if host else HEADERS):
         with open(os.path.join(CSRC, name), "rb") as f:
@@ -92,6 +94,8 @@ def _digest(sources, defines) -> str:
 def _spec(name: str):
     if name == "runtime":
         return RUNTIME_SOURCES, []
+    if name == "ref":
+        return REF_SOURCES, []
     if name == "core":
         return CORE_SOURCES, []
     if name.startswith("attn_hd"):
@@ -123,12 +127,12 @@ def compile_library(name: str, quiet: bool = False) -> str:
     so = os.path.join(out_dir, f"libsynaptix_{name}.so")
     tmp_so = f"{so}.{os.getpid()}.tmp"
     paths = [os.path.join(CSRC, s) for s in sources]
-    if name == "runtime":
+    if name in ("runtime", "ref"):
         cmd = [find_host_compiler()] + HOST_FLAGS + paths + ["-o", tmp_so]
     else:
         cmd = [find_hipcc()] + FLAGS + defines + paths + ["-o", tmp_so]
     if not quiet:
-        target = "the host" if name == "runtime" else ARCH
+        target = "the host" if name in ("runtime", "ref") else ARCH
         _say(f"compiling {os.path.basename(so)} for {target} ({len(sources)} source file(s)) ...")
     t0 = time.time()
     proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, cwd=out_dir)
@@ -176,6 +180,8 @@ def load_library(name: str) -> ctypes.CDLL:
             raise KernelBuildError(f"cannot load {so}: {e}") from None
         if name == "runtime":
             lib.syn_rt_last_error.restype = ctypes.c_char_p
+        elif name == "ref":
+            pass            # the twins check nothing and report nothing: their callers are tests
         else:
             lib.syn_last_error.restype = ctypes.c_char_p
         _LOADED[name] = lib
@@ -184,7 +190,7 @@ def load_library(name: str) -> ctypes.CDLL:
 
 def build_all(head_dims=(16, 32, 64, 128)) -> list:
     """Compile the runtime, the core library and the attention library of each head size, in parallel."""
-    names = ["runtime", "core"] + [f"attn_hd{h}" for h in head_dims]
+    names = ["runtime", "ref", "core"] + [f"attn_hd{h}" for h in head_dims]
     results, errors = {}, []
 
     def work(n):
