@@ -344,8 +344,12 @@ def gemm_slices(M, N, K, dtype):
             return 1
         tiles = -(-M // 256) * -(-N // 256)
         return 4 if tiles * 4 <= 256 and K >= 8192 else (2 if tiles * 2 <= 256 else 1)
-    tiles = -(-N // 64)
-    most = min(4 if M <= 32 else 8, (768 if M <= 32 else 512) // tiles, K // 512)
+    if M <= 32:
+        # 64 rows of W a workgroup, up to three workgroups a compute unit
+        most = min(4, 768 // -(-N // 64), K // 512)
+    else:
+        # 128 rows of W a workgroup, one workgroup a compute unit
+        most = min(8, N_COMPUTE_UNITS // -(-N // 128), K // 512)
     slices = 1
     while slices * 2 <= most:
         slices *= 2
