@@ -255,6 +255,77 @@ static void launch_packed(const bf16* x, const bf16* wp, void* out, Epilogue ep,
       <<<dim3((N + rows - 1) / rows, slices), TILES * KWAVES * SYN_WAVE, 0, stream>>>(x, wp, out, ep, M, N, K, ks_slice);
 }
 
+
+// The same with two adjacent groups of 16 rows of W for every wave (for PAIRED: the gate rows and the up rows of
+// the same 16 outputs): a fragment of x is loaded once for two products, a third fewer loads at 8 rows of x.
+template <int KWAVES, int U, bool PAIRED>
+__global__ void __launch_bounds__(KWAVES * SYN_WAVE)
+gemm_packed2_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void* __restrict__ out, Epilogue ep,
+                    int M, int N, int K, int ks_slice) {
+  __shared__ float part[KWAVES][2][4][64];
+  const int kw = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
+  const int r16 = lane % 16, kq = (lane / 16) * 8;
+  const int nt = (int)blockIdx.x * 2, n_tiles = N / 16;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int nks = K / 32;
+  const bool second = nt + 1 < n_tiles;   // an odd number of groups leaves the last workgroup one
+  const bf16* wt0 = wp + ((size_t)nt * nks * 64 + lane) * 8;
+  const bf16* wt1 = wp + ((size_t)min(nt + 1, n_tiles - 1) * nks * 64 + lane) * 8;
+  const bool xok = r16 < M;
+  const bf16* xrow = x + (size_t)min(r16, M - 1) * K + kq;
+  f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+  const int ks_begin = (int)blockIdx.y * ks_slice, ks_end = min(nks, ks_begin + ks_slice);
+  for (int ks0 = ks_begin + kw * U; ks0 < ks_end; ks0 += KWAVES * U) {
+    bf16x8 b0[U], b1[U], ax[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const bool in = ks0 + u < ks_end;
+      b0[u] = in ? __builtin_nontemporal_load((const bf16x8*)(wt0 + (size_t)(ks0 + u) * 512)) : zero;
+      b1[u] = in ? __builtin_nontemporal_load((const bf16x8*)(wt1 + (size_t)(ks0 + u) * 512)) : zero;
+      ax[u] = (in && xok) ? *(const bf16x8*)(xrow + (ks0 + u) * 32) : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[u], b0[u], acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[u], b1[u], acc1, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) part[kw][0][j][lane] = acc0[j], part[kw][1][j][lane] = acc1[j];
+  __syncthreads();
+  auto summed = [&](int t, int j, int ln) {
+    float s = 0.f;
+#pragma unroll
+    for (int q = 0; q < KWAVES; ++q) s += part[q][t][j][ln];
+    return s;
+  };
+  if constexpr (PAIRED) {
+    for (int idx = threadIdx.x; idx < 4 * 64; idx += KWAVES * SYN_WAVE) {
+      const int j = idx / 64, ln = idx % 64;
+      const int m = 4 * (ln / 16) + j, col = (int)blockIdx.x * 16 + ln % 16;  // N / 2 outputs, 16 a workgroup
+      if (m < M && 2 * col < N) ((bf16*)out)[(size_t)m * (N / 2) + col] = (bf16)gated(ep.act, summed(0, j, ln), summed(1, j, ln));
+    }
+  } else {
+    for (int idx = threadIdx.x; idx < 2 * 4 * 64; idx += KWAVES * SYN_WAVE) {
+      const int t = idx / 256, j = (idx / 64) % 4, ln = idx % 64;
+      const int m = 4 * (ln / 16) + j, n = (nt + t) * 16 + ln % 16;
+      if (m < M && n < N && (t == 0 || second)) {
+        const float v = summed(t, j, ln);
+        if (ep.out_is_f32) ((float*)out)[((size_t)blockIdx.y * M + m) * N + n] = v;
+        else ((bf16*)out)[(size_t)m * N + n] = (bf16)v;
+      }
+    }
+  }
+}
+
+template <int KWAVES, int U, bool PAIRED = false>
+static void launch_packed2(const bf16* x, const bf16* wp, void* out, Epilogue ep, int M, int N, int K,
+                           hipStream_t stream, int slices = 1) {
+  const int ks_slice = (K / 32 + slices - 1) / slices;
+  gemm_packed2_kernel<KWAVES, U, PAIRED>
+      <<<dim3((N + 31) / 32, slices), KWAVES * SYN_WAVE, 0, stream>>>(x, wp, out, ep, M, N, K, ks_slice);
+}
+
 // ------------------------------------------------------------------ shared by the tiled kernels
 // Which tile: workgroup b runs on XCD b % 8, and each XCD has an L2 of its own.  Tiles are grouped
 // into panels of PM x PN (m fastest); a panel goes to one XCD, so the workgroups that run there at
@@ -922,7 +993,12 @@ SYN_EXPORT int syn_gemm_packed(const void* x, const void* wp, void* out, int out
   const bf16* xb = (const bf16*)x;
   const bf16* wb = (const bf16*)wp;
   // from sweeps at N = 4096 .. 151936, K = 4096 and 12288, 1 and 8 rows
-  if (paired) launch_packed<2, 8, 4, true>(xb, wb, out, ep, M, N, K, stream);
+  // gate and up rows of the same outputs: from 5 rows of x on a wave takes both (a fragment of x is then loaded
+  // once for two products: a decode step of 8 sequences 3.88 -> 3.80 ms; at one row 3.30 -> 3.31 ms, at four
+  // within the differences between boxes).  The same for the narrow products (two groups of rows a wave, twice
+  // the slices of K) gained under 1 % at 8 sequences and lost as much at 4.
+  if (paired && M >= 5) launch_packed2<16, 2, true>(xb, wb, out, ep, M, N, K, stream);
+  else if (paired) launch_packed<2, 8, 4, true>(xb, wb, out, ep, M, N, K, stream);
   else if (N <= 8192) launch_packed<1, 16, 2>(xb, wb, out, ep, M, N, K, stream, slices);
   else launch_packed<1, 8, 8>(xb, wb, out, ep, M, N, K, stream, slices);
   SYN_LAUNCH_CHECK("gemm_packed");
