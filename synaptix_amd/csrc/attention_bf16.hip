@@ -590,38 +590,42 @@ SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, co
 
 // ------------------------------------------------------------------ decode: split over keys, then merge
 // A workgroup of up to 8 waves takes (sequence, kv head, up to 16 heads of its group, one split of
-// the key blocks); its waves take the split's blocks in turn and their states are combined in LDS.
+// the keys, in units of half a block); its waves take the split's units in turn and their states are
+// combined in LDS.
 // With one split the workgroup writes the output itself; else it writes a partial
 //   partial[(seq * nh + head) * n_splits + split] = { m, l, o[HD] }   (float)
 // and a second kernel merges the splits.
 constexpr int PART = HD + 2;
-constexpr int DEC_MAX_WAVES = HD > 128 ? 4 : 8;  // as many as keep their registers (about 220 at 128) without spilling
+constexpr int DEC_MAX_WAVES = HD > 128 ? 4 : 8;  // as many as keep their registers (144 at a head size of 128, about twice that at 256) without spilling
 
-// The K and V fragments of one block of 64 keys, all requested before the first product needs one.
-struct KvBlock {
-  kfrag_t ka[4][KSTEPS];
-  bf16x8 va[2][DT];
+// The unit of a wave's work is half a block: 32 keys, whose K rows and whose V fragments are each one
+// contiguous piece of the page (64 * HD bytes).  Whole blocks leave the last round of a workgroup mostly
+// idle where a split holds few of them (33 blocks over 4 splits and 8 waves: two rounds, the second for
+// one wave).  These are the K and V fragments of one unit, all requested before the first product needs one.
+constexpr int UNIT_KEYS = 32;
+struct KvUnit {
+  kfrag_t ka[2][KSTEPS];
+  bf16x8 va[DT];
 };
 
-__device__ __forceinline__ void load_k_decode(KvBlock& b, const bf16* __restrict__ kpage, int lane) {
+// kpage: the unit's first K row
+__device__ __forceinline__ void load_k_decode(KvUnit& b, const bf16* __restrict__ kpage, int lane) {
   const int r16 = lane % 16;
 #pragma unroll
-  for (int t = 0; t < 4; ++t) load_row(b.ka[t], kpage + (size_t)tile_row_key(t, r16) * HD, lane);
+  for (int t = 0; t < 2; ++t) load_row(b.ka[t], kpage + (size_t)tile_row_key(t, r16) * HD, lane);
 }
 
 // a fragment of V is 1 KB of the page, in lane order.  A decode step reads every key and value once: its
 // loads are marked non-temporal (551 MB of cache for 64 sequences: 98.8 -> 88.5 us a layer; never slower
-// from 1 to 64 sequences and 500 to 32,000 tokens).
-__device__ __forceinline__ void load_v_decode(KvBlock& b, const bf16* __restrict__ vpage, int lane) {
+// from 1 to 64 sequences and 500 to 32,000 tokens).  vpage: the unit's first fragment
+__device__ __forceinline__ void load_v_decode(KvUnit& b, const bf16* __restrict__ vpage, int lane) {
 #pragma unroll
-  for (int h = 0; h < 2; ++h)
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-      b.va[h][dt] = __builtin_nontemporal_load((const bf16x8*)(vpage + (size_t)((h * DT + dt) * 64 + lane) * 8));
+  for (int dt = 0; dt < DT; ++dt)
+    b.va[dt] = __builtin_nontemporal_load((const bf16x8*)(vpage + (size_t)(dt * 64 + lane) * 8));
 }
 
-// Head sizes that are a power of two from 32 on: a block's K rows (64 x HD) are one contiguous piece of
-// 128 * HD bytes, and a wave brings them into a piece of LDS of its own with loads of 1 KB that write
+// Head sizes that are a power of two from 32 on: a unit's K rows (32 x HD) are one contiguous piece of
+// 64 * HD bytes, and a wave brings them into a piece of LDS of its own with loads of 1 KB that write
 // LDS directly, then reads its fragments from there.  Loading K fragments straight from memory asks
 // the first-level cache for 16 rows x 64 bytes with every instruction, which was measured to keep
 // the texture addresser busy about 100 cycles an instruction and to bound the kernel at large
@@ -630,8 +634,8 @@ __device__ __forceinline__ void load_v_decode(KvBlock& b, const bf16* __restrict
 // rows a fragment read touches fall into different banks; the permutation is applied to the address
 // that a lane fetches (the slot it fills is fixed by its number) and again by the reader.
 constexpr bool STAGED = !TAIL16 && (HD & (HD - 1)) == 0;
-constexpr int STAGE_BYTES = STAGED ? 128 * HD : 0;   // one block of K
-constexpr int K_CPR = HD / 8;                        // 16-byte chunks in a K row
+constexpr int STAGE_BYTES = STAGED ? 64 * HD : 0;   // the K rows of one unit
+constexpr int K_CPR = HD / 8;                       // 16-byte chunks in a K row
 // the rows of a score tile differ in bits 0, 1, 3 and 4 of the key number: those four bits, less as
 // many low ones as rows fit into the 256 bytes that the banks span
 __device__ __forceinline__ int k_swizzle(int row) {
@@ -642,48 +646,46 @@ __device__ __forceinline__ int k_swizzle(int row) {
 __device__ __forceinline__ void stage_k(const bf16* __restrict__ kpage, char* stage, int lane) {
   const BufferView view = buffer_view(kpage, STAGE_BYTES);
 #pragma unroll
-  for (int i = 0; i < HD / 8; ++i) {
+  for (int i = 0; i < HD / 16; ++i) {
     const int at = 64 * i + lane, row = at / K_CPR, slot = at % K_CPR;
     buffer_to_lds16<true>(view, stage + 1024 * i, (unsigned)((row * K_CPR + (slot ^ k_swizzle(row))) * 16), 0);
   }
 }
-// The staged K has landed: of this wave's loads at most the V fragments requested after it (2 * DT loads)
+// The staged K has landed: of this wave's loads at most the V fragments requested after it (DT loads)
 // are still on their way.  Nothing that reads the piece may move above this.
-__device__ __forceinline__ void staged_landed() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * DT) : "memory"); }
+__device__ __forceinline__ void staged_landed() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DT) : "memory"); }
 // this wave's reads of the staged piece have returned: the piece may be filled again
 __device__ __forceinline__ void staged_read() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
-__device__ __forceinline__ void read_k_staged(KvBlock& b, const char* stage, int lane) {
+__device__ __forceinline__ void read_k_staged(KvUnit& b, const char* stage, int lane) {
   if constexpr (STAGED) {
     const int r16 = lane % 16, g4 = lane / 16;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int t = 0; t < 2; ++t) {
       const int row = tile_row_key(t, r16), sw = k_swizzle(row);
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) b.ka[t][ks] = *(const kfrag_t*)(stage + (row * K_CPR + ((ks * 4 + g4) ^ sw)) * 16);
     }
   }
 }
-// One block of 64 keys in two halves, so that the loads of the next block can follow each half at once:
+// One unit of 32 keys in two parts, so that the loads of the next unit can follow each part at once:
 // the scores and their softmax weights (reads the K fragments), then the weighted values (reads the V fragments).
-__device__ __forceinline__ void decode_scores(AttnState<1>& st, const QFrag& qf, const KvBlock& blk, f32x4 (&s)[4],
-                                              int key0, int qpos, int lo, float scale, int lane) {
-  const int g4 = lane / 16;
-  const auto& ka = blk.ka;
+__device__ __forceinline__ void decode_scores(const QFrag& qf, const KvUnit& unit, f32x4 (&s)[2]) {
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
+  for (int t = 0; t < 2; ++t) {
     s[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) s[t] = mfma_qk(ka[t][ks], qf.k[ks], s[t]);
+    for (int ks = 0; ks < KSTEPS; ++ks) s[t] = mfma_qk(unit.ka[t][ks], qf.k[ks], s[t]);
   }
 }
 
-__device__ __forceinline__ void decode_weights(AttnState<1>& st, f32x4 (&s)[4], int key0, int qpos, int lo, float scale,
+// key0: the unit's first key
+__device__ __forceinline__ void decode_weights(AttnState<1>& st, f32x4 (&s)[2], int key0, int qpos, int lo, float scale,
                                                int lane) {
   const int g4 = lane / 16;
   float mloc = -INFINITY;
 #pragma unroll
-  for (int t = 0; t < 4; ++t)
+  for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int key = key0 + acc_key(t, g4, e);
@@ -700,7 +702,7 @@ __device__ __forceinline__ void decode_weights(AttnState<1>& st, f32x4 (&s)[4], 
   st.m[0] = m_new;
   float lsum = 0.f;
 #pragma unroll
-  for (int t = 0; t < 4; ++t)
+  for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const float p = __expf(s[t][e] - m_use);
@@ -712,29 +714,25 @@ __device__ __forceinline__ void decode_weights(AttnState<1>& st, f32x4 (&s)[4], 
   for (int dt = 0; dt < DT; ++dt) st.o[dt][0] *= alpha;
 }
 
-__device__ __forceinline__ void decode_values(AttnState<1>& st, const KvBlock& blk, const f32x4 (&s)[4], int key0,
+__device__ __forceinline__ void decode_values(AttnState<1>& st, const KvUnit& unit, const f32x4 (&s)[2], int key0,
                                               int kv_len, int lane) {
   const int g4 = lane / 16;
-  const auto& va = blk.va;
-  const bool ragged = key0 + SYN_PAGE > kv_len;
+  const bool ragged = key0 + UNIT_KEYS > kv_len;
+  bf16x8 pb;
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    bf16x8 pb;
+  for (int e = 0; e < 4; ++e) {
+    pb[e] = (bf16)s[0][e];
+    pb[4 + e] = (bf16)s[1][e];
+  }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      pb[e] = (bf16)s[2 * h][e];
-      pb[4 + e] = (bf16)s[2 * h + 1][e];
+  for (int dt = 0; dt < DT; ++dt) {
+    bf16x8 av = unit.va[dt];
+    if (ragged) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (key0 + 8 * g4 + e >= kv_len) av[e] = (bf16)0.f;  // 0 * (whatever lies there) must be 0
     }
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      bf16x8 av = va[h][dt];
-      if (ragged) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (key0 + h * 32 + 8 * g4 + e >= kv_len) av[e] = (bf16)0.f;  // 0 * (whatever lies there) must be 0
-      }
-      st.o[dt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, pb, st.o[dt][0], 0, 0, 0);
-    }
+    st.o[dt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, pb, st.o[dt][0], 0, 0, 0);
   }
 }
 
@@ -789,23 +787,25 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
   const bool new_key = FUSED && in.own_kv;            // the newest key is not read from the cache
   const bool adds_new = new_key && split == 0;        // this workgroup makes it and adds it
 
-  // keys read from the cache: all of them, or all but the newest; the blocks of this split; the first
-  // block of this wave is requested at once, before the workgroup prepares its q heads
+  // keys read from the cache: all of them, or all but the newest; the units of this split; the first
+  // unit of this wave is requested at once, before the workgroup prepares its q heads
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int n_old = new_key ? kv_len - 1 : kv_len;
   const int q_lim = new_key ? pos - 1 : pos;  // the last key position that the loop may see
-  const int b_lo = lo / SYN_PAGE, b_hi = n_old > 0 ? (n_old - 1) / SYN_PAGE : b_lo - 1;
-  const int per = (b_hi - b_lo + n_splits) / n_splits;  // ceil((b_hi - b_lo + 1) / n_splits)
-  const int b0 = b_lo + split * per, b1 = min(b_hi + 1, b0 + per);
-  auto page_of = [&](int kb) {   // the same for all lanes
-    return ((size_t)__builtin_amdgcn_readfirstlane(page_table[(size_t)seq * table_stride + kb]) * nkv + kvh) * SYN_PAGE * HD;
+  const int u_lo = lo / UNIT_KEYS, u_hi = n_old > 0 ? (n_old - 1) / UNIT_KEYS : u_lo - 1;
+  const int per = (u_hi - u_lo + n_splits) / n_splits;  // ceil((u_hi - u_lo + 1) / n_splits)
+  const int u0 = u_lo + split * per, u1 = min(u_hi + 1, u0 + per);
+  constexpr int UNITS = SYN_PAGE / UNIT_KEYS;   // units in a page
+  auto unit_at = [&](int u) {   // where the unit's K rows and V fragments begin in the page arrays; the same for all lanes
+    const int page = __builtin_amdgcn_readfirstlane(page_table[(size_t)seq * table_stride + u / UNITS]);
+    return ((size_t)page * nkv + kvh) * SYN_PAGE * HD + (size_t)(u % UNITS) * UNIT_KEYS * HD;
   };
-  KvBlock blk;
-  if (b0 + wave < b1) {
-    const size_t base = page_of(b0 + wave);
+  KvUnit unit;
+  if (u0 + wave < u1) {
+    const size_t base = unit_at(u0 + wave);
     if constexpr (STAGED) stage_k(k_pages + base, stage, lane);
-    else load_k_decode(blk, k_pages + base, lane);
-    load_v_decode(blk, v_pages + base, lane);
+    else load_k_decode(unit, k_pages + base, lane);
+    load_v_decode(unit, v_pages + base, lane);
   }
 
   float* xs = so + (size_t)n_waves * cols_alloc * SO_LD;
@@ -916,26 +916,27 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
     load_q(qf, valid ? q + ((size_t)seq * nh + kvh * g + hg) * HD : nullptr, lane);
   AttnState<1> st;
   attn_init(st);
-  // K of the next block is requested as soon as the K fragments of this one are in registers (or have
-  // been used), V of the next block as soon as the V fragments have been used: K is on its way during
-  // the products of this block, V during the scores of the next, without a second set of registers
-  for (int kb = b0 + wave; kb < b1; kb += n_waves) {
-    const int next = kb + n_waves;
-    const size_t next_base = next < b1 ? page_of(next) : 0;
-    f32x4 s[4];
+  // K of the next unit is requested as soon as the K fragments of this one are in registers (or have
+  // been used), V of the next unit as soon as the V fragments have been used: K is on its way during
+  // the products of this unit, V during the scores of the next, without a second set of registers
+  for (int u = u0 + wave; u < u1; u += n_waves) {
+    const int next = u + n_waves;
+    const size_t next_base = next < u1 ? unit_at(next) : 0;
+    const int key0 = u * UNIT_KEYS;
+    f32x4 s[2];
     if constexpr (STAGED) {
       staged_landed();
-      read_k_staged(blk, stage, lane);
+      read_k_staged(unit, stage, lane);
       staged_read();
-      if (next < b1) stage_k(k_pages + next_base, stage, lane);
-      decode_scores(st, qf, blk, s, kb * SYN_PAGE, valid ? q_lim : -1, lo, scale, lane);
+      if (next < u1) stage_k(k_pages + next_base, stage, lane);
+      decode_scores(qf, unit, s);
     } else {
-      decode_scores(st, qf, blk, s, kb * SYN_PAGE, valid ? q_lim : -1, lo, scale, lane);
-      if (next < b1) load_k_decode(blk, k_pages + next_base, lane);
+      decode_scores(qf, unit, s);
+      if (next < u1) load_k_decode(unit, k_pages + next_base, lane);
     }
-    decode_weights(st, s, kb * SYN_PAGE, valid ? q_lim : -1, lo, scale, lane);
-    decode_values(st, blk, s, kb * SYN_PAGE, n_old, lane);
-    if (next < b1) load_v_decode(blk, v_pages + next_base, lane);
+    decode_weights(st, s, key0, valid ? q_lim : -1, lo, scale, lane);
+    decode_values(st, unit, s, key0, n_old, lane);
+    if (next < u1) load_v_decode(unit, v_pages + next_base, lane);
   }
   float l = st.l[0];
   l += __shfl_xor(l, 16, SYN_WAVE);
@@ -958,7 +959,7 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
     float acc = 0.f, lsum = 0.f;
     for (int w = 0; w < n_waves; ++w) {
       const float mw = sm[w * 16 + c];
-      if (mw == -INFINITY) continue;  // a wave that had no block
+      if (mw == -INFINITY) continue;  // a wave that had no unit
       const float f = __expf(mw - m);
       acc += f * so[((size_t)w * cols_alloc + c) * SO_LD + d];
       lsum += f * sl[w * 16 + c];
