@@ -371,9 +371,12 @@ __global__ void qk_norm_rope_kv_write_kernel(const TIn* __restrict__ qkv, int n_
 // a head and whose rotation covers the whole head (or is absent): a lane holds 8 values of a head
 // (16-byte load and store), the sum of squares is reduced over the LPH lanes of the head, and the
 // partner of a rotated pair sits LPH / 2 lanes away.  A block takes 256 / LPH heads of one token.
-template <int LPH>
+// PARTS: the rows come as n_parts float partial sums [n_parts][tokens][heads * HD] of a product cut
+// along K (part_stride elements apart), which are added first, in their order.
+template <int LPH, bool PARTS>
 __global__ void __launch_bounds__(256)
-qk_heads_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ q_out, bf16* __restrict__ k_pages,
+qk_heads_kernel(const void* __restrict__ qkv_in, int n_parts, size_t part_stride, bf16* __restrict__ q_out,
+                bf16* __restrict__ k_pages,
                 const int* __restrict__ page_table, int table_stride, const int* __restrict__ tok_seq,
                 const int* __restrict__ tok_pos, const void* __restrict__ q_gain, const void* __restrict__ k_gain,
                 int gain_is_f32, float gain_offset, float eps, const float* __restrict__ cos_t,
@@ -398,14 +401,43 @@ qk_heads_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ q_out, bf16* __
 #pragma unroll
     for (int e = 0; e < 8; ++e) g[e] += gain_offset;
   }
-  bf16x8 raw[TPB];
+  float val[TPB][8];
   int pos[TPB];
   float4 cs[TPB][2], sn[TPB][2];
+  if constexpr (PARTS) {
 #pragma unroll
-  for (int t = 0; t < TPB; ++t) {
-    const int tok = min((int)blockIdx.x * TPB + t, n_tokens - 1);
-    raw[t] = *(const bf16x8*)(qkv + ((size_t)tok * (nh + 2 * nkv) + head) * HD + c * 8);
-    pos[t] = tok_pos[tok];
+    for (int t = 0; t < TPB; ++t) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) val[t][e] = 0.f;
+      pos[t] = tok_pos[min((int)blockIdx.x * TPB + t, n_tokens - 1)];
+    }
+    for (int p = 0; p < n_parts; ++p) {
+      float4 lo4[TPB], hi4[TPB];     // the tokens' loads of one part in flight together
+#pragma unroll
+      for (int t = 0; t < TPB; ++t) {
+        const int tok = min((int)blockIdx.x * TPB + t, n_tokens - 1);
+        const float4* src = (const float4*)((const float*)qkv_in + (size_t)p * part_stride +
+                                            ((size_t)tok * (nh + 2 * nkv) + head) * HD + c * 8);
+        lo4[t] = src[0], hi4[t] = src[1];
+      }
+#pragma unroll
+      for (int t = 0; t < TPB; ++t) {
+        val[t][0] += lo4[t].x, val[t][1] += lo4[t].y, val[t][2] += lo4[t].z, val[t][3] += lo4[t].w;
+        val[t][4] += hi4[t].x, val[t][5] += hi4[t].y, val[t][6] += hi4[t].z, val[t][7] += hi4[t].w;
+      }
+    }
+  } else {
+    bf16x8 raw[TPB];
+#pragma unroll
+    for (int t = 0; t < TPB; ++t) {
+      const int tok = min((int)blockIdx.x * TPB + t, n_tokens - 1);
+      raw[t] = *(const bf16x8*)((const bf16*)qkv_in + ((size_t)tok * (nh + 2 * nkv) + head) * HD + c * 8);
+      pos[t] = tok_pos[tok];
+    }
+#pragma unroll
+    for (int t = 0; t < TPB; ++t)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) val[t][e] = (float)raw[t][e];
   }
   if (cos_t) {
 #pragma unroll
@@ -422,7 +454,7 @@ qk_heads_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ q_out, bf16* __
     float ss = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      v[e] = (float)raw[t][e];
+      v[e] = val[t][e];
       ss += v[e] * v[e];
     }
     if (gain) {
@@ -458,8 +490,10 @@ qk_heads_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ q_out, bf16* __
 // order of v_page_offset, in which 8 consecutive positions of one dim are one 16-byte piece and the
 // 16 dims of a fragment follow each other at 16 bytes.
 #define V_DIMS 32
+template <bool PARTS>   // as for qk_heads_kernel
 __global__ void __launch_bounds__(256)
-v_block_write_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ v_pages, const int* __restrict__ page_table,
+v_block_write_kernel(const void* __restrict__ qkv_in, int n_parts, size_t part_stride, bf16* __restrict__ v_pages,
+                     const int* __restrict__ page_table,
                      int table_stride, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, int n_tokens,
                      int nh, int nkv, int hd) {
   constexpr int LD = V_DIMS + 2, PAIRS = V_DIMS / 2;
@@ -470,9 +504,19 @@ v_block_write_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ v_pages, c
   const int heads = nh + 2 * nkv;
   for (int idx = tid; idx < 64 * PAIRS; idx += 256) {
     const int j = idx / PAIRS, pr = idx % PAIRS;
-    if (t0 + j < n_tokens && d0 + 2 * pr < hd)   // head sizes are even
-      *(uint32_t*)(vtile + j * LD + 2 * pr) =
-          *(const uint32_t*)(qkv + ((size_t)(t0 + j) * heads + nh + nkv + kvh) * hd + d0 + 2 * pr);
+    if (t0 + j < n_tokens && d0 + 2 * pr < hd) {   // head sizes are even
+      const size_t at = ((size_t)(t0 + j) * heads + nh + nkv + kvh) * hd + d0 + 2 * pr;
+      if constexpr (PARTS) {
+        float2 sum = make_float2(0.f, 0.f);
+        for (int p = 0; p < n_parts; ++p) {
+          const float2 v = *(const float2*)((const float*)qkv_in + (size_t)p * part_stride + at);
+          sum.x += v.x, sum.y += v.y;
+        }
+        vtile[j * LD + 2 * pr] = (bf16)sum.x, vtile[j * LD + 2 * pr + 1] = (bf16)sum.y;
+      } else {
+        *(uint32_t*)(vtile + j * LD + 2 * pr) = *(const uint32_t*)((const bf16*)qkv_in + at);
+      }
+    }
   }
   if (tid < 64 && t0 + tid < n_tokens) {
     const int tok = t0 + tid, pos = tok_pos[tok];
@@ -500,7 +544,8 @@ SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, int n_parts, void* q_o
   SYN_CHECK(n_parts >= 0 && n_parts <= 64, "qk_norm_rope_kv_write: %d partial sums", n_parts);
   // prompts in bf16: the kernels that move 16 bytes a lane, where the head size and the rotation allow them
   const int lph = hd / 8;
-  const bool fast = !is_f32 && n_parts == 0 && hd % 8 == 0 && lph >= 2 && lph <= 32 && (lph & (lph - 1)) == 0 &&
+  // (partial sums of up to 64 tokens stay with the one kernel below: two launches cost more than it takes)
+  const bool fast = !is_f32 && (n_parts == 0 || n_tokens > 64) && hd % 8 == 0 && lph >= 2 && lph <= 32 && (lph & (lph - 1)) == 0 &&
                     (cos_t == nullptr || rot == hd) && (uintptr_t)qkv % 16 == 0 && (uintptr_t)q_out % 16 == 0 &&
                     (uintptr_t)k_pages % 16 == 0 && (uintptr_t)q_gain % 16 == 0 && (uintptr_t)k_gain % 16 == 0 &&
                     (uintptr_t)cos_t % 16 == 0 && (uintptr_t)sin_t % 16 == 0;
@@ -508,10 +553,18 @@ SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, int n_parts, void* q_o
     const int n_active = write_kv ? nh + nkv : nh;
     const int hpb = 256 / lph;
     const dim3 grid((n_tokens + 3) / 4, (n_active + hpb - 1) / hpb);
+    const size_t part_stride = (size_t)n_tokens * (nh + 2 * nkv) * hd;
 #define SYN_QKH(L)                                                                                                  \
-  qk_heads_kernel<L><<<grid, 256, 0, stream>>>((const bf16*)qkv, (bf16*)q_out, (bf16*)k_pages, page_table,          \
-                                               table_stride, tok_seq, tok_pos, q_gain, k_gain, gain_is_f32,          \
-                                               gain_offset, eps, cos_t, sin_t, n_tokens, nh, nkv, n_active)
+  if (n_parts > 0)                                                                                                  \
+    qk_heads_kernel<L, true><<<grid, 256, 0, stream>>>(qkv, n_parts, part_stride, (bf16*)q_out, (bf16*)k_pages,    \
+                                                       page_table, table_stride, tok_seq, tok_pos, q_gain, k_gain, \
+                                                       gain_is_f32, gain_offset, eps, cos_t, sin_t, n_tokens, nh,  \
+                                                       nkv, n_active);                                              \
+  else                                                                                                              \
+    qk_heads_kernel<L, false><<<grid, 256, 0, stream>>>(qkv, 0, 0, (bf16*)q_out, (bf16*)k_pages, page_table,       \
+                                                        table_stride, tok_seq, tok_pos, q_gain, k_gain,            \
+                                                        gain_is_f32, gain_offset, eps, cos_t, sin_t, n_tokens, nh, \
+                                                        nkv, n_active)
     switch (lph) {
       case 2: SYN_QKH(2); break;
       case 4: SYN_QKH(4); break;
@@ -522,8 +575,13 @@ SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, int n_parts, void* q_o
 #undef SYN_QKH
     SYN_LAUNCH_CHECK("qk_heads");
     if (write_kv) {
-      v_block_write_kernel<<<dim3((n_tokens + 63) / 64, nkv, (hd + V_DIMS - 1) / V_DIMS), 256, 0, stream>>>(
-          (const bf16*)qkv, (bf16*)v_pages, page_table, table_stride, tok_seq, tok_pos, n_tokens, nh, nkv, hd);
+      const dim3 vgrid((n_tokens + 63) / 64, nkv, (hd + V_DIMS - 1) / V_DIMS);
+      if (n_parts > 0)
+        v_block_write_kernel<true><<<vgrid, 256, 0, stream>>>(qkv, n_parts, part_stride, (bf16*)v_pages, page_table,
+                                                              table_stride, tok_seq, tok_pos, n_tokens, nh, nkv, hd);
+      else
+        v_block_write_kernel<false><<<vgrid, 256, 0, stream>>>(qkv, 0, 0, (bf16*)v_pages, page_table, table_stride,
+                                                               tok_seq, tok_pos, n_tokens, nh, nkv, hd);
       SYN_LAUNCH_CHECK("v_block_write");
     }
     return 0;

@@ -908,7 +908,9 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   // 52 -> 18, down_proj in four 74 -> 34; at 256 rows 59 -> 36, 57 -> 22, 79 -> 62; at 512 rows o_proj
   // 58 -> 39 and q/k/v 63 -> 67; down_proj from 384 rows on and the output head stay on the large tiles).
   const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
-  const bool few_large_tiles = M > 64 && M <= 512 && K % 128 == 0 && tiles128 * slices <= 256;
+  // (cut along K the tiles are 128 x 128 up to 256 rows and 256 x 128 beyond)
+  const long tiles_cut = (long)(M <= 256 ? (M + 127) / 128 : (M + 255) / 256) * ((N + 127) / 128);
+  const bool few_large_tiles = M > 64 && M <= 512 && K % 128 == 0 && (slices > 1 ? tiles_cut : tiles128) * slices <= 256;
   int rc = 0;
   if (M == 1 && slices == 1) {
     // one row: fragments of W straight from memory, K split over the waves
@@ -927,8 +929,16 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
     // sequences: 7.70 -> 7.51 ms with this tile for q/k/v, o_proj and down_proj, 7.26 with it for gate+up
     // as well (though that product then has only 192 workgroups); 64 x 64 tiles in a ring of four: 8.08.
     rc = launch_direct<64, 128, 128, 2, 4, false, 3>(xb, wb, out, ep, M, N, K, stream, slices);
+  } else if (few_large_tiles && slices > 1) {
+    // short prompts of a narrow product whose reader adds partial sums: k-tiles of 64 in a ring of three, 128 rows
+    // of W a workgroup, and as many slices of K as fill the compute units (ops.gemm_slices).  Measured at the
+    // shapes of an 8B layer against the tiles of the branch below: 128 rows: q/k/v in 4 slices 17 us (31 uncut),
+    // down_proj in 8 slices 26 (30 in 4); 256 rows: q/k/v 26 (32), down_proj 39 (50); 512 rows (256 rows of x a
+    // tile): q/k/v in 2 slices 36 (51), o_proj in 4 slices 29 (30), down_proj 57 (55).
+    if (M <= 256) rc = launch_direct<128, 128, 64, 2, 4, false, 3>(xb, wb, out, ep, M, N, K, stream, slices);
+    else rc = launch_direct<256, 128, 64, 4, 2, false, 3>(xb, wb, out, ep, M, N, K, stream, slices);
   } else if (few_large_tiles && K % 128 == 0) {
-    // short prompts of a narrow product: the same tile up to 256 rows, 128 x 128 beyond (a prompt of 256 tokens
+    // the same uncut: 64 x 128 up to 256 rows, 128 x 128 beyond (a prompt of 256 tokens
     // 8.91 -> 8.24 ms, of 512 tokens 12.63 -> 11.59 ms against 64 x 64 tiles)
     if (M <= 256) rc = launch_direct<64, 128, 128, 2, 4, false, 3>(xb, wb, out, ep, M, N, K, stream, slices);
     else rc = launch_direct<128, 128, 128, 2, 4, false, 2>(xb, wb, out, ep, M, N, K, stream, slices);
@@ -966,6 +976,15 @@ SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, i
   } else if (M <= 64) {
     if (K % 128 == 0) rc = launch_direct<64, 128, 128, 2, 2, true, 3>(xb, wb, out, ep, M, N, K, stream);
     else rc = launch_tiled<64, 64, 128, 2, 2, true>(xb, wb, out, ep, M, N, K, stream);
+  } else if (M <= 256 && K % 64 == 0) {
+    // 65 to 256 rows: still bound by reading W.  All of x in one tile, so that W is read once; k-tiles of 64 in a
+    // ring of three or four, so that a workgroup has 60 to 80 KB under way.  Measured for gate+up of an 8B layer
+    // (N = 24576, K = 4096) against the smallest of the large tiles: 128 rows 66 -> 46 us (96 rows of W a
+    // workgroup: 256 workgroups), 192 rows 72 -> 57, 256 rows 80 -> 62; from 320 rows on the large tiles win
+    // (98 against 110 us and more).
+    if (M <= 128) rc = launch_direct<128, 96, 64, 4, 1, true, 4>(xb, wb, out, ep, M, N, K, stream);
+    else if (M <= 192) rc = launch_direct<192, 128, 64, 2, 2, true, 3>(xb, wb, out, ep, M, N, K, stream);
+    else rc = launch_direct<256, 128, 64, 4, 2, true, 3>(xb, wb, out, ep, M, N, K, stream);
   } else {
     rc = launch_large<true>(xb, wb, out, ep, M, N, K, stream);
   }

@@ -342,6 +342,15 @@ def gemm_slices(M, N, K, dtype):
         # at the price of partial sums of M x N floats each
         if K % 128:
             return 1
+        if M <= 512:
+            # short prompts: still bound by reading W; tiles of 128 rows of W (and of 128 rows of x up to 256 rows,
+            # of 256 beyond), cut until they fill the compute units
+            tiles = (-(-M // 128) if M <= 256 else -(-M // 256)) * -(-N // 128)
+            most, slices = min(8, N_COMPUTE_UNITS // tiles, K // 512), 1
+            while slices * 2 <= most:
+                slices *= 2
+            if slices > 1:
+                return slices
         tiles = -(-M // 256) * -(-N // 256)
         return 4 if tiles * 4 <= 256 and K >= 8192 else (2 if tiles * 2 <= 256 else 1)
     if M <= 32:

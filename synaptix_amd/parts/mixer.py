@@ -96,8 +96,9 @@ class GqaAttention(Mixer):
             if qkv.dim() == 2:
                 qkv = qkv.unsqueeze(0)
         else:
-            # (the kernels behind single tokens, and behind prompts of up to 64 tokens, add partial sums themselves)
-            sliced = (N <= 64 or ctx.one_token_each) and ops.gemm_slices(N, self.w_qkv.shape[0], self.hidden, act) > 1
+            # (the kernels behind single tokens, and behind prompts of up to 512 tokens, add partial sums themselves;
+            # longer prompts fill the compute units uncut)
+            sliced = (N <= 512 or ctx.one_token_each) and ops.gemm_slices(N, self.w_qkv.shape[0], self.hidden, act) > 1
             qkv = linear_for_sum(h, self.w_qkv) if sliced else linear(h, self.w_qkv, act)
         cos, sin = self.position.tables(h.device)
         table = ctx.page_table(cache.group)

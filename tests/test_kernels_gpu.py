@@ -226,7 +226,10 @@ def test_gemm_bf16(ops, out_dtype, M, N, K):
 @pytest.mark.parametrize("M,N,K,S", [(1, 48, 4096, 4), (8, 4096, 4096, 4), (8, 100, 1000, 3), (16, 64, 12288, 8),
                                      (40, 70, 2048, 2), (64, 130, 520, 5), (8, 96, 1536, 5), (50, 200, 3072, 7),
                                      (300, 520, 1024, 2), (130, 260, 640, 3), (65, 33, 4096, 4),
-                                     (200, 4096, 1024, 2), (256, 1000, 2048, 4)])
+                                     (200, 4096, 1024, 2), (256, 1000, 2048, 4),
+                                     # short prompts cut along K: tiles of 128 x 128 up to 256 rows, of 256 x 128 beyond
+                                     (66, 6144, 4096, 4), (128, 200, 4096, 8), (129, 4100, 1024, 2), (256, 1000, 2560, 4),
+                                     (257, 520, 4096, 8), (400, 2000, 1152, 2), (512, 4096, 1024, 2)])
 def test_gemm_bf16_partial_sums_over_slices_of_k(ops, M, N, K, S):
     """[S, M, N]: slice s holds the sum over its part of K; the slices add up to the product, also
     when K is no multiple of the slice and the last slices are short or empty."""
@@ -260,7 +263,10 @@ def test_gemm_bf16_partial_sums_over_slices_of_k(ops, M, N, K, S):
 
 @pytest.mark.parametrize("M,I,K", [(1, 48, 64), (1, 2560, 4096), (1, 1008, 1096), (8, 2560, 4096), (7, 112, 1000), (33, 80, 136), (64, 1024, 512),
                                    (300, 400, 264), (2048, 3072, 256), (1000, 6272, 136), (8, 32784, 72),
-                                   (1000, 6272, 128), (300, 400, 192)])
+                                   (1000, 6272, 128), (300, 400, 192),
+                                   # 65 to 256 rows: all of x in one tile of 128, 192 or 256 rows and 96 or 128 rows of W
+                                   (65, 48, 64), (100, 1040, 448), (128, 12288, 512), (129, 400, 192), (192, 2000, 320),
+                                   (193, 80, 1024), (256, 4864, 640), (200, 400, 72)])
 def test_gemm_with_the_gated_activation_inside(ops, M, I, K):
     """silu(x . Wg^T) * (x . Wu^T) from one product over the rows of Wg and Wu in turns of 16,
     against the two products and the activation in 64-bit; every tile shape of the kernel."""
