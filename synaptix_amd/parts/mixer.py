@@ -96,9 +96,9 @@ class GqaAttention(Mixer):
             if qkv.dim() == 2:
                 qkv = qkv.unsqueeze(0)
         else:
-            # (the kernels behind single tokens, and behind prompts of up to 512 tokens, add partial sums themselves;
-            # longer prompts fill the compute units uncut)
-            sliced = (N <= 512 or ctx.one_token_each) and ops.gemm_slices(N, self.w_qkv.shape[0], self.hidden, act) > 1
+            # (every kernel behind it adds partial sums itself; ops.gemm_slices cuts where the product would
+            # otherwise leave compute units without work: single tokens and prompts up to about 1,200 tokens)
+            sliced = ops.gemm_slices(N, self.w_qkv.shape[0], self.hidden, act) > 1
             qkv = linear_for_sum(h, self.w_qkv) if sliced else linear(h, self.w_qkv, act)
         cos, sin = self.position.tables(h.device)
         table = ctx.page_table(cache.group)
