@@ -334,7 +334,7 @@ def gemm_slices(M, N, K, dtype):
     tiles keep three k-tiles in flight, four slices are enough (and leave the reader fewer partial
     sums to add); measured at the shapes of an 8B model (N = 4096 and 6144, K = 4096 and 12288) for
     1, 8, 32 and 64 rows."""
-    if dtype != _BF16 or K % 8 != 0 or N > 8192 or K < 2048:
+    if dtype != _BF16 or K % 8 != 0 or N > 16384 or K < 2048:
         return 1
     if M > 64:
         # prompts: 256 x 256 tiles are the most efficient, but a narrow product has too few of them for
