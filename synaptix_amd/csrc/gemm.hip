@@ -837,7 +837,8 @@ static int launch_large(const bf16* x, const bf16* w, void* out, Epilogue ep, in
                         hipStream_t stream, int slices = 1);
 
 // Which of the large tiles for M > 64: 0 = 256 x 256, 1 = 256 x 192 (one workgroup of four waves a compute
-// unit; a fifth less efficient), 2 = 128 x 128 (two workgroups a compute unit, about as much less efficient).
+// unit; a fifth less efficient), 2 = 128 x 128 (two workgroups a compute unit, about as much less efficient),
+// 3 = 256 x 160 (four waves of 64 x 160; for N = 5120, which it cuts into 32 where 256 x 192 makes 27).
 // The estimate is the number of rounds over the 256 compute units times the work of a tile.  Measured
 // for N = 6144 and 24576 at 1,024 to 8,192 rows: the narrower tile wins where it fills a round that the
 // wide one leaves partly empty (q/k/v at 2,048 and 4,096 rows: 100 against 116 us, 181 against 198) and
@@ -846,12 +847,13 @@ static int launch_large(const bf16* x, const bf16* w, void* out, Epilogue ep, in
 static int pick_large_tile(int M, int N) {
   auto rounds = [](long tiles, long slots) { return (tiles + slots - 1) / slots; };
   auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-  const double cost[3] = {(double)rounds(tiles(256, 256), 256) * 256 * 256,
+  const double cost[4] = {(double)rounds(tiles(256, 256), 256) * 256 * 256,
                           (double)rounds(tiles(256, 192), 256) * 256 * 192 * 1.2,
-                          (double)rounds(tiles(128, 128), 512) * 2 * 128 * 128 * 1.2};
+                          (double)rounds(tiles(128, 128), 512) * 2 * 128 * 128 * 1.2,
+                          (double)rounds(tiles(256, 160), 256) * 256 * 160 * 1.2};
   int best = 0;
-  if (cost[1] < cost[best]) best = 1;
-  if (cost[2] < cost[best]) best = 2;
+  for (int i = 1; i < 4; ++i)
+    if (cost[i] < cost[best]) best = i;
   return best;
 }
 
@@ -864,10 +866,11 @@ static int launch_large(const bf16* x, const bf16* w, void* out, Epilogue ep, in
   if (K % 64 == 0) {
     if (shape == 0) return launch_pipelined<256, 256, 2, 4, PAIRED>(x, w, out, ep, M, N, K, stream);
     if (shape == 1) return launch_pipelined<256, 192, 2, 2, PAIRED>(x, w, out, ep, M, N, K, stream);
+    if (shape == 3) return launch_pipelined<256, 160, 4, 1, PAIRED>(x, w, out, ep, M, N, K, stream);
     return launch_pipelined<128, 128, 2, 2, PAIRED>(x, w, out, ep, M, N, K, stream);
   }
   if (shape == 0) return launch_tiled<256, 256, 64, 4, 2, PAIRED>(x, w, out, ep, M, N, K, stream);
-  if (shape == 1) return launch_tiled<256, 192, 64, 4, 2, PAIRED>(x, w, out, ep, M, N, K, stream);
+  if (shape == 1 || shape == 3) return launch_tiled<256, 192, 64, 4, 2, PAIRED>(x, w, out, ep, M, N, K, stream);
   return launch_tiled<128, 128, 64, 2, 2, PAIRED>(x, w, out, ep, M, N, K, stream);
 }
 

@@ -205,6 +205,7 @@ def test_gemm_f32(ops, M, N, K):
 @pytest.mark.parametrize("M,N,K", [
     (1, 48, 64), (3, 1000, 176), (16, 100, 320), (17, 40, 72), (33, 1000, 128), (48, 70, 2048), (64, 4096, 512),
     (65, 130, 104), (128, 128, 32), (200, 300, 1000), (513, 257, 4096),
+    (1700, 5120, 128),                  # the 256 x 160 tile: 32 tiles along N where 256 x 192 makes 27
     (5, 30, 20), (70, 50, 36),          # K no multiple of 8: the plain kernel takes them
     (2048, 6144, 512), (1000, 12300, 136),   # large enough for the 256 x 256 tiles with 8 waves, ragged edges
     (1000, 12544, 128), (300, 200, 64),   # K a multiple of 64: loads straight into LDS, every tile shape
@@ -266,7 +267,7 @@ def test_gemm_bf16_partial_sums_over_slices_of_k(ops, M, N, K, S):
                                    (1000, 6272, 128), (300, 400, 192),
                                    # 65 to 256 rows: all of x in one tile of 128, 192 or 256 rows and 96 or 128 rows of W
                                    (65, 48, 64), (100, 1040, 448), (128, 12288, 512), (129, 400, 192), (192, 2000, 320),
-                                   (193, 80, 1024), (256, 4864, 640), (200, 400, 72)])
+                                   (193, 80, 1024), (256, 4864, 640), (200, 400, 72), (1700, 2560, 192)])
 def test_gemm_with_the_gated_activation_inside(ops, M, I, K):
     """silu(x . Wg^T) * (x . Wu^T) from one product over the rows of Wg and Wu in turns of 16,
     against the two products and the activation in 64-bit; every tile shape of the kernel."""
