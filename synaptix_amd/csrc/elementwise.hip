@@ -374,16 +374,16 @@ __global__ void qk_norm_rope_kv_write_kernel(const TIn* __restrict__ qkv, int n_
 // PARTS: the rows come as n_parts float partial sums [n_parts][tokens][heads * HD] of a product cut
 // along K (part_stride elements apart), which are added first, in their order.
 template <int LPH, bool PARTS>
-__global__ void __launch_bounds__(256)
-qk_heads_kernel(const void* __restrict__ qkv_in, int n_parts, size_t part_stride, bf16* __restrict__ q_out,
-                bf16* __restrict__ k_pages,
+__device__ __forceinline__ void
+qk_heads_part(int block_x, int block_y, const void* __restrict__ qkv_in, int n_parts, size_t part_stride,
+              bf16* __restrict__ q_out, bf16* __restrict__ k_pages,
                 const int* __restrict__ page_table, int table_stride, const int* __restrict__ tok_seq,
                 const int* __restrict__ tok_pos, const void* __restrict__ q_gain, const void* __restrict__ k_gain,
                 int gain_is_f32, float gain_offset, float eps, const float* __restrict__ cos_t,
                 const float* __restrict__ sin_t, int n_tokens, int nh, int nkv, int n_active) {
   constexpr int HD = LPH * 8, HPB = 256 / LPH, half = HD / 2;
   constexpr int TPB = 4;  // tokens a block takes, their loads in flight together
-  const int head_raw = blockIdx.y * HPB + threadIdx.x / LPH;  // q heads, then k heads
+  const int head_raw = block_y * HPB + threadIdx.x / LPH;  // q heads, then k heads
   const int head = min(head_raw, n_active - 1);                // idle lanes repeat the last head: shuffles need them
   const int c = threadIdx.x % LPH;                             // which 8 values of the head
   const bool is_q = head < nh, low = c < LPH / 2;
@@ -409,13 +409,13 @@ qk_heads_kernel(const void* __restrict__ qkv_in, int n_parts, size_t part_stride
     for (int t = 0; t < TPB; ++t) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) val[t][e] = 0.f;
-      pos[t] = tok_pos[min((int)blockIdx.x * TPB + t, n_tokens - 1)];
+      pos[t] = tok_pos[min(block_x * TPB + t, n_tokens - 1)];
     }
     for (int p = 0; p < n_parts; ++p) {
       float4 lo4[TPB], hi4[TPB];     // the tokens' loads of one part in flight together
 #pragma unroll
       for (int t = 0; t < TPB; ++t) {
-        const int tok = min((int)blockIdx.x * TPB + t, n_tokens - 1);
+        const int tok = min(block_x * TPB + t, n_tokens - 1);
         const float4* src = (const float4*)((const float*)qkv_in + (size_t)p * part_stride +
                                             ((size_t)tok * (nh + 2 * nkv) + head) * HD + c * 8);
         lo4[t] = src[0], hi4[t] = src[1];
@@ -430,7 +430,7 @@ qk_heads_kernel(const void* __restrict__ qkv_in, int n_parts, size_t part_stride
     bf16x8 raw[TPB];
 #pragma unroll
     for (int t = 0; t < TPB; ++t) {
-      const int tok = min((int)blockIdx.x * TPB + t, n_tokens - 1);
+      const int tok = min(block_x * TPB + t, n_tokens - 1);
       raw[t] = *(const bf16x8*)((const bf16*)qkv_in + ((size_t)tok * (nh + 2 * nkv) + head) * HD + c * 8);
       pos[t] = tok_pos[tok];
     }
@@ -449,7 +449,7 @@ qk_heads_kernel(const void* __restrict__ qkv_in, int n_parts, size_t part_stride
   }
 #pragma unroll
   for (int t = 0; t < TPB; ++t) {
-    const int tok = (int)blockIdx.x * TPB + t;
+    const int tok = block_x * TPB + t;
     float v[8];
     float ss = 0.f;
 #pragma unroll
@@ -490,17 +490,17 @@ qk_heads_kernel(const void* __restrict__ qkv_in, int n_parts, size_t part_stride
 // order of v_page_offset, in which 8 consecutive positions of one dim are one 16-byte piece and the
 // 16 dims of a fragment follow each other at 16 bytes.
 #define V_DIMS 32
-template <bool PARTS>   // as for qk_heads_kernel
-__global__ void __launch_bounds__(256)
-v_block_write_kernel(const void* __restrict__ qkv_in, int n_parts, size_t part_stride, bf16* __restrict__ v_pages,
-                     const int* __restrict__ page_table,
+template <bool PARTS>   // as for qk_heads_part
+__device__ __forceinline__ void
+v_block_write_part(int block_x, int block_y, int block_z, const void* __restrict__ qkv_in, int n_parts,
+                   size_t part_stride, bf16* __restrict__ v_pages, const int* __restrict__ page_table,
                      int table_stride, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, int n_tokens,
                      int nh, int nkv, int hd) {
   constexpr int LD = V_DIMS + 2, PAIRS = V_DIMS / 2;
   __shared__ __attribute__((aligned(16))) bf16 vtile[64 * LD];
   __shared__ size_t dst_base[SYN_PAGE];
   __shared__ int dst_slot[SYN_PAGE];
-  const int tid = threadIdx.x, t0 = blockIdx.x * 64, kvh = blockIdx.y, d0 = blockIdx.z * V_DIMS;
+  const int tid = threadIdx.x, t0 = block_x * 64, kvh = block_y, d0 = block_z * V_DIMS;
   const int heads = nh + 2 * nkv;
   for (int idx = tid; idx < 64 * PAIRS; idx += 256) {
     const int j = idx / PAIRS, pr = idx % PAIRS;
@@ -531,6 +531,28 @@ v_block_write_kernel(const void* __restrict__ qkv_in, int n_parts, size_t part_s
       v_pages[dst_base[j] + v_page_offset(hd, d0 + d, dst_slot[j])] = vtile[j * LD + d];
 }
 
+// Both in one launch: the first qk_x * qk_y workgroups take the q and k heads, the others the v tiles
+// (v_x * nkv * v_z of them, none where the layer writes no cache).
+template <int LPH, bool PARTS>
+__global__ void __launch_bounds__(256)
+qkv_prompt_kernel(int qk_x, int qk_y, int v_x, const void* __restrict__ qkv, int n_parts, size_t part_stride,
+                  bf16* __restrict__ q_out, bf16* __restrict__ k_pages, bf16* __restrict__ v_pages,
+                  const int* __restrict__ page_table, int table_stride, const int* __restrict__ tok_seq,
+                  const int* __restrict__ tok_pos, const void* __restrict__ q_gain, const void* __restrict__ k_gain,
+                  int gain_is_f32, float gain_offset, float eps, const float* __restrict__ cos_t,
+                  const float* __restrict__ sin_t, int n_tokens, int nh, int nkv, int n_active) {
+  const int b = blockIdx.x, n_qk = qk_x * qk_y;
+  if (b < n_qk) {
+    qk_heads_part<LPH, PARTS>(b % qk_x, b / qk_x, qkv, n_parts, part_stride, q_out, k_pages, page_table, table_stride,
+                              tok_seq, tok_pos, q_gain, k_gain, gain_is_f32, gain_offset, eps, cos_t, sin_t, n_tokens,
+                              nh, nkv, n_active);
+  } else {
+    const int c = b - n_qk;
+    v_block_write_part<PARTS>(c % v_x, (c / v_x) % nkv, c / (v_x * nkv), qkv, n_parts, part_stride, v_pages, page_table,
+                              table_stride, tok_seq, tok_pos, n_tokens, nh, nkv, LPH * 8);
+  }
+}
+
 SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, int n_parts, void* q_out, void* k_pages, void* v_pages,
                                          int is_f32, const int* page_table, int table_stride, const int* tok_seq,
                                          const int* tok_pos, const void* q_gain, const void* k_gain, int gain_is_f32,
@@ -544,7 +566,7 @@ SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, int n_parts, void* q_o
   SYN_CHECK(n_parts >= 0 && n_parts <= 64, "qk_norm_rope_kv_write: %d partial sums", n_parts);
   // prompts in bf16: the kernels that move 16 bytes a lane, where the head size and the rotation allow them
   const int lph = hd / 8;
-  // (partial sums of up to 64 tokens stay with the one kernel below: two launches cost more than it takes)
+  // (partial sums of up to 64 tokens stay with the kernel below, one wave a head: measured a little faster there)
   const bool fast = !is_f32 && (n_parts == 0 || n_tokens > 64) && hd % 8 == 0 && lph >= 2 && lph <= 32 && (lph & (lph - 1)) == 0 &&
                     (cos_t == nullptr || rot == hd) && (uintptr_t)qkv % 16 == 0 && (uintptr_t)q_out % 16 == 0 &&
                     (uintptr_t)k_pages % 16 == 0 && (uintptr_t)q_gain % 16 == 0 && (uintptr_t)k_gain % 16 == 0 &&
@@ -552,38 +574,30 @@ SYN_EXPORT int syn_qk_norm_rope_kv_write(const void* qkv, int n_parts, void* q_o
   if (fast) {
     const int n_active = write_kv ? nh + nkv : nh;
     const int hpb = 256 / lph;
-    const dim3 grid((n_tokens + 3) / 4, (n_active + hpb - 1) / hpb);
+    const int qk_x = (n_tokens + 3) / 4, qk_y = (n_active + hpb - 1) / hpb;
+    const int v_x = (n_tokens + 63) / 64, v_blocks = write_kv ? v_x * nkv * ((hd + V_DIMS - 1) / V_DIMS) : 0;
     const size_t part_stride = (size_t)n_tokens * (nh + 2 * nkv) * hd;
-#define SYN_QKH(L)                                                                                                  \
+    const long grid = (long)qk_x * qk_y + v_blocks;
+    SYN_CHECK(grid <= 0x7fffffffL, "qk_norm_rope_kv_write: %d tokens are too many for one launch", n_tokens);
+#define SYN_QKV(L)                                                                                                  \
   if (n_parts > 0)                                                                                                  \
-    qk_heads_kernel<L, true><<<grid, 256, 0, stream>>>(qkv, n_parts, part_stride, (bf16*)q_out, (bf16*)k_pages,    \
-                                                       page_table, table_stride, tok_seq, tok_pos, q_gain, k_gain, \
-                                                       gain_is_f32, gain_offset, eps, cos_t, sin_t, n_tokens, nh,  \
-                                                       nkv, n_active);                                              \
+    qkv_prompt_kernel<L, true><<<(unsigned)grid, 256, 0, stream>>>(                                                 \
+        qk_x, qk_y, v_x, qkv, n_parts, part_stride, (bf16*)q_out, (bf16*)k_pages, (bf16*)v_pages, page_table,       \
+        table_stride, tok_seq, tok_pos, q_gain, k_gain, gain_is_f32, gain_offset, eps, cos_t, sin_t, n_tokens, nh,  \
+        nkv, n_active);                                                                                             \
   else                                                                                                              \
-    qk_heads_kernel<L, false><<<grid, 256, 0, stream>>>(qkv, 0, 0, (bf16*)q_out, (bf16*)k_pages, page_table,       \
-                                                        table_stride, tok_seq, tok_pos, q_gain, k_gain,            \
-                                                        gain_is_f32, gain_offset, eps, cos_t, sin_t, n_tokens, nh, \
-                                                        nkv, n_active)
+    qkv_prompt_kernel<L, false><<<(unsigned)grid, 256, 0, stream>>>(                                                \
+        qk_x, qk_y, v_x, qkv, 0, 0, (bf16*)q_out, (bf16*)k_pages, (bf16*)v_pages, page_table, table_stride, tok_seq, \
+        tok_pos, q_gain, k_gain, gain_is_f32, gain_offset, eps, cos_t, sin_t, n_tokens, nh, nkv, n_active)
     switch (lph) {
-      case 2: SYN_QKH(2); break;
-      case 4: SYN_QKH(4); break;
-      case 8: SYN_QKH(8); break;
-      case 16: SYN_QKH(16); break;
-      default: SYN_QKH(32); break;
+      case 2: SYN_QKV(2); break;
+      case 4: SYN_QKV(4); break;
+      case 8: SYN_QKV(8); break;
+      case 16: SYN_QKV(16); break;
+      default: SYN_QKV(32); break;
     }
-#undef SYN_QKH
-    SYN_LAUNCH_CHECK("qk_heads");
-    if (write_kv) {
-      const dim3 vgrid((n_tokens + 63) / 64, nkv, (hd + V_DIMS - 1) / V_DIMS);
-      if (n_parts > 0)
-        v_block_write_kernel<true><<<vgrid, 256, 0, stream>>>(qkv, n_parts, part_stride, (bf16*)v_pages, page_table,
-                                                              table_stride, tok_seq, tok_pos, n_tokens, nh, nkv, hd);
-      else
-        v_block_write_kernel<false><<<vgrid, 256, 0, stream>>>(qkv, 0, 0, (bf16*)v_pages, page_table, table_stride,
-                                                               tok_seq, tok_pos, n_tokens, nh, nkv, hd);
-      SYN_LAUNCH_CHECK("v_block_write");
-    }
+#undef SYN_QKV
+    SYN_LAUNCH_CHECK("qkv_prompt");
     return 0;
   }
   const int wpb = 4;
