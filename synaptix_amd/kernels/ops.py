@@ -259,6 +259,7 @@ def gemm_swiglu(x, w_paired, out, activation="silu"):
 
 
 PACKED_MAX_ROWS = 8   # up to this many rows of x the products over packed weights are the faster ones
+PACKED_MAX_ROWS_GATED = 16   # the gated product, whose waves take two groups of rows of W for every fragment of x
 
 
 def pack_weight(w):

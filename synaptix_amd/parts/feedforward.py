@@ -52,7 +52,7 @@ class GatedMlp(FeedForward):
     def forward(self, h, ctx):
         m = torch.empty((h.shape[0], self.intermediate), dtype=h.dtype, device=h.device)
         if self.paired and h.dtype == torch.bfloat16:
-            if self.p_gate_up is not None and h.shape[0] <= ops.PACKED_MAX_ROWS:
+            if self.p_gate_up is not None and h.shape[0] <= ops.PACKED_MAX_ROWS_GATED:
                 ops.gemm_packed(h, self.p_gate_up, m, paired=True, activation=self.activation)
             else:
                 ops.gemm_swiglu(h, self.w_gate_up, m, self.activation)

@@ -318,7 +318,8 @@ def test_gemm_over_weights_in_fragment_order(ops, out_dtype, M, N, K):
         ops.gemm_packed(torch.zeros((17, K), dtype=BF16, device=DEV), wp, torch.empty((17, N), dtype=out_dtype, device=DEV))
 
 
-@pytest.mark.parametrize("M,I,K", [(1, 16, 32), (1, 2560, 4096), (8, 2560, 4096), (7, 112, 992), (4, 16400, 64)])
+@pytest.mark.parametrize("M,I,K", [(1, 16, 32), (1, 2560, 4096), (8, 2560, 4096), (7, 112, 992), (4, 16400, 64),
+                                   (9, 2560, 4096), (13, 48, 992), (16, 12288, 512)])       # up to 16 rows: the engine's limit for this product
 def test_gated_product_over_weights_in_fragment_order(ops, M, I, K):
     x, wg, wu = rnd((M, K), 28, BF16), rnd((I, K), 29, BF16), rnd((I, K), 30, BF16)
     wp = ops.pack_weight(ops.pair_rows(wg.to(DEV), wu.to(DEV)))
