@@ -1,4 +1,5 @@
-from .qwen3 import ConfigError, Qwen3Config
+from .errors import ConfigError
+from .qwen3 import Qwen3Config
 from .registry import (Architecture, register_architecture, resolve_architecture, known_architectures,
                        load_config, read_config_json)
 

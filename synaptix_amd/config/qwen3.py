@@ -16,9 +16,7 @@ from typing import Optional
 
 import numpy as np
 
-
-class ConfigError(ValueError):
-    """A config.json that cannot be read, parsed or honoured."""
+from .errors import ConfigError
 
 
 @dataclass(frozen=True)

@@ -11,7 +11,7 @@ import os
 from dataclasses import dataclass
 from typing import Callable
 
-from .qwen3 import ConfigError
+from .errors import ConfigError
 
 
 @dataclass(frozen=True)

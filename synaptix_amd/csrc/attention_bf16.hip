@@ -26,8 +26,6 @@
 //            A second kernel merges the splits when there is more than one.
 // Reference counterparts: flash_splitq.cu (prefill), flash_decode.cu:92-205,340-387 (split + merge,
 // one block a q-head there, scalar dot products).
-#include <mutex>
-
 #include "common.h"
 #include "no_alloc.h"
 
@@ -565,12 +563,12 @@ SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, co
   const int tiles = n_tokens / PF_ROWS + n_seqs;  // an upper bound; surplus workgroups leave at once
   SYN_CHECK(tiles <= 65535, "attention_prefill: %d tiles of %d rows exceed the grid", tiles, PF_ROWS);
   const size_t lds = (size_t)2 * PF_TILE * sizeof(bf16);
-  static bool raised = false;
-  if (lds > 65536 && !raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)lds);
+  static OncePerDevice raised;
+  if (lds > 65536) {
+    const hipError_t e = once_per_device(raised, [&] {
+      return hipFuncSetAttribute((const void*)attn_prefill_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    });
     SYN_CHECK(e == hipSuccess, "attention_prefill: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
-    raised = true;
   }
   if constexpr (PF2_OK) {
     if (variant == 2 || (variant == 0 && scale > 0.f)) {
@@ -1030,6 +1028,20 @@ attn_decode_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ o
   }
 }
 
+// the decode kernels may use all of a compute unit's LDS: asked for once on each device
+constexpr size_t DEC_LDS_MAX = 160 * 1024;
+static hipError_t raise_decode_lds() {
+  static OncePerDevice once;
+  return once_per_device(once, [] {
+    hipError_t e = hipFuncSetAttribute((const void*)attn_decode_split_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)DEC_LDS_MAX);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)attn_decode_split_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)DEC_LDS_MAX);
+    return e;
+  });
+}
+
 // workspace: n_seqs * nh * n_splits * (HD + 2) floats (unused with one split)
 static int launch_decode(const void* q, const QkvIntake* in, void* k_pages, void* v_pages, const int* page_table,
                          int table_stride, const int* seq_len, int n_seqs, void* out, float* workspace, int n_splits,
@@ -1047,20 +1059,14 @@ static int launch_decode(const void* q, const QkvIntake* in, void* k_pages, void
     if (in) b += ((size_t)waves * HD + 16) * sizeof(float) + (size_t)(cols_alloc + 2) * HD * sizeof(bf16);
     return b;
   };
-  constexpr size_t LDS_MAX = 160 * 1024;
+  constexpr size_t LDS_MAX = DEC_LDS_MAX;
   int waves = DEC_MAX_WAVES;
   while (waves > 2 && (lds_for(waves) > LDS_MAX || (long)n_seqs * nkv * chunks * n_splits * waves > 2048)) waves /= 2;
   if (waves < 4 && lds_for(4) <= LDS_MAX) waves = 4;
   const size_t lds = lds_for(waves);
   SYN_CHECK(lds <= LDS_MAX, "attention_decode: %zu bytes of LDS for %d heads a group", lds, nh / nkv);
-  static bool raised = false;
-  if (!raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)attn_decode_split_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)attn_decode_split_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_MAX);
-    SYN_CHECK(e == hipSuccess, "attention_decode: %zu bytes of LDS refused: %s", LDS_MAX, hipGetErrorString(e));
-    raised = true;
-  }
+  const hipError_t raised = raise_decode_lds();
+  SYN_CHECK(raised == hipSuccess, "attention_decode: %zu bytes of LDS refused: %s", LDS_MAX, hipGetErrorString(raised));
   const dim3 grid(n_seqs, nkv * chunks, n_splits);
   if (in)
     attn_decode_split_kernel<true><<<grid, waves * SYN_WAVE, lds, stream>>>(
@@ -1091,9 +1097,30 @@ SYN_EXPORT int syn_attention_decode_bf16(const void* q, const void* k_pages, con
 // an address to hand to a kernel.  Each GPU holds its own copy at its own address: the address is
 // looked up once per device, with that device current, and kept.
 static __device__ __align__(256) unsigned char scratch[SYN_NOALLOC_SCRATCH_BYTES];
-#define SYN_NOALLOC_MAX_DEVICES 64
-static float* scratch_of_device[SYN_NOALLOC_MAX_DEVICES];
-static std::mutex scratch_lock;
+static float* scratch_of_device[SYN_MAX_DEVICES];
+
+// What a first call on a device does besides launching: the address of this device's copy of the array, and
+// the decode kernels' LDS limit.  Neither is stream work, so neither may happen while a stream is captured:
+// callers that capture call this (or the entry point once) beforehand, with the device current.
+SYN_EXPORT int syn_attention_decode_noalloc_init() {
+  static OncePerDevice once;
+  hipError_t e = once_per_device(once, [] {
+    int dev = -1;
+    hipError_t r = hipGetDevice(&dev);
+    if (r != hipSuccess) return r;
+    void* p = nullptr;
+    r = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (r != hipSuccess) return r;
+    if (p == nullptr) return hipErrorInvalidSymbol;
+    scratch_of_device[dev] = (float*)p;   // once_per_device has checked dev and holds its lock
+    return hipSuccess;
+  });
+  SYN_CHECK(e == hipSuccess, "attention_decode_noalloc: the scratch array has no address on the current device: %s",
+            hipGetErrorString(e));
+  e = raise_decode_lds();
+  SYN_CHECK(e == hipSuccess, "attention_decode_noalloc: %zu bytes of LDS refused: %s", DEC_LDS_MAX, hipGetErrorString(e));
+  return 0;
+}
 
 SYN_EXPORT int syn_attention_decode_bf16_noalloc(const void* q, const void* k_pages, const void* v_pages,
                                                  const int* page_table, int table_stride, const int* seq_len,
@@ -1105,22 +1132,12 @@ SYN_EXPORT int syn_attention_decode_bf16_noalloc(const void* q, const void* k_pa
             "attention_decode_noalloc: %d sequences x %d heads x %d splits need %llu bytes of partial results, the "
             "library keeps %u; use fewer splits or the entry point with a workspace argument",
             n_seqs, nh, n_splits, need, (unsigned)SYN_NOALLOC_SCRATCH_BYTES);
+  if (const int rc = syn_attention_decode_noalloc_init()) return rc;   // after the first call on a device: two flag reads
   int dev = -1;
-  hipError_t e = hipGetDevice(&dev);
-  SYN_CHECK(e == hipSuccess && dev >= 0 && dev < SYN_NOALLOC_MAX_DEVICES, "attention_decode_noalloc: no current device (%s)",
+  const hipError_t e = hipGetDevice(&dev);
+  SYN_CHECK(e == hipSuccess && dev >= 0 && dev < SYN_MAX_DEVICES, "attention_decode_noalloc: no current device (%s)",
             hipGetErrorString(e));
-  float* ws;
-  {
-    std::lock_guard<std::mutex> hold(scratch_lock);
-    if (scratch_of_device[dev] == nullptr) {
-      void* p = nullptr;
-      e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-      SYN_CHECK(e == hipSuccess && p != nullptr, "attention_decode_noalloc: the scratch array has no address on device %d: %s",
-                dev, hipGetErrorString(e));
-      scratch_of_device[dev] = (float*)p;
-    }
-    ws = scratch_of_device[dev];
-  }
+  float* ws = scratch_of_device[dev];   // written once, before the flag that the init call has just read under its lock
   return launch_decode(q, nullptr, (void*)k_pages, (void*)v_pages, page_table, table_stride, seq_len, n_seqs, out, ws,
                        n_splits, scale, window, nh, nkv, hd, stream);
 }

@@ -6,6 +6,7 @@
 #include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <mutex>
 
 #define SYN_WAVE 64
 #define SYN_PAGE 64  // tokens per cache page; the host side asserts the same number
@@ -46,6 +47,28 @@ void syn_set_error(const char* fmt, ...);
       return 2;                                                         \
     }                                                                   \
   } while (0)
+
+// ---- once on each device ----
+// What has to happen once on a device before a kernel's first launch there (raising its limit of dynamic LDS,
+// looking up a device symbol): the flags are kept per device under a lock, so that two threads or two GPUs
+// neither skip the step nor run it twice.
+#define SYN_MAX_DEVICES 64
+struct OncePerDevice {
+  std::mutex lock;
+  bool done[SYN_MAX_DEVICES] = {};
+};
+template <typename F>
+static inline hipError_t once_per_device(OncePerDevice& once, F&& step) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= SYN_MAX_DEVICES) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> hold(once.lock);
+  if (once.done[dev]) return hipSuccess;
+  e = step();
+  if (e == hipSuccess) once.done[dev] = true;
+  return e;
+}
 
 // ---- conversions ----
 template <typename T> __device__ __forceinline__ float to_f32(T v);

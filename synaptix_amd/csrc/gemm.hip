@@ -507,15 +507,17 @@ static int launch_tiled(const bf16* x, const bf16* w, void* out, Epilogue ep, in
   const int k_slice = ((K + slices - 1) / slices + 127) / 128 * 128;  // the same cut as launch_direct makes
   const int grid = tile_grid(M, N, BM, BN);
   const size_t lds = (size_t)2 * (BM + BN) * (BK + 8) * sizeof(bf16);
-  static bool raised = false;
-  if (lds > 65536 && !raised) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, WM, WN, false, PAIRED>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, WM, WN, true, PAIRED>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  static OncePerDevice raised;
+  if (lds > 65536) {
+    const hipError_t e = once_per_device(raised, [&] {
+      hipError_t r = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, WM, WN, false, PAIRED>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (r == hipSuccess)
+        r = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, WM, WN, true, PAIRED>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      return r;
+    });
     SYN_CHECK(e == hipSuccess, "gemm: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
-    raised = true;
   }
   // whole k-tiles only, and no slice that begins at or beyond the end of K: then no chunk needs a check
   if (K % BK == 0 && k_slice % BK == 0 && (long)(slices - 1) * k_slice < K)
@@ -657,12 +659,13 @@ static int launch_direct(const bf16* x, const bf16* w, void* out, Epilogue ep, i
   const int step = BK > 128 ? BK : 128;
   const int k_slice = ((K + slices - 1) / slices + step - 1) / step * step;  // a multiple of BK
   const size_t lds = (size_t)STAGES * (BM + BN) * BK * sizeof(bf16);
-  static bool raised = false;
-  if (lds > 65536 && !raised) {
-    const hipError_t e = hipFuncSetAttribute((const void*)gemm_direct_kernel<BM, BN, BK, WM, WN, PAIRED, STAGES>,
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  static OncePerDevice raised;
+  if (lds > 65536) {
+    const hipError_t e = once_per_device(raised, [&] {
+      return hipFuncSetAttribute((const void*)gemm_direct_kernel<BM, BN, BK, WM, WN, PAIRED, STAGES>,
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    });
     SYN_CHECK(e == hipSuccess, "gemm: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
-    raised = true;
   }
   gemm_direct_kernel<BM, BN, BK, WM, WN, PAIRED, STAGES>
       <<<dim3(tile_grid(M, N, BM, BN), slices), 64 * WM * WN, lds, stream>>>(x, w, out, ep, M, N, K, k_slice);
@@ -819,12 +822,13 @@ static int launch_pipelined(const bf16* x, const bf16* w, void* out, Epilogue ep
   const int k_slice = ((K + slices - 1) / slices + 127) / 128 * 128;  // the same cut as the tiles for few rows make
   SYN_CHECK((long)(slices - 1) * k_slice < K, "gemm: %d slices of %d leave the last one empty (K = %d)", slices, k_slice, K);
   const size_t lds = (size_t)2 * (BM + BN) * 64 * sizeof(bf16);
-  static bool raised = false;
-  if (lds > 65536 && !raised) {
-    const hipError_t e = hipFuncSetAttribute((const void*)gemm_pipelined_kernel<BM, BN, WM, WN, PAIRED>,
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  static OncePerDevice raised;
+  if (lds > 65536) {
+    const hipError_t e = once_per_device(raised, [&] {
+      return hipFuncSetAttribute((const void*)gemm_pipelined_kernel<BM, BN, WM, WN, PAIRED>,
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    });
     SYN_CHECK(e == hipSuccess, "gemm: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
-    raised = true;
   }
   gemm_pipelined_kernel<BM, BN, WM, WN, PAIRED>
       <<<dim3(tile_grid(M, N, BM, BN), slices), 64 * WM * WN, lds, stream>>>(x, w, out, ep, M, N, K, k_slice);
@@ -835,6 +839,22 @@ static int launch_pipelined(const bf16* x, const bf16* w, void* out, Epilogue ep
 template <bool PAIRED>
 static int launch_large(const bf16* x, const bf16* w, void* out, Epilogue ep, int M, int N, int K,
                         hipStream_t stream, int slices = 1);
+
+// Compute units of the current device (256 on an MI355X), asked once a device: what the rules for tiles fill.
+// The host's rules for slices of K ask the same number (kernels/ops.py: compute_units).
+static int compute_units() {
+  static int of_device[SYN_MAX_DEVICES];
+  static OncePerDevice once;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= SYN_MAX_DEVICES) return 256;
+  const hipError_t e = once_per_device(once, [&] {
+    int n = 0;
+    const hipError_t r = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    of_device[dev] = (r == hipSuccess && n > 0) ? n : 256;
+    return hipSuccess;
+  });
+  return e == hipSuccess ? of_device[dev] : 256;
+}
 
 // Which of the large tiles for M > 64: 0 = 256 x 256, 1 = 256 x 192 (one workgroup of four waves a compute
 // unit; a fifth less efficient), 2 = 128 x 128 (two workgroups a compute unit, about as much less efficient),
@@ -847,10 +867,11 @@ static int launch_large(const bf16* x, const bf16* w, void* out, Epilogue ep, in
 static int pick_large_tile(int M, int N) {
   auto rounds = [](long tiles, long slots) { return (tiles + slots - 1) / slots; };
   auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-  const double cost[4] = {(double)rounds(tiles(256, 256), 256) * 256 * 256,
-                          (double)rounds(tiles(256, 192), 256) * 256 * 192 * 1.2,
-                          (double)rounds(tiles(128, 128), 512) * 2 * 128 * 128 * 1.2,
-                          (double)rounds(tiles(256, 160), 256) * 256 * 160 * 1.2};
+  const long cus = compute_units();
+  const double cost[4] = {(double)rounds(tiles(256, 256), cus) * 256 * 256,
+                          (double)rounds(tiles(256, 192), cus) * 256 * 192 * 1.2,
+                          (double)rounds(tiles(128, 128), 2 * cus) * 2 * 128 * 128 * 1.2,
+                          (double)rounds(tiles(256, 160), cus) * 256 * 160 * 1.2};
   int best = 0;
   for (int i = 1; i < 4; ++i)
     if (cost[i] < cost[best]) best = i;
@@ -913,7 +934,7 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
   // (cut along K the tiles are 128 x 128 up to 256 rows and 256 x 128 beyond)
   const long tiles_cut = (long)(M <= 256 ? (M + 127) / 128 : (M + 255) / 256) * ((N + 127) / 128);
-  const bool few_large_tiles = M > 64 && M <= 512 && K % 128 == 0 && (slices > 1 ? tiles_cut : tiles128) * slices <= 256;
+  const bool few_large_tiles = M > 64 && M <= 512 && K % 128 == 0 && (slices > 1 ? tiles_cut : tiles128) * slices <= compute_units();
   int rc = 0;
   if (M == 1 && slices == 1) {
     // one row: fragments of W straight from memory, K split over the waves

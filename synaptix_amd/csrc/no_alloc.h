@@ -13,7 +13,10 @@
 //     GPU that the library runs on, held until the process ends); a larger call is refused with an
 //     error text and launches nothing.
 //   * The call allocates and frees nothing, on the device or through any library.  The address of
-//     the array is looked up once per device, at the first call on that device.
+//     the array is looked up once per device (and the decode kernels' LDS limit raised there), by
+//     syn_attention_decode_noalloc_init or else at the first call on that device.  Neither is stream
+//     work and neither may happen while a stream is captured: a caller that captures calls the init
+//     (or the entry point once) on that device beforehand.
 //   * All calls on one GPU share that GPU's array, which keeps the last call's contents.  Nothing
 //     in it has to start at zero: every split of every (sequence, head) writes its maximum, its sum
 //     and its values before the merge reads them, an empty split writes a maximum of -inf.  Two
@@ -23,6 +26,9 @@
 #include <hip/hip_runtime.h>
 
 #define SYN_NOALLOC_SCRATCH_BYTES (8u << 20)
+
+// 0, or a code after an error text (syn_last_error): with the device current, before any capture
+extern "C" __attribute__((visibility("default"))) int syn_attention_decode_noalloc_init();
 
 extern "C" __attribute__((visibility("default"))) int syn_attention_decode_bf16_noalloc(
     const void* q, const void* k_pages, const void* v_pages, const int* page_table, int table_stride,

@@ -60,7 +60,8 @@ class Engine:
         from ..parts.base import StateNeed
         # a captured step is run more than once while it is recorded: only steps that write the
         # same values again may be captured, which a mixer with a running state is not
-        self.graph_ok = not any(isinstance(n, StateNeed) for n in model.cache_needs())
+        self.has_states = any(isinstance(n, StateNeed) for n in model.cache_needs())
+        self.graph_ok = not self.has_states
 
     # ------------------------------------------------------------------ construction
     @classmethod

@@ -53,25 +53,31 @@ class GenerationStats:
 
 
 def plan_batch(waiting: list, prompt_lens: list, max_new: list, free_slots: int, free_pages: int,
-               max_batch: int | None, capacity: int | None) -> list:
+               max_batch: int | None, capacity: int | None, held: dict | None = None) -> list:
     """Which of the waiting requests (indices, in order) start together now.
 
     A request needs a slot and pages for its prompt and all tokens it may produce, so that a
     batch never runs out of pages half way.  Requests are not reordered: the first that does not
     fit ends the batch.  A request that can never fit raises ValueError.
+    held: {request: tokens it keeps in a slot of its own}: such a request needs no slot and only the pages
+    beyond those that its kept tokens lie in.
     """
-    chosen, pages = [], 0
+    chosen, pages, slots = [], 0, 0
     for r in waiting:
         total = prompt_lens[r] + max(max_new[r], 1)
         if capacity is not None:
             total = min(total, capacity)
         need = pages_for(total)
+        own_slot = held is not None and r in held
+        if own_slot:
+            need = max(0, need - pages_for(held[r]))
         if max_batch is not None and len(chosen) >= max_batch:
             break
-        if len(chosen) >= free_slots or pages + need > free_pages:
+        if (not own_slot and slots >= free_slots) or pages + need > free_pages:
             break
         chosen.append(r)
         pages += need
+        slots += 0 if own_slot else 1
     if not chosen and waiting:
         r = waiting[0]
         raise ValueError(f"request {r} ({prompt_lens[r]} prompt tokens + {max_new[r]} new) does not fit the cache "
@@ -99,19 +105,32 @@ def graph_step(engine, live, longest):
 
 
 class _Live:
-    def __init__(self, request, slot, prompt, config, sampler):
+    def __init__(self, request, slot, prompt, config, sampler, kept=0, owned=True):
         self.request, self.slot, self.prompt, self.config, self.sampler = request, slot, prompt, config, sampler
+        self.kept, self.owned = kept, owned     # prompt tokens that the slot already holds; whether the loop gives the slot back
         self.out = []
         self.stop = config.stop_set()
         self.finish = None
 
 
-def generate(engine, prompts, config=None, on_token=None, max_batch: int | None = None, use_graph: bool = True):
+def generate(engine, prompts, config=None, on_token=None, max_batch: int | None = None, use_graph: bool = True,
+             resume: dict | None = None):
     """prompts: a list of token-id lists.  config: one GenerationConfig for all, or one each
     (with one for all, request i draws from the stream of seed + i).  on_token(request, token)
     -> bool: False cancels that request.  use_graph: decode steps are replayed from a captured
     graph where the engine allows it (the reference's --no-graph switches the same thing off).
+    resume: {request: slot}: the caller holds that slot, and the tokens it caches are the beginning of the
+    request's prompt (the caller vouches for that, as in the reference's generate_streaming_resume,
+    crates/synaptix-models/llm/common/src/generate.rs:233-250): min(cached, prompt - 1) of them are kept, only
+    the rest of the prompt is run, new tokens go into the same slot, and the slot stays with the caller.
     Returns ([GenerationOutput], GenerationStats)."""
+    resume = dict(resume or {})
+    for r, slot in resume.items():
+        if not (0 <= r < len(prompts)):
+            raise ValueError(f"resume names request {r}; there are {len(prompts)}")
+        engine.length(slot)                       # raises for a slot that is not held
+    if len(set(resume.values())) != len(resume):
+        raise ValueError("resume: two requests name the same slot")
     if config is None:
         config = GenerationConfig()
     shared = isinstance(config, GenerationConfig)
@@ -134,21 +153,33 @@ def generate(engine, prompts, config=None, on_token=None, max_batch: int | None 
         caps = [c for c in (engine.max_positions, seq.config.max_seq) if c is not None]
         return min(caps) if caps else None
 
+    def kept_tokens(r):
+        return min(engine.length(resume[r]), lens[r] - 1)
+
     while waiting:
         free_pages = min(g.pool.free_pages for g in engine.cache.groups) if engine.cache.groups else 1 << 30
         batch = plan_batch(waiting, lens, max_new, engine.cache.free_slots, free_pages, max_batch,
-                           engine.max_positions)
+                           engine.max_positions, held={r: kept_tokens(r) for r in waiting if r in resume})
         waiting = waiting[len(batch):]
         stats.batches += 1
         live = []
         for r in batch:
             seed = configs[r].seed + r if shared else configs[r].seed
-            live.append(_Live(r, engine.acquire(), list(prompts[r]), configs[r],
-                              SequenceSampler(configs[r], prompts[r], seed)))
+            sampler = SequenceSampler(configs[r], prompts[r], seed)
+            if r in resume:
+                kept = kept_tokens(r)
+                if kept < engine.length(resume[r]):
+                    if getattr(engine, "has_states", False):     # a running state cannot be rewound by a length
+                        raise ValueError(f"request {r}: its slot holds {engine.length(resume[r])} tokens and a state of "
+                                         f"fixed size; restore a snapshot taken at {kept} tokens or fewer first")
+                    engine.cache.truncate(resume[r], kept)
+                live.append(_Live(r, resume[r], list(prompts[r]), configs[r], sampler, kept=kept, owned=False))
+            else:
+                live.append(_Live(r, engine.acquire(), list(prompts[r]), configs[r], sampler))
         try:
             # ---- the prompts, in one step (or in chunks of prefill_batch tokens each)
             t0 = time.perf_counter()
-            fed = [0] * len(live)
+            fed = [s.kept for s in live]
             logits_rows = {}
             while True:
                 entries, who = [], []
@@ -195,7 +226,8 @@ def generate(engine, prompts, config=None, on_token=None, max_batch: int | None 
                         still.append(s)
                     else:
                         outputs[s.request] = GenerationOutput(s.out, s.finish, len(s.prompt))
-                        engine.release(s.slot)           # at once: the slot is free for the next batch
+                        if s.owned:
+                            engine.release(s.slot)       # at once: the slot is free for the next batch
                         s.slot = None
                 live = still
                 if not live:
@@ -215,7 +247,7 @@ def generate(engine, prompts, config=None, on_token=None, max_batch: int | None 
             stats.decode_ms += (time.perf_counter() - t1) * 1000.0
         finally:
             for s in live:
-                if s.slot is not None:
+                if s.slot is not None and s.owned:
                     engine.release(s.slot)
     stats.new_tokens = sum(len(o.tokens) for o in outputs if o is not None)
     return outputs, stats

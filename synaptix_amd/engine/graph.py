@@ -83,8 +83,7 @@ class DecodeRunner:
             raise ops.KernelError("op_timing: per-op times need eager steps; a captured decode step cannot be timed op by op")
         if B > self.rows:
             raise ValueError(f"{B} sequences for a graph of {self.rows} rows")
-        for s in slots:
-            eng.cache.reserve(s, 1)
+        eng.cache.reserve_step(slots, [1] * B)        # all pages of the step, or none
         i = self.turn
         self.turn ^= 1
         if self.copied[i] is not None:

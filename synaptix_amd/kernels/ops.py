@@ -302,7 +302,18 @@ def gemm_packed(x, wp, out, paired=False, activation="silu"):
           M, N, K, 1 if paired else 0, activation_code(activation), slices, _stream())
 
 
-N_COMPUTE_UNITS = 256     # of the MI355X: what the rules below fill
+_compute_units = None
+
+
+def compute_units() -> int:
+    """Compute units of the GPU that the rules below fill: asked of the device once (256 on an MI355X, which is also
+    what the rules assume where no GPU is present, as in tests of the rules themselves).  The C side asks the
+    device the same question (csrc/gemm.hip: compute_units)."""
+    global _compute_units
+    if _compute_units is None:
+        _compute_units = (torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+                          if torch.cuda.is_available() else 256)
+    return _compute_units
 
 
 def packed_slices(N, K):
@@ -311,11 +322,11 @@ def packed_slices(N, K):
     multiple of the compute units the last round runs half empty (N = 5120: 320 workgroups, two rounds for
     the work of 1.25; N = 2560: 160 compute units of 256).  The smallest cut that fills its rounds to 90 %
     is taken, if one exists among up to 8 slices of at least 1,024."""
-    groups = -(-N // 16)
+    groups, units = -(-N // 16), compute_units()
 
     def fill(s):
-        work = groups * s / N_COMPUTE_UNITS
-        return work / -(-groups * s // N_COMPUTE_UNITS)
+        work = groups * s / units
+        return work / -(-groups * s // units)
 
     best = 1
     for s in (1, 2, 3, 4, 5, 6, 8):
@@ -337,6 +348,7 @@ def gemm_slices(M, N, K, dtype):
     1, 8, 32 and 64 rows."""
     if dtype != _BF16 or K % 8 != 0 or N > 16384 or K < 2048:
         return 1
+    units = compute_units()
     if M > 64:
         # prompts: 256 x 256 tiles are the most efficient, but a narrow product has too few of them for
         # the 256 compute units (128 at 2,048 rows and N = 4096); two or four slices of K fill the chip,
@@ -347,19 +359,19 @@ def gemm_slices(M, N, K, dtype):
             # short prompts: still bound by reading W; tiles of 128 rows of W (and of 128 rows of x up to 256 rows,
             # of 256 beyond), cut until they fill the compute units
             tiles = (-(-M // 128) if M <= 256 else -(-M // 256)) * -(-N // 128)
-            most, slices = min(8, N_COMPUTE_UNITS // tiles, K // 512), 1
+            most, slices = min(8, units // tiles, K // 512), 1
             while slices * 2 <= most:
                 slices *= 2
             if slices > 1:
                 return slices
         tiles = -(-M // 256) * -(-N // 256)
-        return 4 if tiles * 4 <= 256 and K >= 8192 else (2 if tiles * 2 <= 256 else 1)
+        return 4 if tiles * 4 <= units and K >= 8192 else (2 if tiles * 2 <= units else 1)
     if M <= 32:
         # 64 rows of W a workgroup, up to three workgroups a compute unit
-        most = min(4, 768 // -(-N // 64), K // 512)
+        most = min(4, 3 * units // -(-N // 64), K // 512)
     else:
         # 128 rows of W a workgroup, one workgroup a compute unit
-        most = min(8, N_COMPUTE_UNITS // -(-N // 128), K // 512)
+        most = min(8, units // -(-N // 128), K // 512)
     slices = 1
     while slices * 2 <= most:
         slices *= 2

@@ -126,3 +126,35 @@ def test_single_tokens_give_the_same_logits_with_and_without_packed_weight_copie
         eng.step([(s, toks[:9])], want=None)
         got.append(torch.cat([eng.step([(s, [t])], want="last") for t in toks[9:]]))
     assert float((got[0] - got[1]).abs().max()) <= 2e-2
+
+
+def test_generation_that_resumes_a_kept_prefix_equals_a_fresh_one():
+    """The reference's prefix_cache_resume_matches_fresh (crates/synaptix-models/llm/qwen3/src/pipeline.rs:395-424): half
+    of the prompt is run into a slot beforehand; generation that resumes there runs only the other half and gives
+    the fresh run's greedy tokens.  A slot that holds more than the prompt is cut back to prompt - 1 tokens; the
+    slot stays with the caller and holds everything that was run."""
+    from synaptix_amd.engine.generate import generate, GenerationConfig
+    eng = make_engine("C", "float32", 1024, sharp=True)
+    V = CONFIGS["C"]["vocab_size"]
+    full = scenarios.random_tokens(V, 90, 4)          # crosses a page edge
+    other = scenarios.random_tokens(V, 20, 5)
+    cfg = GenerationConfig(max_new_tokens=6, temperature=0.0)
+    fresh, _ = generate(eng, [full, other], cfg)
+    slot = eng.acquire()
+    eng.step([(slot, full[:45])], want=None)
+    steps = []
+    step = eng.step
+    eng.step = lambda entries, want="last": (steps.append([(s_, len(t)) for s_, t in entries]), step(entries, want))[1]
+    resumed, st = generate(eng, [full, other], cfg, resume={0: slot})
+    assert [o.tokens for o in resumed] == [o.tokens for o in fresh]
+    assert (slot, 45) in steps[0] and st.prompt_tokens == 110           # only the tail of the resumed prompt was run
+    assert eng.length(slot) == 90 + 5                                   # the last token has not been run yet
+    # the slot now holds more than the prompt: all but the prompt's last token is kept, one token is run
+    steps.clear()
+    again, _ = generate(eng, [full], cfg, resume={0: slot})
+    assert again[0].tokens == fresh[0].tokens and steps[0] == [(slot, 1)]
+    eng.release(slot)
+    eng.cache.check()
+    assert not eng.cache.live_slots()
+    with pytest.raises(CacheError):
+        generate(eng, [full], cfg, resume={0: slot})                    # a slot that is not held

@@ -68,6 +68,34 @@ def test_rope_is_complex_multiplication_of_split_pairs(theta, hd):
     assert torch.allclose(y[:half], zr.real, atol=1e-12) and torch.allclose(y[half:], zr.imag, atol=1e-12)
 
 
+def test_rope_is_the_split_case_that_the_reference_checks_its_own_rotation_against():
+    """The reference tests its Split rotation (the only layout its decoder calls,
+    crates/synaptix-models/llm/common/src/model.rs:2555-2561) against a case made by
+    scripts/reference/gen_pos.py:27-58 (crates/synaptix-ops/tests/ref_pos.rs:13-25, to 1e-5): seed 0, q and k
+    [2, 8, 32, 64], full-width tables cos|cos and sin|sin, out = x * cos + cat(-x2, x1) * sin.  The case's data
+    file is not among the reference's files; its recipe is, and the plain rotation equals it.  The interleaved
+    pairing differs from it by more than 1."""
+    torch.manual_seed(0)
+    batch, heads, seq, hd = 2, 8, 32, 64
+    q = torch.randn(batch, heads, seq, hd, dtype=torch.float32)
+    k = torch.randn(batch, heads, seq, hd, dtype=torch.float32)
+    theta = 10000.0 ** (-torch.arange(0, hd, 2, dtype=torch.float32) / hd)
+    freqs = torch.outer(torch.arange(seq, dtype=torch.float32), theta)
+    cos_full, sin_full = freqs.cos().repeat(1, 2), freqs.sin().repeat(1, 2)
+    cos, sin = P.rope_tables(hd, seq, 10000.0)
+    for x in (q, k):
+        half = hd // 2
+        want = x * cos_full + torch.cat([-x[..., half:], x[..., :half]], -1) * sin_full
+        # the plain function takes [S, n, hd]: tokens first
+        got = torch.stack([P.apply_rope(x[b].transpose(0, 1), cos, sin, list(range(seq))).transpose(0, 1)
+                           for b in range(batch)])
+        assert torch.allclose(got, want, atol=1e-5, rtol=1e-5)
+        pairs = x.reshape(batch, heads, seq, half, 2)          # what an interleaved pairing would turn
+        c, s_ = freqs.cos(), freqs.sin()
+        inter = torch.stack([pairs[..., 0] * c - pairs[..., 1] * s_, pairs[..., 0] * s_ + pairs[..., 1] * c], -1)
+        assert (inter.reshape(x.shape) - want).abs().max() > 1.0
+
+
 def test_rope_scores_depend_on_distance_only():
     cos, sin = P.rope_tables(32, 200, 1e6, F64)
     q, k = rnd((1, 1, 32), 4, F64), rnd((1, 1, 32), 5, F64)
