@@ -155,6 +155,6 @@ def test_generation_that_resumes_a_kept_prefix_equals_a_fresh_one():
     assert again[0].tokens == fresh[0].tokens and steps[0] == [(slot, 1)]
     eng.release(slot)
     eng.cache.check()
-    assert not eng.cache.live_slots()
+    assert not eng.cache.live_slots
     with pytest.raises(CacheError):
         generate(eng, [full], cfg, resume={0: slot})                    # a slot that is not held
