@@ -169,6 +169,76 @@ static void launch_skinny(const bf16* x, const bf16* w, void* out, Epilogue ep, 
       <<<(N + rows - 1) / rows, TILES * KWAVES * SYN_WAVE, 0, stream>>>(x, w, out, ep, M, N, K);
 }
 
+// ------------------------------------------------------------------ a norm between two products for few rows
+// RMSNorm between two products for few rows of x needs every element of a row, which no workgroup of the product
+// before it holds; as a kernel of its own it moves a few KB and costs a launch.  The products over packed
+// weights therefore carry it between them in two halves:
+//   * the product BEFORE the norm (resid != null; one slice of K, float sums) adds its sums into the float residual
+//     rows, stores xs[m, n] = bf16((gain_offset + gain[n]) * resid[m, n]) (the norm's input with the gain, without
+//     the row's factor) and, for each group of 16 columns, ss_out[m, group] = the sum of resid[m, n]^2 over them;
+//   * the product AFTER the norm (ss != null) takes xs as its x and multiplies its finished sums of row m by
+//     rsqrt(sum over groups of ss[m, :] / dim + eps): the product is linear in x, so the row's factor can wait.
+// A row's statistic is added up in a fixed order (groups in turn over the lanes, then the wave's tree).
+struct RowNorm {
+  const float* ss;    // [M, ss_groups] of the product before, or null
+  int ss_groups;
+  float inv_dim;      // 1 / width of the normed rows
+  float eps;
+  float* resid;       // [M, N] float, or null
+  bf16* xs;           // [M, N]
+  float* ss_out;      // [M, N / 16]
+  const void* gain;   // [N] bf16 or float
+  int gain_is_f32;
+  float gain_offset;
+};
+
+// inv[m] for the rows of x into LDS (16 floats): wave w takes rows w and w + n_waves (up to 16 rows, 8 waves or more).
+// The statistic's first 256 groups a row are asked for before the product's loop (row_stat_load) and added up behind
+// it (row_stat_finish), so that their way from memory is not the tail of the workgroup.
+struct RowStat {
+  float v[2][4];
+};
+__device__ __forceinline__ void row_stat_load(const RowNorm& rn, int M, int wave, int n_waves, int lane, RowStat& st) {
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const int m = wave + r * n_waves;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int t = lane + SYN_WAVE * i;
+      st.v[r][i] = (rn.ss && m < M && t < rn.ss_groups) ? rn.ss[(size_t)m * rn.ss_groups + t] : 0.f;
+    }
+  }
+}
+__device__ __forceinline__ void row_stat_finish(const RowNorm& rn, int M, int wave, int n_waves, int lane, const RowStat& st,
+                                                float* inv) {
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const int m = wave + r * n_waves;
+    if (m >= M) break;   // the same for the whole wave
+    float s = (st.v[r][0] + st.v[r][1]) + (st.v[r][2] + st.v[r][3]);
+    for (int t = lane + 4 * SYN_WAVE; t < rn.ss_groups; t += SYN_WAVE) s += rn.ss[(size_t)m * rn.ss_groups + t];
+    s = wave_sum(s);
+    if (lane == 0) inv[m] = rsqrtf(s * rn.inv_dim + rn.eps);
+  }
+}
+
+// the epilogue of the product before the norm for output (m, n) with its finished sum v; all 16 lanes of a
+// group of columns call it together (rows beyond M with in == false); r0 and g: resid[m, n] and the gain of
+// column n, asked for before the product's loop
+__device__ __forceinline__ void resid_norm_store(const RowNorm& rn, bool in, int m, int n, int N, float v, float r0, float g) {
+  float r = 0.f;
+  if (in) {
+    const size_t at = (size_t)m * N + n;
+    r = r0 + v;
+    rn.resid[at] = r;
+    rn.xs[at] = (bf16)(g * r);
+  }
+  float q = r * r;
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) q += __shfl_xor(q, off, SYN_WAVE);
+  if (in && (n & 15) == 0) rn.ss_out[(size_t)m * (N / 16) + n / 16] = q;
+}
+
 // ------------------------------------------------------------------ few rows of x, W in fragment order
 // The same scheme as gemm_skinny (up to 16 rows of x, K split over the waves of a group, partial
 // tiles summed in LDS in a fixed order) over a copy of W that is kept in the order of the MFMA
@@ -182,10 +252,11 @@ static void launch_skinny(const bf16* x, const bf16* w, void* out, Epilogue ep, 
 template <int TILES, int KWAVES, int U, bool PAIRED>
 __global__ void __launch_bounds__(TILES * KWAVES * SYN_WAVE)
 gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void* __restrict__ out, Epilogue ep,
-                   int M, int N, int K, int ks_slice) {
+                   int M, int N, int K, int ks_slice, RowNorm rn) {
   static_assert(!PAIRED || TILES == 2, "a pair is two tiles");
   constexpr int WAVES = TILES * KWAVES;
   __shared__ float part[WAVES][4][64];
+  __shared__ float inv[16];
   const int wave = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
   const int tile = wave / KWAVES, kw = wave % KWAVES;
   const int r16 = lane % 16, kq = (lane / 16) * 8;
@@ -197,6 +268,16 @@ gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void
   const bool xok = r16 < M;
   const bf16* xrow = x + (size_t)min(r16, M - 1) * K + kq;
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  // what the epilogue needs of a norm's halves is asked for now, not behind the loop
+  RowStat stat;
+  if (rn.ss) row_stat_load(rn, M, wave, WAVES, lane, stat);
+  float r0 = 0.f, g0 = 0.f;
+  static_assert(TILES * 256 <= WAVES * SYN_WAVE, "every thread stores at most one output");
+  if (!PAIRED && rn.resid && threadIdx.x < TILES * 256) {
+    const int t = threadIdx.x / 256, j = (threadIdx.x / 64) % 4, ln = threadIdx.x % 64;
+    const int m = 4 * (ln / 16) + j, n = ((int)blockIdx.x * TILES + t) * 16 + ln % 16;
+    if (m < M && n < N) r0 = rn.resid[(size_t)m * N + n], g0 = load_gain(rn.gain, rn.gain_is_f32, n, rn.gain_offset);
+  }
   // blockIdx.y = which slice of K (ks_slice k-steps of 32) this workgroup sums; its output is slice blockIdx.y
   // of a float [slices, M, N] that the reader adds up (a product with few rows of W gets more workgroups so)
   const int ks_begin = (int)blockIdx.y * ks_slice, ks_end = min(nks, ks_begin + ks_slice);
@@ -215,6 +296,7 @@ gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void
   }
 #pragma unroll
   for (int j = 0; j < 4; ++j) part[wave][j][lane] = acc[j];
+  if (rn.ss) row_stat_finish(rn, M, wave, WAVES, lane, stat, inv);
   __syncthreads();
   auto summed = [&](int t, int j, int ln) {
     float s = 0.f;
@@ -227,7 +309,8 @@ gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void
       const int j = idx / 64, ln = idx % 64;
       const int m = 4 * (ln / 16) + j, col = (int)blockIdx.x * 16 + ln % 16;  // N / 2 outputs, 16 a workgroup
       if (m < M && 2 * col < N) {
-        const float g = summed(0, j, ln), up = summed(1, j, ln);
+        const float f = rn.ss ? inv[m] : 1.f;
+        const float g = summed(0, j, ln) * f, up = summed(1, j, ln) * f;
         ((bf16*)out)[(size_t)m * (N / 2) + col] = (bf16)gated(ep.act, g, up);
       }
     }
@@ -235,8 +318,12 @@ gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void
     for (int idx = threadIdx.x; idx < TILES * 4 * 64; idx += WAVES * SYN_WAVE) {
       const int t = idx / 256, j = (idx / 64) % 4, ln = idx % 64;
       const int m = 4 * (ln / 16) + j, n = ((int)blockIdx.x * TILES + t) * 16 + ln % 16;
-      if (m < M && n < N) {
-        const float v = summed(t, j, ln);
+      const bool in = m < M && n < N;
+      float v = summed(t, j, ln);
+      if (rn.ss && in) v *= inv[m];
+      if (rn.resid) {   // the same for the whole workgroup
+        resid_norm_store(rn, in, m, n, N, v, r0, g0);
+      } else if (in) {
         if (ep.out_is_f32)
           ((float*)out)[((size_t)blockIdx.y * M + m) * N + n] = v;
         else
@@ -248,11 +335,11 @@ gemm_packed_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void
 
 template <int TILES, int KWAVES, int U, bool PAIRED = false>
 static void launch_packed(const bf16* x, const bf16* wp, void* out, Epilogue ep, int M, int N, int K,
-                          hipStream_t stream, int slices = 1) {
+                          hipStream_t stream, int slices, const RowNorm& rn) {
   const int rows = TILES * 16;
   const int ks_slice = (K / 32 + slices - 1) / slices;
   gemm_packed_kernel<TILES, KWAVES, U, PAIRED>
-      <<<dim3((N + rows - 1) / rows, slices), TILES * KWAVES * SYN_WAVE, 0, stream>>>(x, wp, out, ep, M, N, K, ks_slice);
+      <<<dim3((N + rows - 1) / rows, slices), TILES * KWAVES * SYN_WAVE, 0, stream>>>(x, wp, out, ep, M, N, K, ks_slice, rn);
 }
 
 
@@ -261,8 +348,9 @@ static void launch_packed(const bf16* x, const bf16* wp, void* out, Epilogue ep,
 template <int KWAVES, int U, bool PAIRED>
 __global__ void __launch_bounds__(KWAVES * SYN_WAVE)
 gemm_packed2_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, void* __restrict__ out, Epilogue ep,
-                    int M, int N, int K, int ks_slice) {
+                    int M, int N, int K, int ks_slice, RowNorm rn) {
   __shared__ float part[KWAVES][2][4][64];
+  __shared__ float inv[16];
   const int kw = threadIdx.x / SYN_WAVE, lane = threadIdx.x % SYN_WAVE;
   const int r16 = lane % 16, kq = (lane / 16) * 8;
   const int nt = (int)blockIdx.x * 2, n_tiles = N / 16;
@@ -274,6 +362,8 @@ gemm_packed2_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, voi
   const bool xok = r16 < M;
   const bf16* xrow = x + (size_t)min(r16, M - 1) * K + kq;
   f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+  RowStat stat;
+  if (rn.ss) row_stat_load(rn, M, kw, KWAVES, lane, stat);
   const int ks_begin = (int)blockIdx.y * ks_slice, ks_end = min(nks, ks_begin + ks_slice);
   for (int ks0 = ks_begin + kw * U; ks0 < ks_end; ks0 += KWAVES * U) {
     bf16x8 b0[U], b1[U], ax[U];
@@ -292,6 +382,7 @@ gemm_packed2_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, voi
   }
 #pragma unroll
   for (int j = 0; j < 4; ++j) part[kw][0][j][lane] = acc0[j], part[kw][1][j][lane] = acc1[j];
+  if (rn.ss) row_stat_finish(rn, M, kw, KWAVES, lane, stat, inv);
   __syncthreads();
   auto summed = [&](int t, int j, int ln) {
     float s = 0.f;
@@ -303,14 +394,18 @@ gemm_packed2_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, voi
     for (int idx = threadIdx.x; idx < 4 * 64; idx += KWAVES * SYN_WAVE) {
       const int j = idx / 64, ln = idx % 64;
       const int m = 4 * (ln / 16) + j, col = (int)blockIdx.x * 16 + ln % 16;  // N / 2 outputs, 16 a workgroup
-      if (m < M && 2 * col < N) ((bf16*)out)[(size_t)m * (N / 2) + col] = (bf16)gated(ep.act, summed(0, j, ln), summed(1, j, ln));
+      if (m < M && 2 * col < N) {
+        const float f = rn.ss ? inv[m] : 1.f;
+        ((bf16*)out)[(size_t)m * (N / 2) + col] = (bf16)gated(ep.act, summed(0, j, ln) * f, summed(1, j, ln) * f);
+      }
     }
   } else {
     for (int idx = threadIdx.x; idx < 2 * 4 * 64; idx += KWAVES * SYN_WAVE) {
       const int t = idx / 256, j = (idx / 64) % 4, ln = idx % 64;
       const int m = 4 * (ln / 16) + j, n = (nt + t) * 16 + ln % 16;
       if (m < M && n < N && (t == 0 || second)) {
-        const float v = summed(t, j, ln);
+        float v = summed(t, j, ln);
+        if (rn.ss) v *= inv[m];
         if (ep.out_is_f32) ((float*)out)[((size_t)blockIdx.y * M + m) * N + n] = v;
         else ((bf16*)out)[(size_t)m * N + n] = (bf16)v;
       }
@@ -320,10 +415,10 @@ gemm_packed2_kernel(const bf16* __restrict__ x, const bf16* __restrict__ wp, voi
 
 template <int KWAVES, int U, bool PAIRED = false>
 static void launch_packed2(const bf16* x, const bf16* wp, void* out, Epilogue ep, int M, int N, int K,
-                           hipStream_t stream, int slices = 1) {
+                           hipStream_t stream, int slices, const RowNorm& rn) {
   const int ks_slice = (K / 32 + slices - 1) / slices;
   gemm_packed2_kernel<KWAVES, U, PAIRED>
-      <<<dim3((N + 31) / 32, slices), KWAVES * SYN_WAVE, 0, stream>>>(x, wp, out, ep, M, N, K, ks_slice);
+      <<<dim3((N + 31) / 32, slices), KWAVES * SYN_WAVE, 0, stream>>>(x, wp, out, ep, M, N, K, ks_slice, rn);
 }
 
 // ------------------------------------------------------------------ shared by the tiled kernels
@@ -1021,8 +1116,14 @@ SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, i
 // gemm_packed_kernel; N a multiple of 16, K of 32).  out_code: 1 = bf16 [M, N], 2 = float [M, N];
 // paired: W holds gate and up rows in turns of 16 and out is bf16 [M, N / 2] = act(gate) * up.
 // slices > 1 (float out, not paired): out is [slices, M, N], slice s holds the sum over its part of K.
-SYN_EXPORT int syn_gemm_packed(const void* x, const void* wp, void* out, int out_code, int M, int N, int K, int paired,
-                               int act, int slices, hipStream_t stream) {
+// The norm between two such products (RowNorm above):
+//   ss [M, ss_groups] float (or null): the sums of row m are multiplied by rsqrt(sum(ss[m, :]) / norm_dim + eps);
+//   resid [M, N] float (or null; then float sums, one slice, not paired, `out` unused): resid += sums,
+//   xs [M, N] bf16 = (gain_offset + gain[n]) * resid, ss_out [M, N / 16] = sums of resid^2 over groups of 16 columns.
+SYN_EXPORT int syn_gemm_packed_norm(const void* x, const void* wp, void* out, int out_code, int M, int N, int K, int paired,
+                                    int act, int slices, const float* ss, int ss_groups, int norm_dim, float eps,
+                                    float* resid, void* xs, float* ss_out, const void* gain, int gain_is_f32,
+                                    float gain_offset, hipStream_t stream) {
   SYN_CHECK(act >= 0 && act < SYN_ACT_COUNT, "gemm_packed: unknown activation code %d", act);
   SYN_CHECK(slices >= 1 && slices <= 64 && (slices == 1 || (out_code == 2 && !paired)),
             "gemm_packed: %d slices of K need a float output [slices, M, N] and no activation", slices);
@@ -1033,6 +1134,17 @@ SYN_EXPORT int syn_gemm_packed(const void* x, const void* wp, void* out, int out
   SYN_CHECK(out_code == 1 || out_code == 2, "gemm_packed: unknown output code %d", out_code);
   SYN_CHECK(!paired || out_code == 1, "gemm_packed: the gated product is stored as bf16");
   SYN_CHECK((uintptr_t)x % 16 == 0 && (uintptr_t)wp % 16 == 0, "gemm_packed: operands must be 16-byte aligned");
+  RowNorm rn = {};
+  if (ss) {
+    SYN_CHECK(ss_groups > 0 && norm_dim > 0, "gemm_packed: %d groups of a row statistic over %d columns", ss_groups, norm_dim);
+    rn.ss = ss, rn.ss_groups = ss_groups, rn.inv_dim = 1.f / (float)norm_dim, rn.eps = eps;
+  }
+  if (resid) {
+    SYN_CHECK(!paired && slices == 1 && out_code == 2 && xs && ss_out && gain,
+              "gemm_packed: the product before a norm is one slice of float sums with xs, ss_out and a gain");
+    rn.resid = resid, rn.xs = (bf16*)xs, rn.ss_out = ss_out, rn.gain = gain, rn.gain_is_f32 = gain_is_f32;
+    rn.gain_offset = gain_offset;
+  }
   const bf16* xb = (const bf16*)x;
   const bf16* wb = (const bf16*)wp;
   // from sweeps at N = 4096 .. 151936, K = 4096 and 12288, 1 and 8 rows
@@ -1040,10 +1152,16 @@ SYN_EXPORT int syn_gemm_packed(const void* x, const void* wp, void* out, int out
   // once for two products: a decode step of 8 sequences 3.88 -> 3.80 ms; at one row 3.30 -> 3.31 ms, at four
   // within the differences between boxes).  The same for the narrow products (two groups of rows a wave, twice
   // the slices of K) gained under 1 % at 8 sequences and lost as much at 4.
-  if (paired && M >= 5) launch_packed2<16, 2, true>(xb, wb, out, ep, M, N, K, stream);
-  else if (paired) launch_packed<2, 8, 4, true>(xb, wb, out, ep, M, N, K, stream);
-  else if (N <= 8192) launch_packed<1, 16, 2>(xb, wb, out, ep, M, N, K, stream, slices);
-  else launch_packed<1, 8, 8>(xb, wb, out, ep, M, N, K, stream, slices);
+  if (paired && M >= 5) launch_packed2<16, 2, true>(xb, wb, out, ep, M, N, K, stream, 1, rn);
+  else if (paired) launch_packed<2, 8, 4, true>(xb, wb, out, ep, M, N, K, stream, 1, rn);
+  else if (N <= 8192) launch_packed<1, 16, 2>(xb, wb, out, ep, M, N, K, stream, slices, rn);
+  else launch_packed<1, 8, 8>(xb, wb, out, ep, M, N, K, stream, slices, rn);
   SYN_LAUNCH_CHECK("gemm_packed");
   return 0;
+}
+
+SYN_EXPORT int syn_gemm_packed(const void* x, const void* wp, void* out, int out_code, int M, int N, int K, int paired,
+                               int act, int slices, hipStream_t stream) {
+  return syn_gemm_packed_norm(x, wp, out, out_code, M, N, K, paired, act, slices, nullptr, 0, 0, 0.f, nullptr, nullptr,
+                              nullptr, nullptr, 0, 0.f, stream);
 }

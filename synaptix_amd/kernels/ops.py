@@ -278,10 +278,16 @@ def unpack_weight(wp):
     return wp.view(nt, nks, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(nt * 16, nks * 32).contiguous()
 
 
-def gemm_packed(x, wp, out, paired=False, activation="silu"):
+def gemm_packed(x, wp, out, paired=False, activation="silu", row_scale=None, resid_norm=None):
     """out[M, N] (bf16 or float) = x[M, K] . W^T for M <= 16 with wp = pack_weight(W); paired: W holds gate and
     up rows in turns of 16 (pair_rows) and out [M, N / 2] bf16 = act(gate) * up.  A float out of shape
-    [S, M, N] receives S partial sums over slices of K instead."""
+    [S, M, N] receives S partial sums over slices of K instead.
+
+    The two halves of an RMSNorm that lies between two such products (csrc/gemm.hip: RowNorm):
+    resid_norm = (resid [M, N] float, gain [N], gain_offset, xs [M, N] bf16, ss [M, N / 16] float) with out None:
+    the sums are added into resid, xs = (gain_offset + gain) * resid, ss = sums of resid^2 over groups of 16 columns;
+    row_scale = (ss [M, G] float, dim, eps): the sums of row m are multiplied by rsqrt(sum(ss[m]) / dim + eps), which
+    makes this the product over the normed rows when x is the xs that came with ss."""
     _need(x, "gemm_packed.x", _BF16, (None, None))
     M, K = x.shape
     if K % 32:
@@ -291,15 +297,42 @@ def gemm_packed(x, wp, out, paired=False, activation="silu"):
     if M > 16 or (paired and N % 32):
         raise KernelError(f"gemm_packed: M = {M} (at most 16), N = {N}")
     slices = 1
-    if paired:
+    ss = resid = xs = ss_out = gain = None
+    groups = dim = 0
+    eps = gain_offset = 0.0
+    if row_scale is not None:
+        ss, dim, eps = row_scale
+        _need(ss, "gemm_packed.row_scale", _F32, (M, None))
+        groups = ss.shape[1]
+        if groups < 1 or dim < 1:
+            raise KernelError(f"gemm_packed: a row statistic of {groups} groups over {dim} columns")
+    if resid_norm is not None:
+        resid, gain, gain_offset, xs, ss_out = resid_norm
+        if paired or out is not None:
+            raise KernelError("gemm_packed: the product before a norm is not gated and has no output beside resid, xs and ss")
+        _need(resid, "gemm_packed.resid", _F32, (M, N))
+        _need(gain, "gemm_packed.gain", (_BF16, _F32), (N,))
+        _need(xs, "gemm_packed.xs", _BF16, (M, N))
+        _need(ss_out, "gemm_packed.ss", _F32, (M, N // 16))
+        out_code = 2
+    elif paired:
         _need(out, "gemm_packed.out", _BF16, (M, N // 2))
+        out_code = 1
     elif out.dim() == 3:          # float partial sums over slices of K, which the reader adds
         slices = out.shape[0]
         _need(out, "gemm_packed.out", _F32, (slices, M, N))
+        out_code = 2
     else:
         _need(out, "gemm_packed.out", (_BF16, _F32), (M, N))
-    _call(load_library("core"), "syn_gemm_packed", _ptr(x), _ptr(wp), _ptr(out), 2 if out.dtype == _F32 else 1,
-          M, N, K, 1 if paired else 0, activation_code(activation), slices, _stream())
+        out_code = 2 if out.dtype == _F32 else 1
+    if row_scale is None and resid_norm is None:
+        _call(load_library("core"), "syn_gemm_packed", _ptr(x), _ptr(wp), _ptr(out), out_code,
+              M, N, K, 1 if paired else 0, activation_code(activation), slices, _stream())
+        return
+    _call(load_library("core"), "syn_gemm_packed_norm", _ptr(x), _ptr(wp), _ptr(out), out_code, M, N, K,
+          1 if paired else 0, activation_code(activation), slices, _ptr(ss), int(groups), int(dim), ctypes.c_float(eps),
+          _ptr(resid), _ptr(xs), _ptr(ss_out), _ptr(gain), _is_f32(gain) if gain is not None else 0,
+          ctypes.c_float(gain_offset), _stream())
 
 
 _compute_units = None

@@ -19,7 +19,7 @@ import torch
 
 from ..kernels import ops
 from ..parts.base import Part
-from ..parts.linear import linear, packed_copy
+from ..parts.linear import linear, packed_copy, as_delta, as_rows
 from ..weights.source import TensorSpec
 
 
@@ -137,8 +137,13 @@ class DecoderModel:
             resid = self.embedding.forward(tokens)
             pending = None
             for run, owner in zip(self.schedule, self._owner):
-                pending = self.blocks[run.block].forward(resid, pending, ctx, cache.layer_view(run.cache), owner)
+                block = self.blocks[run.block]
+                if not block.takes_deferred_product:
+                    pending = as_delta(pending)      # a product that the last block left for a norm to take in
+                pending = block.forward(resid, pending, ctx, cache.layer_view(run.cache), owner)
             if want_rows is None:
                 return None          # nothing is asked for: the cache has been written, that is all
+            if not getattr(self.final_norm, "takes_deferred_product", False):
+                pending = as_delta(pending)
             h = self.final_norm.add_apply(resid, pending, ctx.act_dtype, rows=want_rows)
-            return self.head.forward(h)
+            return self.head.forward(as_rows(h))

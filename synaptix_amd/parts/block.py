@@ -8,6 +8,7 @@ unsummed and takes the previous block's.
 from __future__ import annotations
 
 from .base import Part
+from .linear import as_rows, as_delta
 
 
 class Block(Part):
@@ -15,12 +16,21 @@ class Block(Part):
     resid [N, hidden] float is updated in place; pending is a delta not yet added (or None)."""
 
     mixer = None
+    # True: `pending` may arrive as a parts.linear.DeferredProduct (a product that the block's first norm can take
+    # in); False (the default): the model runs such a product before it calls the block
+    takes_deferred_product = False
 
     def forward(self, resid, pending, ctx, cache, owner=True):
         raise NotImplementedError
 
 
+def _norm_input(norm, delta):
+    return delta if getattr(norm, "takes_deferred_product", False) else as_delta(delta)
+
+
 class PreNormBlock(Block):
+    takes_deferred_product = True
+
     def __init__(self, norm1, mixer, norm2, feed_forward):
         self.norm1, self.mixer, self.norm2, self.feed_forward = norm1, mixer, norm2, feed_forward
 
@@ -42,7 +52,9 @@ class PreNormBlock(Block):
             p.check(dtype)
 
     def forward(self, resid, pending, ctx, cache, owner=True):
-        h = self.norm1.add_apply(resid, pending, ctx.act_dtype)
-        a = self.mixer.forward(h, ctx, cache, owner)
-        h2 = self.norm2.add_apply(resid, a, ctx.act_dtype)
-        return self.feed_forward.forward(h2, ctx)
+        # a norm may hand on rows whose last step a product finishes, and take a product that has not been run
+        # (parts.linear.ScaledRows, DeferredProduct); parts that do not say they take them get plain tensors
+        h = self.norm1.add_apply(resid, _norm_input(self.norm1, pending), ctx.act_dtype)
+        a = self.mixer.forward(h if self.mixer.takes_scaled_rows else as_rows(h), ctx, cache, owner)
+        h2 = self.norm2.add_apply(resid, _norm_input(self.norm2, a), ctx.act_dtype)
+        return self.feed_forward.forward(h2 if self.feed_forward.takes_scaled_rows else as_rows(h2), ctx)

@@ -10,17 +10,21 @@ import torch
 from ..kernels import ops
 from ..weights.source import TensorSpec
 from .base import Part
-from .linear import linear, linear_for_sum, packed_copy
+from .linear import linear, linear_for_sum, deferred_product, as_rows, ScaledRows, packed_copy
 
 
 class FeedForward(Part):
     """Interface: forward(h [N, hidden] activation type, ctx) -> residual delta [N, hidden] float."""
+
+    takes_scaled_rows = False     # as Mixer.takes_scaled_rows
 
     def forward(self, h, ctx):
         raise NotImplementedError
 
 
 class GatedMlp(FeedForward):
+    takes_scaled_rows = True
+
     def __init__(self, prefix: str, hidden: int, intermediate: int, activation: str = "silu"):
         try:
             ops.activation_code(activation)       # the kernels apply it by its code; an unknown name is refused here
@@ -53,9 +57,13 @@ class GatedMlp(FeedForward):
         m = torch.empty((h.shape[0], self.intermediate), dtype=h.dtype, device=h.device)
         if self.paired and h.dtype == torch.bfloat16:
             if self.p_gate_up is not None and h.shape[0] <= ops.PACKED_MAX_ROWS_GATED:
-                ops.gemm_packed(h, self.p_gate_up, m, paired=True, activation=self.activation)
+                if isinstance(h, ScaledRows):      # the norm's last step is the product's epilogue
+                    ops.gemm_packed(h.rows, self.p_gate_up, m, paired=True, activation=self.activation, row_scale=h.row_scale)
+                else:
+                    ops.gemm_packed(h, self.p_gate_up, m, paired=True, activation=self.activation)
             else:
-                ops.gemm_swiglu(h, self.w_gate_up, m, self.activation)
+                ops.gemm_swiglu(as_rows(h), self.w_gate_up, m, self.activation)
         else:
+            h = as_rows(h)
             ops.swiglu(linear(h, self.w_gate_up, h.dtype), m, self.activation)
-        return linear_for_sum(m, self.w_down, self.p_down)
+        return deferred_product(m, self.w_down, self.p_down)

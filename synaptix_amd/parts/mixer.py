@@ -15,7 +15,7 @@ import torch
 from ..kernels import ops
 from ..weights.source import TensorSpec
 from .base import Part, KvNeed
-from .linear import linear, linear_for_sum, packed_copy
+from .linear import linear, linear_for_sum, deferred_product, as_rows, ScaledRows, packed_copy
 from .position import Position, NoPosition
 
 
@@ -29,6 +29,10 @@ class Mixer(Part):
     or as partial sums [S, N, hidden] that the following norm adds up.
     """
 
+    # True: `h` may arrive as parts.linear.ScaledRows (rows whose norm a product over packed weights finishes)
+    # and the returned delta may be a parts.linear.DeferredProduct; False (the default): plain tensors both ways
+    takes_scaled_rows = False
+
     def cache_need(self):
         return None
 
@@ -37,6 +41,8 @@ class Mixer(Part):
 
 
 class GqaAttention(Mixer):
+    takes_scaled_rows = True
+
     def __init__(self, prefix: str, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, *,
                  position: Position | None = None, qk_norm_eps: float | None = None, scale: float | None = None,
                  window: int | None = None, qk_gain_offset: float = 0.0):
@@ -96,6 +102,7 @@ class GqaAttention(Mixer):
             if qkv.dim() == 2:
                 qkv = qkv.unsqueeze(0)
         else:
+            h = as_rows(h)
             # (every kernel behind it adds partial sums itself; ops.gemm_slices cuts where the product would
             # otherwise leave compute units without work: single tokens and prompts up to about 1,200 tokens)
             sliced = ops.gemm_slices(N, self.w_qkv.shape[0], self.hidden, act) > 1
@@ -112,7 +119,7 @@ class GqaAttention(Mixer):
                                             self.scale, window, nh, nkv, hd, self.q_gain, self.k_gain,
                                             self.qk_norm_eps or 0.0, cos, sin, write_kv=owner,
                                             gain_offset=self.qk_gain_offset)
-            return linear_for_sum(o, self.w_o, self.p_o)
+            return deferred_product(o, self.w_o, self.p_o)
         q = torch.empty((N, nh * hd), dtype=act, device=h.device)
         ops.qk_norm_rope_kv_write(qkv, q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos,
                                   self.q_gain, self.k_gain, self.qk_norm_eps or 0.0, cos, sin, nh, nkv, hd,
@@ -128,4 +135,4 @@ class GqaAttention(Mixer):
         else:
             ops.attention_prefill_bf16(q, cache.k_pages, cache.v_pages, table, ctx.seq_start, ctx.seq_past, o,
                                        self.scale, window, nh, nkv, hd)
-        return linear_for_sum(o, self.w_o, self.p_o)
+        return deferred_product(o, self.w_o, self.p_o)

@@ -72,18 +72,39 @@ def gemm_swiglu(x, w_paired, out, activation="silu"):
     out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
 
 
-def gemm_packed(x, wp, out, paired=False, activation="silu"):
+def gemm_packed(x, wp, out, paired=False, activation="silu", row_scale=None, resid_norm=None):
     from synaptix_amd.kernels import ops
     w = ops.unpack_weight(wp)
+    factor = None
+    if row_scale is not None:      # the second half of a norm carried between two products
+        ss, dim, eps = row_scale
+        factor = torch.rsqrt(ss.sum(1) / torch.tensor(float(dim), dtype=F32) + torch.tensor(eps, dtype=F32))[:, None]
+    if resid_norm is not None:     # the first half: sums into the residual rows, the gain, the statistic in groups of 16
+        resid, gain, gain_offset, xs, ss_out = resid_norm
+        sums = x.to(F32) @ w.to(F32).T
+        if factor is not None:
+            sums = sums * factor
+        resid += sums
+        xs.copy_(((gain_offset + gain.to(F32)) * resid).to(xs.dtype))
+        ss_out.copy_((resid * resid).view(resid.shape[0], -1, 16).sum(2))
+        return
     if paired:
-        gemm_swiglu(x, w, out)
+        N, K = w.shape
+        wv = w.view(N // (2 * PAIR), 2, PAIR, K)
+        g = x.to(F32) @ wv[:, 0].reshape(N // 2, K).to(F32).T
+        u = x.to(F32) @ wv[:, 1].reshape(N // 2, K).to(F32).T
+        if factor is not None:
+            g, u = g * factor, u * factor
+        out.copy_((g / (1 + torch.exp(-g)) * u).to(out.dtype))
     elif out.dim() == 3:                    # partial sums over slices of K (whole k-steps of 32)
         S, K = out.shape[0], w.shape[1]
         step = -(-(K // 32) // S) * 32
         for i in range(S):
-            out[i] = x[:, i * step:(i + 1) * step].to(F32) @ w[:, i * step:(i + 1) * step].to(F32).T
+            part = x[:, i * step:(i + 1) * step].to(F32) @ w[:, i * step:(i + 1) * step].to(F32).T
+            out[i] = part if factor is None else part * factor
     else:
-        out.copy_((x.to(F32) @ w.to(F32).T).to(out.dtype))
+        y = x.to(F32) @ w.to(F32).T
+        out.copy_((y if factor is None else y * factor).to(out.dtype))
 
 
 def stream_scope():

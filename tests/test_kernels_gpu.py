@@ -330,6 +330,65 @@ def test_gated_product_over_weights_in_fragment_order(ops, M, I, K):
     close(out, want, 2e-3 * K + 0.02, 1e-2, f"packed gated product {M}x{I}x{K}")
 
 
+@pytest.mark.parametrize("gain_dtype,gain_offset", [(BF16, 0.0), (F32, 1.0)])
+@pytest.mark.parametrize("M,H,K,N2", [(1, 64, 96, 48), (8, 4096, 4096, 6144), (5, 208, 1120, 80), (8, 4096, 12288, 24576),
+                                      (3, 10240, 64, 32), (16, 48, 32, 16400)])
+def test_norm_carried_between_two_products_over_packed_weights(ops, gain_dtype, gain_offset, M, H, K, N2):
+    """The two halves of an RMSNorm between two products for few rows.  First half, as the epilogue of the product
+    before it: resid += x . W^T, xs = gain * resid, ss = sums of resid^2 over groups of 16 columns.  Second half, as
+    the epilogue of the product after it: sums of row m times rsqrt(sum(ss[m]) / H + eps), plain, gated, and in
+    slices of K.  Together they equal the product over the normed rows."""
+    eps = 1e-5
+    x, w = rnd((M, K), 41, BF16), rnd((H, K), 42, BF16, 0.05)
+    resid0 = rnd((M, H), 43)
+    resid0[0] *= 30.0                    # rows of unequal size: a factor applied to the wrong row would show
+    gain = (1 + 0.2 * rnd((H,), 44) - gain_offset).to(gain_dtype)
+    wp = ops.pack_weight(w.to(DEV))
+    resid = resid0.to(DEV)
+    xs = torch.full((M, H), float("nan"), dtype=BF16, device=DEV)
+    ss = torch.full((M, H // 16), float("nan"), dtype=F32, device=DEV)
+    ops.gemm_packed(x.to(DEV), wp, None, resid_norm=(resid, gain.to(DEV), gain_offset, xs, ss))
+    r = resid0.double() + x.double() @ w.double().T
+    close(resid, r.float(), 1e-3 * math.sqrt(K) * 0.05 + 1e-5, 1e-6, "residual rows")
+    r32 = resid.cpu()                    # what the kernel kept: the rest is computed from it
+    g_all = gain_offset + gain.double()
+    close(xs, (g_all * r32.double()).float(), 1e-6, 2 ** -8, "rows with the gain")
+    close(ss, (r32.double() ** 2).view(M, H // 16, 16).sum(2).float(), 1e-6, 1e-5, "row statistic in groups")
+    inv = torch.rsqrt((r32.double() ** 2).sum(1) / H + eps)[:, None]
+    xs64 = xs.cpu().double()
+    scale = (ss, H, eps)
+    # plain product after the norm, bf16 and float, and in slices
+    w2 = rnd((N2, H), 45, BF16, 0.05)
+    wp2 = ops.pack_weight(w2.to(DEV))
+    want = ((xs64 @ w2.double().T) * inv).float()
+    atol = 2e-3 * float(want.abs().max()) + 1e-6
+    out = torch.full((M, N2), float("nan"), dtype=F32, device=DEV)
+    ops.gemm_packed(xs, wp2, out, row_scale=scale)
+    close(out, want, atol, 1e-5, "product after the norm")
+    parts = torch.full((3, M, N2), float("nan"), dtype=F32, device=DEV)
+    ops.gemm_packed(xs, wp2, parts, row_scale=scale)
+    close(parts.sum(0), want, atol, 1e-5, "product after the norm in slices")
+    outb = torch.full((M, N2), float("nan"), dtype=BF16, device=DEV)
+    ops.gemm_packed(xs, wp2, outb, row_scale=scale)
+    close(outb, want, atol, 2 ** -7, "product after the norm, bf16")
+    # it equals the product over the normed rows up to the rounding of those rows
+    normed = (g_all * r32.double() * inv).to(BF16)
+    direct = (normed.double() @ w2.double().T).float()
+    assert float((want - direct).abs().max()) <= 0.02 * float(direct.abs().max()) + 1e-6
+    # gated product after the norm
+    if N2 % 32 == 0:
+        I = N2 // 2
+        wg, wu = w2[:I], w2[I:]
+        wpg = ops.pack_weight(ops.pair_rows(wg.to(DEV), wu.to(DEV)))
+        outg = torch.full((M, I), float("nan"), dtype=BF16, device=DEV)
+        ops.gemm_packed(xs, wpg, outg, paired=True, row_scale=scale)
+        gg, uu = (xs64 @ wg.double().T) * inv, (xs64 @ wu.double().T) * inv
+        wantg = (gg / (1 + torch.exp(-gg)) * uu).float()
+        close(outg, wantg, 2e-3 * float(wantg.abs().max()) + 1e-6, 2 ** -7, "gated product after the norm")
+    with pytest.raises(Exception, match="not gated"):
+        ops.gemm_packed(x.to(DEV), wp, xs, resid_norm=(resid, gain.to(DEV), gain_offset, xs, ss))
+
+
 def _sampled(M, N, n, seed):
     g = torch.Generator().manual_seed(seed)
     rows = torch.cat([torch.tensor([0, M - 1, 0, M - 1]), torch.randint(0, M, (n,), generator=g)])
