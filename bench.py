@@ -15,6 +15,12 @@ tokens each, through the generation loop itself (engine.generate.generate: its p
 prefill step for all prompts, its captured decode steps and its sampling); a step is one of its
 decode steps.  The whole run is done once untimed (it captures the graphs) and once timed.
 
+The default run (8b, without --no-points) measures the other workloads as well and puts them under
+`points`: the same 8 sequences through the generation loop (decode_b8_through_generate: the loop's
+own clock over its last `steps` decode steps, to stand beside `value`), the 4b workload
+(decode_4b_unequal16, its fraction of the HBM roofline and its prompts' rate) and the 32b shape at
+8 sequences (decode_32b_b8), each with the sizes it ran at as a text.
+
 Method after the reference's own harnesses (crates/synaptix-models/llm/qwen3/examples/format_perf.rs:41-122,
 crates/synaptix-cli/src/commands/bench.rs:35-96): synthetic ids, warm-up first, device synchronised
 at both ends of the timed region only.
@@ -71,9 +77,10 @@ def prefill_flops(cfg, lengths) -> int:
     return total
 
 
-def unequal_prompts_through_generate(args, shape) -> int:
+def unequal_prompts_through_generate(args, shape, emit=True):
     """16 prompts of seeded lengths uniform in [64, 4096], 128 greedy tokens each, through the
-    generation loop; its own clocks (GenerationStats) give the numbers."""
+    generation loop; its own clocks (GenerationStats) give the numbers.  emit: print the line and return the
+    exit code; else return the line."""
     import torch
     from synaptix_amd import Qwen3Config, Engine
     from synaptix_amd.engine.generate import generate, GenerationConfig
@@ -125,8 +132,37 @@ def unequal_prompts_through_generate(args, shape) -> int:
                    "step_ms_max": round(steps_sorted[-1], 4),
                    "end_to_end_tok_s": round(n_prompts * new_tokens / ((st.prefill_ms + st.decode_ms) / 1e3), 1)},
     }
+    if not emit:
+        del eng
+        return line
     print(json.dumps(line))
     return 0
+
+
+def sizes_text(cfg, layers_run=None) -> str:
+    """The sizes a point was measured at, as one text (a record keeps no nested values)."""
+    L = cfg.num_hidden_layers if layers_run is None else layers_run
+    return (f"{L} of {cfg.num_hidden_layers} layers, hidden {cfg.hidden_size}, {cfg.num_attention_heads} heads / "
+            f"{cfg.num_key_value_heads} kv heads of {cfg.head_dim}, intermediate {cfg.intermediate_size}, vocab {cfg.vocab_size}, "
+            f"tie {cfg.tie_word_embeddings}")
+
+
+def through_generate(eng, cfg, batch, prompt_len, warmup, steps, weight_bytes, use_graph=True):
+    """`batch` prompts of prompt_len tokens through engine.generate.generate; the loop's own clock over its last
+    `steps` decode steps (the first `warmup` are left out: the first run also captures the graph)."""
+    import torch
+    from synaptix_amd.engine.generate import generate, GenerationConfig
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, cfg.vocab_size, (prompt_len,), generator=g).tolist() for _ in range(batch)]
+    gen = GenerationConfig(max_new_tokens=warmup + steps + 1, temperature=0.0, eos_token_ids=(-1,))
+    outs, st = generate(eng, prompts, gen, use_graph=use_graph, max_batch=batch)
+    torch.cuda.synchronize()
+    assert st.batches == 1 and st.decode_steps == warmup + steps
+    tail = st.step_ms[-steps:]
+    step_s = sum(tail) / 1e3 / steps
+    mean_ctx = prompt_len + 1 + warmup + (steps - 1) / 2
+    step_bytes = weight_bytes + batch * mean_ctx * eng.cache.bytes_per_token()
+    return batch / step_s, step_s, step_bytes
 
 
 def main() -> int:
@@ -254,6 +290,13 @@ def main() -> int:
             points[f"decode_b{b}"] = round(rate, 1)
             points[f"decode_b{b}_hbm_frac"] = round(step_bytes / step_s / 1e9 / HBM_PEAK_GBS, 4)
 
+    if not args.no_points:
+        # the same sequences through the generation loop: its planning, its bucket of rows, its sampling
+        rate, step_s, step_bytes = through_generate(eng, cfg, args.batch, prompt_len, args.warmup, args.steps, weight_bytes,
+                                                    use_graph=not args.no_graph)
+        points[f"decode_b{args.batch}_through_generate"] = round(rate, 1)
+        points[f"decode_b{args.batch}_through_generate_ms_per_step"] = round(step_s * 1e3, 4)
+
     achieved = main_bytes / main_step / 1e9
     # what this machine gives to kernels that only read, or only multiply: measured, beside the vendor's peaks
     read_gbs, mfma_tflops = ops.measure_ceilings(eng.device)
@@ -277,6 +320,34 @@ def main() -> int:
         "points": points,
         "measured": measured,
     }
+    if not args.no_points and args.shape == "8b" and args.layers == shape["num_hidden_layers"]:
+        # the other workloads, each on an engine of its own after this one has gone
+        import gc
+        del eng
+        gc.collect()
+        torch.cuda.empty_cache()
+        sub = argparse.Namespace(**vars(args))
+        sub.steps, sub.warmup, sub.layers = min(args.steps, 127), 1, SHAPES["4b"]["num_hidden_layers"]
+        four = unequal_prompts_through_generate(sub, SHAPES["4b"], emit=False)
+        points["decode_4b_unequal16"] = four["value"]
+        points["decode_4b_unequal16_hbm_frac"] = four["roofline"]["frac"]
+        points["prefill_4b_unequal16"] = four["prefill"]["value"]
+        points["prefill_4b_unequal16_frac"] = four["prefill"]["frac"]
+        points["config_4b_unequal16"] = (sizes_text(Qwen3Config.from_dict(SHAPES["4b"])) +
+                                         f", 16 prompts of {four['config']['min_prompt']} to {four['config']['max_prompt']} tokens "
+                                         f"({four['prefill']['tokens']} in all), {four['config']['new_tokens']} new tokens each, "
+                                         "through engine.generate.generate")
+        gc.collect()
+        torch.cuda.empty_cache()
+        big = Qwen3Config.from_dict(SHAPES["32b"])
+        k, w = min(args.steps, 32), min(args.warmup, 4)
+        per = (prompt_len + k + w + 8 + 63) // 64 * 64
+        eng = Engine.from_config(big, seed=0, dtype="bfloat16", max_tokens=8 * per + 64, max_seq=8192)
+        rate, step_s, step_bytes = through_generate(eng, big, 8, prompt_len, w, k, decode_weight_bytes(big))
+        points["decode_32b_b8"] = round(rate, 1)
+        points["decode_32b_b8_hbm_frac"] = round(step_bytes / step_s / 1e9 / HBM_PEAK_GBS, 4)
+        points["config_32b_b8"] = sizes_text(big) + f", 8 prompts of {prompt_len} tokens, {w} + {k} decode steps, through engine.generate.generate"
+        del eng
     print(json.dumps(line))
     return 0
 

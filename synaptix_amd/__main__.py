@@ -4,7 +4,8 @@ the same option names and meanings where this engine has the feature.
 
     python -m synaptix_amd run MODEL [PROMPT] [--prompt-file F | --prompt-ids 1,2,3 | --prompt-ids-file F]
            [--max-tokens 128] [--temperature 1.0] [--seed 0] [--device cuda] [--max-seq N]
-           [--compute-dtype bf16|f32] [--no-graph] [--warmup] [--op-times]
+           [--compute-dtype bf16|f32] [--no-graph] [--warmup] [--op-times] [--batch N]
+    python -m synaptix_amd run --random CONFIG_JSON ...      (no model folder: random weights drawn with --seed)
     python -m synaptix_amd bench MODEL [--n-tokens 128] [--prompt-tokens 32] [--batch-size 1] [--warmup 3] [--dtype bf16]
     python -m synaptix_amd random CONFIG_JSON OUT_DIR [--seed 0] [--dtype bf16|f32]
 
@@ -27,7 +28,19 @@ def cmd_run(a) -> int:
     from .pipeline import Pipeline
     from .sampling import GenerationConfig
 
-    pipe = Pipeline.load(a.model, device=a.device, dtype=a.compute_dtype, max_seq=a.max_seq)
+    if a.random is not None:
+        # no folder: the configuration alone, weights drawn on the device from --seed; the one positional
+        # argument left, if any, is the prompt
+        if a.prompt:
+            print("synaptix_amd run: with --random CONFIG there is no MODEL argument; give the prompt alone", file=sys.stderr)
+            return 1
+        a.prompt, a.model = a.model or "", None
+        pipe = Pipeline.random(a.random, seed=a.seed, device=a.device, dtype=a.compute_dtype, max_seq=a.max_seq)
+    elif not a.model:
+        print("synaptix_amd run: a MODEL folder or --random CONFIG_JSON is needed", file=sys.stderr)
+        return 1
+    else:
+        pipe = Pipeline.load(a.model, device=a.device, dtype=a.compute_dtype, max_seq=a.max_seq)
     as_text = False
     if a.prompt_ids is not None:
         prompt = _ids(a.prompt_ids)
@@ -48,15 +61,22 @@ def cmd_run(a) -> int:
         import dataclasses
         pipe.generate(prompt, dataclasses.replace(cfg, max_new_tokens=4, temperature=0.0), use_graph=not a.no_graph)
     t0 = time.perf_counter()
-    if a.op_times:      # the reference's per-op profile (model.rs:22-99): every op synchronised and timed, eager steps
+    if a.batch > 1:     # the prompt a.batch times in one batch; sequence i draws from the stream of seed + i
+        outs, st = pipe.generate_batch([prompt] * a.batch, cfg, use_graph=not a.no_graph)
+        ms = (time.perf_counter() - t0) * 1e3
+        for o in outs:
+            print(pipe.decode(o.tokens) if as_text else " ".join(str(t) for t in o.tokens))
+        ids = None
+    elif a.op_times:    # the reference's per-op profile (model.rs:22-99): every op synchronised and timed, eager steps
         from .kernels import ops
         with ops.op_timing() as times:
             ids, st = pipe.generate(prompt, cfg, use_graph=False)
         print(times.report(), file=sys.stderr)
     else:
         ids, st = pipe.generate(prompt, cfg, use_graph=not a.no_graph)
-    ms = (time.perf_counter() - t0) * 1e3
-    print(pipe.decode(ids) if as_text else " ".join(str(t) for t in ids))
+    if ids is not None:
+        ms = (time.perf_counter() - t0) * 1e3
+        print(pipe.decode(ids) if as_text else " ".join(str(t) for t in ids))
     # the reference's line: crates/synaptix-cli/src/commands/run.rs:234
     print(f"synaptix_amd run: {st.prompt_tokens} prompt + {st.new_tokens} new tokens in {ms:.0f} ms | "
           f"prefill {st.prefill_ms:.0f} ms | decode {st.decode_ms:.0f} ms "
@@ -71,7 +91,7 @@ def cmd_bench(a) -> int:
 
     pipe = Pipeline.load(a.model, device=a.device, dtype=a.dtype,
                          max_tokens=a.batch_size * ((a.prompt_tokens + a.n_tokens + 127) // 64 * 64))
-    V = pipe.config.vocab_size
+    V = pipe.engine.vocab
     prompts = [[((i * 7 + 13 + b) % min(200, V - 5)) + 5 for i in range(a.prompt_tokens)] for b in range(a.batch_size)]
     cfg = GenerationConfig(max_new_tokens=a.n_tokens, temperature=0.0, eos_token_ids=(-1,))     # never stops early
     for _ in range(a.warmup):
@@ -102,8 +122,11 @@ def main(argv=None) -> int:
                                  formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="cmd", required=True)
     r = sub.add_parser("run", help="generate from one prompt")
-    r.add_argument("model")
+    r.add_argument("model", nargs="?", default="")
     r.add_argument("prompt", nargs="?", default="")
+    r.add_argument("--random", metavar="CONFIG_JSON", default=None,
+                   help="no model folder: this config.json with random weights drawn from --seed")
+    r.add_argument("--batch", type=int, default=1, help="generate this many sequences from the prompt in one batch")
     r.add_argument("--prompt-file")
     r.add_argument("--prompt-ids", help="token ids, separated by commas or blanks (no tokenizer needed)")
     r.add_argument("--prompt-ids-file")

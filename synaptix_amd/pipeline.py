@@ -50,6 +50,27 @@ class Pipeline:
                           max_seq=max_seq, device=device)
         return cls(eng, path)
 
+    @classmethod
+    def random(cls, config_json: str, seed: int = 0, device: str = "cuda", dtype: str = "bf16", max_seq: int | None = None,
+               max_tokens: int | None = None, max_batch: int | None = None) -> "Pipeline":
+        """No model folder: the architecture and sizes of `config_json` (a config.json file) with random weights
+        drawn on the device from `seed` (for measurements and trials; nothing is written)."""
+        import json
+        from .config import resolve_architecture
+        if dtype not in _DTYPE_NAMES:
+            raise ValueError(f"dtype {dtype!r}: bf16 or f32 (f16 and quantized types are not built)")
+        if device == "cuda":
+            device = "cuda:0"
+        with open(config_json) as f:
+            d = json.load(f)
+        cfg = resolve_architecture(d).config_cls.from_dict(d)
+        longest = max_seq or cfg.max_position_embeddings
+        if max_tokens is None:
+            max_tokens = max(min(8 * longest, 65536), longest)
+        eng = Engine.from_config(cfg, seed=seed, dtype=_DTYPE_NAMES[dtype], max_tokens=max_tokens, max_slots=max_batch,
+                                 max_seq=max_seq, device=device)
+        return cls(eng, None)
+
     # ------------------------------------------------------------------ text, when the folder has a tokenizer
     def _tok(self):
         if self._tokenizer is None:

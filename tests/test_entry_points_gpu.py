@@ -1,5 +1,6 @@
 """Greedy generation through the entry points a user has: the Python pipeline and the command line."""
 import json
+import os
 import subprocess
 import sys
 
@@ -60,6 +61,17 @@ def test_command_line_run_and_bench():
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert [int(t) for t in proc.stdout.split()] == want
     assert "12 prompt + 7 new tokens" in proc.stderr and "tok/s" in proc.stderr
+    # no folder: a config.json alone with weights drawn from --seed, and the prompt several times in one batch
+    cmd = [sys.executable, "-m", "synaptix_amd", "run", "--random", os.path.join(folder, "config.json"), "--seed", "3",
+           "--prompt-ids", "5,6,7,8,9", "--max-tokens", "4", "--temperature", "0", "--batch", "3"]
+    runs = [subprocess.run(cmd, capture_output=True, text=True, cwd=ROOT, timeout=300) for _ in range(2)]
+    assert all(r.returncode == 0 for r in runs), runs[0].stderr[-2000:]
+    rows = [[int(t) for t in line.split()] for line in runs[0].stdout.strip().splitlines()]
+    assert len(rows) == 3 and rows[0] == rows[1] == rows[2] and len(rows[0]) == 4       # greedy: the same three times
+    assert all(0 <= t < CONFIGS[name]["vocab_size"] for t in rows[0]) and runs[0].stdout == runs[1].stdout
+    assert "15 prompt + 12 new tokens" in runs[0].stderr
+    proc = subprocess.run(cmd[:4] + cmd[6:], capture_output=True, text=True, cwd=ROOT, timeout=60)   # neither MODEL nor --random
+    assert proc.returncode == 1 and "MODEL" in proc.stderr
     cmd = [sys.executable, "-m", "synaptix_amd", "bench", folder, "--n-tokens", "16", "--prompt-tokens", "9",
            "--batch-size", "3", "--warmup", "1"]
     proc = subprocess.run(cmd, capture_output=True, text=True, cwd=ROOT, timeout=300)
@@ -129,6 +141,14 @@ def test_bench_line_keeps_its_contract():
     assert roof["bound"] == "hbm" and roof["unit"] == "GB/s" and roof["peak"] == 8000.0
     assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
     assert rec["value"] > 0 and abs(rec["value"] - 2 / (rec["ms_per_step"] * 1e-3)) < 0.01 * rec["value"]
+    # with points: batch 1 and 64 and the same batch through the generation loop (the other shapes' points come
+    # with the whole model only)
+    proc = subprocess.run(cmd + ["--layers", "1", "--steps", "3", "--warmup", "1", "--batch", "2", "--prompt", "128"],
+                          capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    pts = json.loads([l for l in proc.stdout.splitlines() if l.strip()][-1])["points"]
+    assert pts["decode_b1"] > 0 and pts["decode_b64"] > 0 and pts["decode_b2_through_generate"] > 0
+    assert all(not isinstance(v, (dict, list)) for v in pts.values()) and "decode_32b_b8" not in pts
     # the other shapes: the same keys, the shape's own sizes
     proc = subprocess.run(cmd + ["--shape", "4b", "--layers", "1", "--steps", "3", "--warmup", "1"], capture_output=True,
                           text=True, timeout=600)

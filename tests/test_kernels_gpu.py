@@ -569,6 +569,7 @@ ATTN_SHAPES = [
     (6, 2, 48, [33], [300], 50),                  # a chunk over several pages with a window
     (8, 4, 64, [5, 0, 190], [260, 129, 3], 70),   # head size 64 with a window, sequences that end inside pages
     (16, 2, 128, [0, 77], [513, 200], 0),         # eight heads a group, several tiles of 128 rows
+    (32, 8, 128, [5, 190], [260, 131], 70),       # the head size of the large models with a window whose edge lies inside pages
 ]
 
 
@@ -579,7 +580,9 @@ def test_attention_prefill(ops, dtype, nh, nkv, hd, past, new, window):
     lens = [p + n for p, n in zip(past, new)]
     width = max((T + 63) // 64 for T in lens) + 1
     table = shuffled_table(B, width, 3)
-    k, v = make_cache(B * width, nkv, hd, dtype, 30, fill="nan" if (hd == 64 and dtype == BF16) else "garbage")
+    # what lies in the pages behind a sequence's end is NaN for the head sizes of the kernel with 32 query rows a
+    # wave (and finite garbage elsewhere): a value that leaked from there, times a weight of zero, would show
+    k, v = make_cache(B * width, nkv, hd, dtype, 30, fill="nan" if (hd in (64, 128) and dtype == BF16) else "garbage")
     fill_sequences(k, v, table, lens, nkv, hd, dtype, 31)
     tok_seq, tok_pos, starts, past_t, len_t = step_arrays(past, new)
     N = len(tok_seq)
