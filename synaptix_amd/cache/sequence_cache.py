@@ -69,13 +69,18 @@ class _Group:
     k: torch.Tensor = None
     v: torch.Tensor = None
     spare_page: int = 0               # a page beyond the pool that no sequence owns (padding rows write there)
+    n_pages: int = 0                  # pages of the group's pool (a group that keeps a window may have fewer)
 
 
 class SequenceCache:
     def __init__(self, needs: list, max_tokens: int, max_slots: int | None, dtype, device,
-                 max_positions: int | None = None):
+                 max_positions: int | None = None, max_step_tokens: int | None = None):
         """needs[i]: KvNeed, StateNeed or None of cache layer i.  max_tokens: the most tokens that
-        live sequences hold together, each sequence's count rounded up to whole pages."""
+        live sequences hold together, each sequence's count rounded up to whole pages.
+        max_step_tokens: the most tokens that one step brings for one sequence, if the caller can promise
+        it: a group of layers that keeps a window then gets pages for the window and one such step of every
+        slot only (a step holds the pages of all its new tokens before the window gives old ones back), not
+        for max_tokens; None: every group gets pages for max_tokens."""
         if max_tokens <= 0:
             raise CacheError("max_tokens must be positive")
         self.dtype, self.device = dtype, torch.device(device)
@@ -108,17 +113,23 @@ class SequenceCache:
         if rt.lib().syn_rt_page_tokens() != PAGE_TOKENS:
             raise RuntimeError("the runtime library was built for another page size")
         windows = [-1 if g.need.window is None else int(g.need.window) for g in self.groups]
-        self._h = rt.lib().syn_cache_new(len(self.groups), rt.longs(windows), self.n_pages, self.max_slots,
+        for g in self.groups:
+            g.n_pages = self.n_pages
+            if g.need.window is not None and max_step_tokens is not None:
+                # at most window + step tokens of a sequence are held at once, and they may begin anywhere in a page
+                g.n_pages = min(self.n_pages, self.max_slots * (pages_for(int(g.need.window) + int(max_step_tokens)) + 1))
+        self._h = rt.lib().syn_cache_new(len(self.groups), rt.longs(windows), self.n_pages,
+                                         rt.ints([g.n_pages for g in self.groups]), self.max_slots,
                                          -1 if max_positions is None else int(max_positions))
         if not self._h:
             raise CacheError(rt.last_error())
         for gi, g in enumerate(self.groups):
             n, nd = len(g.layers), g.need
-            g.pool = _GroupPool(self, gi, self.n_pages)
+            g.pool = _GroupPool(self, gi, g.n_pages)
             # zeros: what a kernel may touch beyond a sequence's end is at least a number
-            g.spare_page = self.n_pages
-            g.k = torch.zeros((n, self.n_pages + 1, nd.kv_heads, PAGE_TOKENS, nd.head_dim), dtype=dtype, device=self.device)
-            g.v = torch.zeros((n, self.n_pages + 1, nd.kv_heads, nd.head_dim, PAGE_TOKENS), dtype=dtype, device=self.device)
+            g.spare_page = g.n_pages
+            g.k = torch.zeros((n, g.n_pages + 1, nd.kv_heads, PAGE_TOKENS, nd.head_dim), dtype=dtype, device=self.device)
+            g.v = torch.zeros((n, g.n_pages + 1, nd.kv_heads, nd.head_dim, PAGE_TOKENS), dtype=dtype, device=self.device)
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
@@ -166,6 +177,18 @@ class SequenceCache:
         out = C.c_long()
         rt.check(rt.lib().syn_cache_pages_needed(self._h, self._sid(sid), int(n_new), C.byref(out)))
         return out.value
+
+    def pages_for_sequence(self, total_tokens: int, longest_step: int) -> list:
+        """Pages of each group that a sequence of total_tokens can hold at once when no step brings more than
+        longest_step of its tokens: all its pages where every key is kept, the window's and one step's where a window
+        is (a planner's bound: what `reserve` will ask for at most)."""
+        out = []
+        for g in self.groups:
+            n = pages_for(total_tokens)
+            if g.need.window is not None:
+                n = min(n, pages_for(int(g.need.window) + int(longest_step)) + 1)
+            out.append(n)
+        return out
 
     def reserve(self, sid: int, n_new: int) -> None:
         """Hold pages for n_new more tokens in every group, or raise CacheFull and change nothing."""

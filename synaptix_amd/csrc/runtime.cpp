@@ -183,15 +183,23 @@ RT_API const char* syn_rt_last_error() { return g_error; }
 RT_API int syn_rt_page_tokens() { return PAGE_TOKENS; }
 
 // ------------------------------------------------------------------ cache bookkeeping
-RT_API void* syn_cache_new(int n_groups, const long* windows, int n_pages, int max_slots, long max_positions) {
+// group_pages: the pages of each group's pool (a group that keeps a window needs fewer than one that keeps every
+// key), or null: n_pages for every group
+RT_API void* syn_cache_new(int n_groups, const long* windows, int n_pages, const int* group_pages, int max_slots,
+                           long max_positions) {
   if (n_groups < 0 || n_pages <= 0 || max_slots <= 0) {
     fail(MISUSE, "a cache needs pages and slots (%d pages, %d slots)", n_pages, max_slots);
     return nullptr;
   }
+  for (int g = 0; group_pages && g < n_groups; ++g)
+    if (group_pages[g] <= 0) {
+      fail(MISUSE, "group %d of the cache has %d pages", g, group_pages[g]);
+      return nullptr;
+    }
   Cache* c = new Cache;
   c->n_pages = n_pages, c->max_slots = max_slots, c->max_positions = max_positions;
   for (int g = 0; g < n_groups; ++g) {
-    c->pools.emplace_back(n_pages);
+    c->pools.emplace_back(group_pages ? group_pages[g] : n_pages);
     c->windows.push_back(windows[g]);
   }
   c->slots.resize(max_slots);
@@ -381,19 +389,21 @@ RT_API int syn_cache_check(void* h) {
   for (size_t g = 0; g < c->pools.size(); ++g) {
     const int rc = c->pools[g].check();
     if (rc) return rc;
-    std::vector<uint8_t> owned(c->n_pages, 0);
+    const int pool_pages = c->pools[g].n_pages;
+    std::vector<uint8_t> owned(pool_pages, 0);
     long held = 0;
     for (const Slot& s : c->slots) {
       if (!s.live) continue;
       for (int p : s.pages[g]) {
         if (p < 0) continue;
+        if (p >= pool_pages) return fail(MISUSE, "group %d: page %d does not exist", (int)g, p);
         if (owned[p]) return fail(MISUSE, "group %d: a page is held by two sequences", (int)g);
         owned[p] = 1;
         ++held;
       }
     }
-    if (held + c->pools[g].free_pages() != c->n_pages)
-      return fail(MISUSE, "group %d: %ld pages lost", (int)g, c->n_pages - held - c->pools[g].free_pages());
+    if (held + c->pools[g].free_pages() != pool_pages)
+      return fail(MISUSE, "group %d: %ld pages lost", (int)g, pool_pages - held - c->pools[g].free_pages());
   }
   return OK;
 }

@@ -37,8 +37,9 @@ def parse_dtype(dtype) -> torch.dtype:
 
 
 class Engine:
-    def __init__(self, model, dtype, max_tokens: int, max_slots: int | None = None):
-        """`model` has its weights loaded on a GPU."""
+    def __init__(self, model, dtype, max_tokens: int, max_slots: int | None = None, max_step_tokens: int | None = None):
+        """`model` has its weights loaded on a GPU.  max_step_tokens: see SequenceCache (smaller storage for
+        groups of layers that keep a window, if no step brings more tokens than this for one sequence)."""
         self.model = model
         self.dtype = parse_dtype(dtype)
         self.device = model.device
@@ -52,7 +53,7 @@ class Engine:
                 max_positions = cap if max_positions is None else min(max_positions, cap)
         self.max_positions = max_positions
         self.cache = SequenceCache(model.cache_needs(), max_tokens, max_slots, self.dtype, self.device,
-                                   max_positions=max_positions)
+                                   max_positions=max_positions, max_step_tokens=max_step_tokens)
         self._scratch = ScratchPool(self.device)      # of the eager steps; captured steps have their own
         self._host = None
         self._dev = None

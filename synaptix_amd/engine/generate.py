@@ -52,8 +52,8 @@ class GenerationStats:
     batches_first_tokens: int = 0
 
 
-def plan_batch(waiting: list, prompt_lens: list, max_new: list, free_slots: int, free_pages: int,
-               max_batch: int | None, capacity: int | None, held: dict | None = None) -> list:
+def plan_batch(waiting: list, prompt_lens: list, max_new: list, free_slots: int, free_pages,
+               max_batch: int | None, capacity: int | None, held: dict | None = None, group_need=None) -> list:
     """Which of the waiting requests (indices, in order) start together now.
 
     A request needs a slot and pages for its prompt and all tokens it may produce, so that a
@@ -61,27 +61,31 @@ def plan_batch(waiting: list, prompt_lens: list, max_new: list, free_slots: int,
     fit ends the batch.  A request that can never fit raises ValueError.
     held: {request: tokens it keeps in a slot of its own}: such a request needs no slot and only the pages
     beyond those that its kept tokens lie in.
+    free_pages: one number, or one for each group of cache layers together with group_need(request, total tokens)
+    -> the pages of each group that the request can hold at once (groups that keep a window need fewer).
     """
-    chosen, pages, slots = [], 0, 0
+    many = isinstance(free_pages, (list, tuple))
+    free = list(free_pages) if many else [free_pages]
+    chosen, pages, slots = [], [0] * len(free), 0
     for r in waiting:
         total = prompt_lens[r] + max(max_new[r], 1)
         if capacity is not None:
             total = min(total, capacity)
-        need = pages_for(total)
+        need = list(group_need(r, total)) if (many and group_need is not None) else [pages_for(total)] * len(free)
         own_slot = held is not None and r in held
         if own_slot:
-            need = max(0, need - pages_for(held[r]))
+            need = [max(0, n - pages_for(held[r])) for n in need]
         if max_batch is not None and len(chosen) >= max_batch:
             break
-        if (not own_slot and slots >= free_slots) or pages + need > free_pages:
+        if (not own_slot and slots >= free_slots) or any(p + n > f for p, n, f in zip(pages, need, free)):
             break
         chosen.append(r)
-        pages += need
+        pages = [p + n for p, n in zip(pages, need)]
         slots += 0 if own_slot else 1
     if not chosen and waiting:
         r = waiting[0]
         raise ValueError(f"request {r} ({prompt_lens[r]} prompt tokens + {max_new[r]} new) does not fit the cache "
-                         f"({free_pages} pages of 64 tokens and {free_slots} slots are free)")
+                         f"({min(free)} pages of 64 tokens and {free_slots} slots are free)")
     return chosen
 
 
@@ -156,10 +160,15 @@ def generate(engine, prompts, config=None, on_token=None, max_batch: int | None 
     def kept_tokens(r):
         return min(engine.length(resume[r]), lens[r] - 1)
 
+    def group_need(r, total):
+        step = configs[r].prefill_batch if configs[r].prefill_batch > 0 else lens[r]
+        return engine.cache.pages_for_sequence(total, min(step, lens[r]))
+
     while waiting:
-        free_pages = min(g.pool.free_pages for g in engine.cache.groups) if engine.cache.groups else 1 << 30
+        free_pages = [g.pool.free_pages for g in engine.cache.groups] if engine.cache.groups else [1 << 30]
         batch = plan_batch(waiting, lens, max_new, engine.cache.free_slots, free_pages, max_batch,
-                           engine.max_positions, held={r: kept_tokens(r) for r in waiting if r in resume})
+                           engine.max_positions, held={r: kept_tokens(r) for r in waiting if r in resume},
+                           group_need=group_need if engine.cache.groups else None)
         waiting = waiting[len(batch):]
         stats.batches += 1
         live = []

@@ -21,7 +21,7 @@ _IP, _LP, _FP, _UP = C.POINTER(C.c_int), C.POINTER(C.c_long), C.POINTER(C.c_floa
 
 _SIGNATURES = {
     "syn_rt_page_tokens": (_I, []),
-    "syn_cache_new": (_P, [_I, _LP, _I, _I, _L]),
+    "syn_cache_new": (_P, [_I, _LP, _I, _IP, _I, _L]),
     "syn_cache_delete": (None, [_P]),
     "syn_cache_free_slots": (_I, [_P]),
     "syn_cache_free_pages": (_I, [_P, _I]),

@@ -94,6 +94,29 @@ def test_window_group_gives_pages_back_early():
     c.check()
 
 
+def test_window_group_of_its_own_size():
+    """With a promise about the longest step a group that keeps a window gets pages for the window and one step of
+    every slot, not for all tokens; its pool, its spare page and its storage follow, the other group keeps its size,
+    and long sequences still fit because the window gives pages back."""
+    c = SequenceCache([KvNeed(1, 16), KvNeed(1, 16, window=70)], 64 * 40, 2, torch.float32, "cpu", max_step_tokens=64)
+    full, win = c.groups[0], c.groups[1]
+    assert full.n_pages == 40 and win.n_pages == 2 * (3 + 1)           # window 70 + step 64 = 134 tokens: 3 pages, + 1
+    assert win.k.shape[1] == win.n_pages + 1 and win.spare_page == win.n_pages and full.k.shape[1] == 41
+    a, b = c.acquire(), c.acquire()
+    for _ in range(15):                                                # 960 tokens each, far beyond the small pool
+        for s in (a, b):
+            c.reserve(s, 64); c.commit(s, 64)
+        c.check()
+    assert c.length(a) == 960 and win.pool.free_pages >= 2 and full.pool.free_pages == 40 - 30
+    assert max(c.page_table(1, [a, b]).max(), 0) < win.n_pages
+    with pytest.raises(CacheFull):                                     # a step beyond the promise does not fit the small pool
+        c.reserve(a, 64 * 9)
+    c.check()
+    c.release(a); c.release(b)
+    assert win.pool.free_pages == win.n_pages and full.pool.free_pages == 40
+    c.check()
+
+
 def test_state_is_zeroed_when_a_slot_is_taken():
     c = make(needs=[StateNeed((4,))], max_slots=2)
     s = c.acquire()

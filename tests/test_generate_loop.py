@@ -108,6 +108,25 @@ def test_max_batch_and_page_budget():
     assert st.batches == 2 and outs[2].tokens == [4, 5, 6]
 
 
+def test_batches_are_planned_for_each_group_of_cache_layers():
+    """A group that keeps a window has a small pool of its own (with a promise about the longest step); the plan counts
+    each group's pages against that group's pool, so long prompts in chunks start together although the small pool
+    could never hold them whole."""
+    assert plan_batch([0, 1], [300, 300], [20, 20], free_slots=4, free_pages=[40, 8], max_batch=None, capacity=None,
+                      group_need=lambda r, total: [5, 4]) == [0, 1]
+    assert plan_batch([0, 1], [300, 300], [20, 20], free_slots=4, free_pages=[40, 7], max_batch=None, capacity=None,
+                      group_need=lambda r, total: [5, 4]) == [0]
+    eng = CounterEngine(max_tokens=64 * 40, max_slots=2)
+    eng.cache = SequenceCache([KvNeed(1, 16), KvNeed(1, 16, window=70)], 64 * 40, 2, torch.float32, "cpu", max_step_tokens=64)
+    assert eng.cache.groups[1].n_pages == 8
+    prompts = [[(3 * i) % V for i in range(300)], [(5 * i + 1) % V for i in range(290)]]
+    outs, st = generate(eng, prompts, GenerationConfig(max_new_tokens=20, prefill_batch=64))
+    assert st.batches == 1 and all(len(o.tokens) == 20 for o in outs)
+    assert eng.steps[0] == [(0, 64), (1, 64)]
+    eng.cache.check()
+    assert eng.cache.groups[1].pool.free_pages == 8 and eng.cache.groups[0].pool.free_pages == 40
+
+
 def test_capacity_ends_a_sequence():
     eng = CounterEngine(max_positions=6)
     outs, _ = generate(eng, [[1, 2, 3, 4]], GenerationConfig(max_new_tokens=50))
