@@ -151,7 +151,7 @@ __global__ void __launch_bounds__(PF_THREADS)
 attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
                     const int* __restrict__ page_table, int table_stride, const int* __restrict__ seq_start,
                     const int* __restrict__ seq_past, int n_seqs, bf16* __restrict__ out, float scale,
-                    int window, int nh, int nkv) {
+                    int window, int nh, int nkv, ScoreTerms terms) {
   extern __shared__ __attribute__((aligned(16))) bf16 lds[];  // [2][PF_TILE]
   // Heads run fastest through the grid; workgroups go round the eight dies in turn, and the heads are
   // dealt so that each die gets neighbouring heads, which share their K and V.
@@ -184,6 +184,8 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages
   const int g_kmin = window > 0 ? max(0, past + q0 - window + 1) : 0;
   const int kb_lo = g_kmin / SYN_PAGE, kb_hi = g_kmax / SYN_PAGE;
   const float scale2 = scale * 1.44269504088896340736f;
+  const bool with_terms = score_terms_on(terms);
+  const float slope = terms.slopes ? terms.slopes[head] : 0.f;
 
   AttnState<PF_QB> st;
   attn_init(st);
@@ -259,6 +261,9 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             float v = s[t][c][e] * scale2;
+            if (with_terms)   // in natural units, then into the exponent's base
+              v = score_with_terms(s[t][c][e] * scale, slope, terms.softcap, qpos[c], key0 + acc_key(t, g4, e)) *
+                  1.44269504088896340736f;
             if (need_mask) {
               const int key = key0 + acc_key(t, g4, e);
               if (key > qpos[c] || key < lo[c]) v = -INFINITY;
@@ -551,12 +556,17 @@ attn_prefill32_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pag
 SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, const void* v_pages,
                                           const int* page_table, int table_stride, const int* seq_start,
                                           const int* seq_past, int n_seqs, int n_tokens, void* out, float scale,
-                                          int window, int nh, int nkv, int hd, int variant, hipStream_t stream) {
+                                          int window, int nh, int nkv, int hd, int variant, const float* slopes,
+                                          float softcap, hipStream_t stream) {
   // variant: 0 = whichever is faster for this head size, 1 = waves of 16 query rows (every head size),
-  // 2 = waves of 32 query rows (head sizes 64 and 128, a positive scale)
+  // 2 = waves of 32 query rows (head sizes 64 and 128, a positive scale, no terms on the scores)
+  // slopes [nh] float or null, softcap (0: none): see ScoreTerms; the kernel with waves of 16 rows applies them
   SYN_CHECK(variant >= 0 && variant <= 2, "attention_prefill: unknown variant %d", variant);
-  SYN_CHECK(variant != 2 || (PF2_OK && scale > 0.f), "attention_prefill: waves of 32 rows take head sizes 64 and 128 and "
-            "a positive scale (head size %d, scale %g)", HD, (double)scale);
+  SYN_CHECK(softcap >= 0.f, "attention_prefill: a soft cap of %g", (double)softcap);
+  const ScoreTerms terms = {slopes, softcap};
+  const bool with_terms = slopes != nullptr || softcap > 0.f;
+  SYN_CHECK(variant != 2 || (PF2_OK && scale > 0.f && !with_terms), "attention_prefill: waves of 32 rows take head sizes 64 "
+            "and 128, a positive scale and no terms on the scores (head size %d, scale %g)", HD, (double)scale);
   SYN_CHECK(hd == HD, "attention_prefill: library built for head size %d, called with %d", HD, hd);
   SYN_CHECK(n_seqs > 0 && n_tokens >= n_seqs && nh > 0 && nkv > 0, "attention_prefill: empty input");
   SYN_CHECK(nh % nkv == 0, "attention_prefill: %d heads do not divide into %d kv heads", nh, nkv);
@@ -571,7 +581,7 @@ SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, co
     SYN_CHECK(e == hipSuccess, "attention_prefill: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
   }
   if constexpr (PF2_OK) {
-    if (variant == 2 || (variant == 0 && scale > 0.f)) {
+    if (variant == 2 || (variant == 0 && scale > 0.f && !with_terms)) {
       attn_prefill32_kernel<<<dim3(nh, tiles), PF2_THREADS, 2 * PF2_BUF, stream>>>(
           (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, page_table, table_stride, seq_start, seq_past,
           n_seqs, (bf16*)out, scale, window, nh, nkv);
@@ -581,7 +591,7 @@ SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, co
   }
   attn_prefill_kernel<<<dim3(nh, tiles), PF_THREADS, lds, stream>>>(
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, page_table, table_stride, seq_start, seq_past, n_seqs,
-      (bf16*)out, scale, window, nh, nkv);
+      (bf16*)out, scale, window, nh, nkv, terms);
   SYN_LAUNCH_CHECK("attention_prefill");
   return 0;
 }
@@ -678,8 +688,10 @@ __device__ __forceinline__ void decode_scores(const QFrag& qf, const KvUnit& uni
 }
 
 // key0: the unit's first key
+// qpos: the last key position that this column may see (-1: none); pos: the query's own position; slope, cap: the
+// terms on the scores of this lane's head (with_terms false: none)
 __device__ __forceinline__ void decode_weights(AttnState<1>& st, f32x4 (&s)[2], int key0, int qpos, int lo, float scale,
-                                               int lane) {
+                                               int lane, bool with_terms, float slope, float cap, int pos) {
   const int g4 = lane / 16;
   float mloc = -INFINITY;
 #pragma unroll
@@ -688,6 +700,7 @@ __device__ __forceinline__ void decode_weights(AttnState<1>& st, f32x4 (&s)[2], 
     for (int e = 0; e < 4; ++e) {
       const int key = key0 + acc_key(t, g4, e);
       float v = s[t][e] * scale;
+      if (with_terms) v = score_with_terms(v, slope, cap, pos, key);
       if (key > qpos || key < lo) v = -INFINITY;
       s[t][e] = v;
       mloc = fmaxf(mloc, v);
@@ -762,7 +775,7 @@ __global__ void __launch_bounds__(DEC_MAX_WAVES * SYN_WAVE)
 attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages, bf16* __restrict__ v_pages,
                          const int* __restrict__ page_table, int table_stride, const int* __restrict__ seq_len,
                          float* __restrict__ partial, bf16* __restrict__ out, float scale, int window, int nh, int nkv,
-                         int n_splits, int cols_alloc, QkvIntake in) {
+                         int n_splits, int cols_alloc, QkvIntake in, ScoreTerms terms) {
   // LDS: with STAGED first a piece of STAGE_BYTES for each wave; then
   //      sm[waves][16] running maxima, sl[waves][16] sums, so[waves][cols_alloc][HD + 4] outputs;
   // FUSED: then xs[waves][HD] floats, snew[16] scores of the new key, qs[cols_alloc][HD], knew[HD], vnew[HD] bf16
@@ -784,6 +797,8 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
   const int n_cols = min(16, g - chunk * 16);
   const bool new_key = FUSED && in.own_kv;            // the newest key is not read from the cache
   const bool adds_new = new_key && split == 0;        // this workgroup makes it and adds it
+  const bool with_terms = score_terms_on(terms);
+  const float slope = (terms.slopes && valid) ? terms.slopes[kvh * g + hg] : 0.f;
 
   // keys read from the cache: all of them, or all but the newest; the units of this split; the first
   // unit of this wave is requested at once, before the workgroup prepares its q heads
@@ -902,7 +917,8 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
         float dot = 0.f;
         for (int d = lane; d < HD; d += SYN_WAVE) dot += (float)qs[c * HD + d] * (float)knew[d];
         dot = wave_sum(dot);
-        if (lane == 0) snew[c] = dot * scale;
+        // (the new key lies at the query's own position: a soft cap applies, a penalty in the distance is zero)
+        if (lane == 0) snew[c] = with_terms ? score_with_terms(dot * scale, 0.f, terms.softcap, pos, pos) : dot * scale;
       }
     }
   }
@@ -932,7 +948,7 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
       decode_scores(qf, unit, s);
       if (next < u1) load_k_decode(unit, k_pages + next_base, lane);
     }
-    decode_weights(st, s, key0, valid ? q_lim : -1, lo, scale, lane);
+    decode_weights(st, s, key0, valid ? q_lim : -1, lo, scale, lane, with_terms, slope, terms.softcap, pos);
     decode_values(st, unit, s, key0, n_old, lane);
     if (next < u1) load_v_decode(unit, v_pages + next_base, lane);
   }
@@ -1045,7 +1061,9 @@ static hipError_t raise_decode_lds() {
 // workspace: n_seqs * nh * n_splits * (HD + 2) floats (unused with one split)
 static int launch_decode(const void* q, const QkvIntake* in, void* k_pages, void* v_pages, const int* page_table,
                          int table_stride, const int* seq_len, int n_seqs, void* out, float* workspace, int n_splits,
-                         float scale, int window, int nh, int nkv, int hd, hipStream_t stream) {
+                         float scale, int window, int nh, int nkv, int hd, hipStream_t stream,
+                         ScoreTerms terms = ScoreTerms{nullptr, 0.f}) {
+  SYN_CHECK(terms.softcap >= 0.f, "attention_decode: a soft cap of %g", (double)terms.softcap);
   SYN_CHECK(hd == HD, "attention_decode: library built for head size %d, called with %d", HD, hd);
   SYN_CHECK(n_seqs > 0 && nh > 0 && nkv > 0 && n_splits > 0, "attention_decode: empty input");
   SYN_CHECK(nh % nkv == 0, "attention_decode: %d heads do not divide into %d kv heads", nh, nkv);
@@ -1071,11 +1089,11 @@ static int launch_decode(const void* q, const QkvIntake* in, void* k_pages, void
   if (in)
     attn_decode_split_kernel<true><<<grid, waves * SYN_WAVE, lds, stream>>>(
         nullptr, (bf16*)k_pages, (bf16*)v_pages, page_table, table_stride, seq_len, workspace, (bf16*)out, scale,
-        window, nh, nkv, n_splits, cols_alloc, *in);
+        window, nh, nkv, n_splits, cols_alloc, *in, terms);
   else
     attn_decode_split_kernel<false><<<grid, waves * SYN_WAVE, lds, stream>>>(
         (const bf16*)q, (bf16*)k_pages, (bf16*)v_pages, page_table, table_stride, seq_len, workspace, (bf16*)out,
-        scale, window, nh, nkv, n_splits, cols_alloc, QkvIntake{});
+        scale, window, nh, nkv, n_splits, cols_alloc, QkvIntake{}, terms);
   SYN_LAUNCH_CHECK("attention_decode_split");
   if (n_splits > 1) {
     attn_decode_merge_kernel<<<n_seqs * nh, SYN_WAVE, 0, stream>>>(workspace, (bf16*)out, n_splits);
@@ -1090,6 +1108,16 @@ SYN_EXPORT int syn_attention_decode_bf16(const void* q, const void* k_pages, con
                                          int nkv, int hd, hipStream_t stream) {
   return launch_decode(q, nullptr, (void*)k_pages, (void*)v_pages, page_table, table_stride, seq_len, n_seqs, out,
                        workspace, n_splits, scale, window, nh, nkv, hd, stream);
+}
+
+// the same with terms on the scores: slopes [nh] float or null, softcap (0: none), see ScoreTerms
+SYN_EXPORT int syn_attention_decode_terms_bf16(const void* q, const void* k_pages, const void* v_pages,
+                                               const int* page_table, int table_stride, const int* seq_len, int n_seqs,
+                                               void* out, float* workspace, int n_splits, float scale, int window,
+                                               int nh, int nkv, int hd, const float* slopes, float softcap,
+                                               hipStream_t stream) {
+  return launch_decode(q, nullptr, (void*)k_pages, (void*)v_pages, page_table, table_stride, seq_len, n_seqs, out,
+                       workspace, n_splits, scale, window, nh, nkv, hd, stream, ScoreTerms{slopes, softcap});
 }
 
 // ---- the same without a workspace argument: see no_alloc.h ----
@@ -1153,7 +1181,8 @@ SYN_EXPORT int syn_attention_decode_fused_bf16(const void* qkv, int n_parts, voi
                                                int window, int nh, int nkv, int hd, const void* q_gain,
                                                const void* k_gain, int gain_is_f32, float gain_offset, float eps,
                                                const float* cos_t,
-                                               const float* sin_t, int rot, int own_kv, hipStream_t stream) {
+                                               const float* sin_t, int rot, int own_kv, const float* slopes,
+                                               float softcap, hipStream_t stream) {
   SYN_CHECK(rot % 2 == 0 && rot >= 0 && rot <= hd, "attention_decode_fused: rotary size %d does not fit head size %d",
             rot, hd);
   SYN_CHECK((cos_t == nullptr) == (sin_t == nullptr), "attention_decode_fused: cos and sin come together");
@@ -1165,5 +1194,5 @@ SYN_EXPORT int syn_attention_decode_fused_bf16(const void* qkv, int n_parts, voi
   in.q_gain = q_gain, in.k_gain = k_gain, in.gain_is_f32 = gain_is_f32, in.gain_offset = gain_offset, in.eps = eps;
   in.cos_t = cos_t, in.sin_t = sin_t, in.rot = rot, in.own_kv = own_kv;
   return launch_decode(nullptr, &in, k_pages, v_pages, page_table, table_stride, seq_len, n_seqs, out, workspace,
-                       n_splits, scale, window, nh, nkv, hd, stream);
+                       n_splits, scale, window, nh, nkv, hd, stream, ScoreTerms{slopes, softcap});
 }

@@ -16,7 +16,7 @@ __global__ void __launch_bounds__(SYN_WAVE)
 attn_f32_kernel(const float* __restrict__ q, const float* __restrict__ k_pages, const float* __restrict__ v_pages,
                 const int* __restrict__ page_table, int table_stride, const int* __restrict__ tok_seq,
                 const int* __restrict__ tok_pos, float* __restrict__ out, float scale, int window, int nh, int nkv,
-                int hd) {
+                int hd, ScoreTerms terms) {
   __shared__ float qs[ATTN32_MAX_HD];
   __shared__ float ps[SYN_PAGE];
   const int tok = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
@@ -27,6 +27,8 @@ attn_f32_kernel(const float* __restrict__ q, const float* __restrict__ k_pages, 
   __syncthreads();
 
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const bool with_terms = score_terms_on(terms);
+  const float slope = terms.slopes ? terms.slopes[head] : 0.f;
   float m = -INFINITY, l = 0.f;
   float o[ATTN32_MAX_HD / SYN_WAVE] = {0.f, 0.f, 0.f, 0.f};
   for (int kb = lo / SYN_PAGE; kb <= pos / SYN_PAGE; ++kb) {
@@ -40,6 +42,7 @@ attn_f32_kernel(const float* __restrict__ q, const float* __restrict__ k_pages, 
       float dot = 0.f;
       for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], kr[d], dot);
       s = dot * scale;
+      if (with_terms) s = score_with_terms(s, slope, terms.softcap, pos, key);
     }
     const float m_new = fmaxf(m, wave_max(s));  // every block of the range holds a visible key
     const float alpha = expf(m - m_new);
@@ -71,14 +74,18 @@ attn_f32_kernel(const float* __restrict__ q, const float* __restrict__ k_pages, 
   }
 }
 
+// slopes [nh] float or null, softcap (0: none): see ScoreTerms
 SYN_EXPORT int syn_attention_f32(const float* q, const float* k_pages, const float* v_pages, const int* page_table,
                                  int table_stride, const int* tok_seq, const int* tok_pos, float* out, float scale,
-                                 int window, int n_tokens, int nh, int nkv, int hd, hipStream_t stream) {
+                                 int window, int n_tokens, int nh, int nkv, int hd, const float* slopes, float softcap,
+                                 hipStream_t stream) {
+  SYN_CHECK(softcap >= 0.f, "attention_f32: a soft cap of %g", (double)softcap);
   SYN_CHECK(n_tokens > 0 && nh > 0 && nkv > 0, "attention_f32: empty input");
   SYN_CHECK(nh % nkv == 0, "attention_f32: %d heads do not divide into %d kv heads", nh, nkv);
   SYN_CHECK(hd > 0 && hd <= ATTN32_MAX_HD, "attention_f32: head size %d is outside 1..%d", hd, ATTN32_MAX_HD);
   attn_f32_kernel<<<dim3(n_tokens, nh), SYN_WAVE, 0, stream>>>(q, k_pages, v_pages, page_table, table_stride, tok_seq,
-                                                               tok_pos, out, scale, window, nh, nkv, hd);
+                                                               tok_pos, out, scale, window, nh, nkv, hd,
+                                                               ScoreTerms{slopes, softcap});
   SYN_LAUNCH_CHECK("attention_f32");
   return 0;
 }

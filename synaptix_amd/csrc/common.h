@@ -102,6 +102,22 @@ __device__ __forceinline__ float gate_activation(int act, float g) {
 }
 __device__ __forceinline__ float gated(int act, float gate, float up) { return gate_activation(act, gate) * up; }
 
+// ---- what an attention kernel may do to a scaled score before the mask and the softmax ----
+// A soft cap, cap * tanh(score / cap), and a penalty in the distance between query and key, - slope[head] * (q - k)
+// (the linear bias of crates/synaptix-ops/src/pos/alibi.rs:47-66 for keys at or before the query).  Neither is set
+// by the one architecture built here (slopes == nullptr, cap == 0: the kernels then run the code they ran before
+// these arguments existed); they are what a position scheme that acts on the scores, or a capped attention, needs.
+struct ScoreTerms {
+  const float* slopes;   // [n_heads] or nullptr
+  float softcap;         // 0: none
+};
+__device__ __forceinline__ bool score_terms_on(const ScoreTerms& t) { return t.slopes != nullptr || t.softcap > 0.f; }
+// v: the scaled score in natural units; slope: of the query's head (0 without slopes)
+__device__ __forceinline__ float score_with_terms(float v, float slope, float cap, int q_pos, int key) {
+  if (cap > 0.f) v = cap * tanhf(v / cap);
+  return v - slope * (float)(q_pos - key);
+}
+
 // ---- reductions over the 64 lanes of a wave ----
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

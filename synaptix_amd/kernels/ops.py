@@ -486,9 +486,21 @@ def qk_norm_rope_kv_write(qkv, q_out, k_pages, v_pages, page_table, tok_seq, tok
           1 if write_kv else 0, _stream())
 
 
+def _score_terms(name, slopes, softcap, n_heads):
+    """The optional terms on the scores as the entry points take them: (pointer to slopes [n_heads] float or null,
+    soft cap as a C float; 0 = none).  score = cap * tanh(score / cap), then - slope[head] * (query position - key
+    position); see csrc/common.h: ScoreTerms."""
+    if slopes is not None:
+        _need(slopes, name + ".slopes", _F32, (n_heads,))
+    softcap = float(softcap or 0.0)
+    if softcap < 0.0:
+        raise KernelError(f"{name}: a soft cap of {softcap}")
+    return _ptr(slopes), ctypes.c_float(softcap)
+
+
 def attention_f32(q, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale, window, n_heads, n_kv_heads,
-                  head_dim):
-    """True 32-bit attention of every token (prefill and decode alike)."""
+                  head_dim, slopes=None, softcap=0.0):
+    """True 32-bit attention of every token (prefill and decode alike).  slopes, softcap: see _score_terms."""
     nh, nkv, hd = n_heads, n_kv_heads, head_dim
     _need(q, "attention_f32.q", _F32, (None, nh * hd))
     N = q.shape[0]
@@ -499,7 +511,7 @@ def attention_f32(q, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale,
     _need(out, "attention_f32.out", _F32, (N, nh * hd))
     _call(load_library("core"), "syn_attention_f32", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
           page_table.shape[1], _ptr(tok_seq), _ptr(tok_pos), _ptr(out), ctypes.c_float(scale), int(window or 0),
-          N, nh, nkv, hd, _stream())
+          N, nh, nkv, hd, *_score_terms("attention_f32", slopes, softcap, nh), _stream())
 
 
 def _attn_lib(hd):
@@ -509,11 +521,12 @@ def _attn_lib(hd):
 
 
 def attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, seq_past, out, scale, window, n_heads,
-                           n_kv_heads, head_dim, variant=0):
+                           n_kv_heads, head_dim, variant=0, slopes=None, softcap=0.0):
     """Causal attention of the new tokens of each sequence over its cache (which already holds them).
     seq_start [B+1]: offsets of the sequences' new tokens in q; seq_past [B]: tokens cached before.
     variant: 0 = the kernel's own choice, 1 = waves of 16 query rows (every head size), 2 = waves of 32
-    query rows (head sizes 64 and 128); for comparisons."""
+    query rows (head sizes 64 and 128); for comparisons.  slopes, softcap: see _score_terms (they take the kernel
+    with waves of 16 rows)."""
     nh, nkv, hd = n_heads, n_kv_heads, head_dim
     _need(q, "attention_prefill.q", _BF16, (None, nh * hd))
     N = q.shape[0]
@@ -527,7 +540,7 @@ def attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, seq_past,
     _need(out, "attention_prefill.out", _BF16, (N, nh * hd))
     _call(_attn_lib(hd), "syn_attention_prefill_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
           page_table.shape[1], _ptr(seq_start), _ptr(seq_past), B, N, _ptr(out), ctypes.c_float(scale),
-          int(window or 0), nh, nkv, hd, int(variant), _stream())
+          int(window or 0), nh, nkv, hd, int(variant), *_score_terms("attention_prefill", slopes, softcap, nh), _stream())
 
 
 def decode_splits(n_seqs, n_kv_heads, max_pages):
@@ -550,9 +563,9 @@ def decode_splits(n_seqs, n_kv_heads, max_pages):
 
 
 def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
-                          n_heads, n_kv_heads, head_dim):
+                          n_heads, n_kv_heads, head_dim, slopes=None, softcap=0.0):
     """One query for each sequence (its last token, already in the cache); seq_len [B] counts it.
-    workspace: float [B * nh * n_splits * (hd + 2)]."""
+    workspace: float [B * nh * n_splits * (hd + 2)].  slopes, softcap: see _score_terms."""
     nh, nkv, hd = n_heads, n_kv_heads, head_dim
     _need(q, "attention_decode.q", _BF16, (None, nh * hd))
     B = q.shape[0]
@@ -565,14 +578,19 @@ def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspa
     _need(workspace, "attention_decode.workspace", _F32)
     if workspace.numel() < B * nh * n_splits * (hd + 2):
         raise KernelError(f"attention_decode: workspace of {workspace.numel()} floats is too small")
-    _call(_attn_lib(hd), "syn_attention_decode_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
+    if slopes is None and not softcap:
+        _call(_attn_lib(hd), "syn_attention_decode_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
+              page_table.shape[1], _ptr(seq_len), B, _ptr(out), _ptr(workspace), int(n_splits), ctypes.c_float(scale),
+              int(window or 0), nh, nkv, hd, _stream())
+        return
+    _call(_attn_lib(hd), "syn_attention_decode_terms_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
           page_table.shape[1], _ptr(seq_len), B, _ptr(out), _ptr(workspace), int(n_splits), ctypes.c_float(scale),
-          int(window or 0), nh, nkv, hd, _stream())
+          int(window or 0), nh, nkv, hd, *_score_terms("attention_decode", slopes, softcap, nh), _stream())
 
 
 def attention_decode_fused_bf16(qkv, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
                                 n_heads, n_kv_heads, head_dim, q_gain, k_gain, eps, cos, sin, write_kv=True,
-                                gain_offset=0.0):
+                                gain_offset=0.0, slopes=None, softcap=0.0):
     """attention_decode_bf16 for one new token a sequence whose q, k and v come straight from the
     fused projection: qkv [B, (nh + 2 nkv) * hd] in bf16, or float partial sums [S, B, ...] that are
     added first.  The q/k RMSNorm (if gains are given), the rotation at position seq_len - 1 (if
@@ -614,7 +632,8 @@ def attention_decode_fused_bf16(qkv, k_pages, v_pages, page_table, seq_len, out,
     _call(_attn_lib(hd), "syn_attention_decode_fused_bf16", _ptr(qkv), n_parts, _ptr(k_pages), _ptr(v_pages),
           _ptr(page_table), page_table.shape[1], _ptr(seq_len), B, _ptr(out), _ptr(workspace), int(n_splits),
           ctypes.c_float(scale), int(window or 0), nh, nkv, hd, _ptr(q_gain), _ptr(k_gain), gain_f32,
-          ctypes.c_float(gain_offset), ctypes.c_float(eps), _ptr(cos), _ptr(sin), rot, 1 if write_kv else 0, _stream())
+          ctypes.c_float(gain_offset), ctypes.c_float(eps), _ptr(cos), _ptr(sin), rot, 1 if write_kv else 0,
+          *_score_terms("attention_decode_fused", slopes, softcap, nh), _stream())
 
 
 # ----------------------------------------------------------------------------- sampling

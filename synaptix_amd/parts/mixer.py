@@ -45,7 +45,7 @@ class GqaAttention(Mixer):
 
     def __init__(self, prefix: str, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, *,
                  position: Position | None = None, qk_norm_eps: float | None = None, scale: float | None = None,
-                 window: int | None = None, qk_gain_offset: float = 0.0):
+                 window: int | None = None, qk_gain_offset: float = 0.0, score_softcap: float | None = None):
         if n_kv_heads <= 0 or n_heads % n_kv_heads:
             raise ValueError(f"{n_heads} heads do not divide into {n_kv_heads} kv heads")
         self.prefix = prefix
@@ -55,6 +55,10 @@ class GqaAttention(Mixer):
         self.qk_gain_offset = float(qk_gain_offset)     # the q/k gains are this + their tensors
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
         self.window = window
+        # a soft cap on the scaled scores, cap * tanh(score / cap); None: none.  What the position scheme adds to the
+        # scores (Position.score_slopes) is asked for at the first step.
+        self.score_softcap = float(score_softcap) if score_softcap else 0.0
+        self._slopes = {}
         self.w_qkv = self.w_o = self.q_gain = self.k_gain = None
 
     def tensor_specs(self):
@@ -90,9 +94,17 @@ class GqaAttention(Mixer):
             raise ValueError(f"{self.prefix}: the bf16 attention kernels take head sizes in steps of 16 "
                              f"(16, 32, ..., {ops.MAX_HEAD_DIM}); {self.hd} runs in float32 only")
 
+    def _score_terms(self, device):
+        key = str(device)
+        if key not in self._slopes:
+            sl = self.position.score_slopes(self.nh, device)
+            self._slopes[key] = None if sl is None else sl.to(device=device, dtype=torch.float32).contiguous()
+        return dict(slopes=self._slopes[key], softcap=self.score_softcap)
+
     def forward(self, h, ctx, cache, owner=True):
         nh, nkv, hd = self.nh, self.nkv, self.hd
         N, act = h.shape[0], h.dtype
+        terms = self._score_terms(h.device)
         cap = self.position.capacity
         if cap is not None and ctx.max_position >= cap:
             raise ValueError(f"position {ctx.max_position} is beyond the position encoding's capacity {cap}")
@@ -118,7 +130,7 @@ class GqaAttention(Mixer):
             ops.attention_decode_fused_bf16(qkv, cache.k_pages, cache.v_pages, table, ctx.seq_len, o, work, splits,
                                             self.scale, window, nh, nkv, hd, self.q_gain, self.k_gain,
                                             self.qk_norm_eps or 0.0, cos, sin, write_kv=owner,
-                                            gain_offset=self.qk_gain_offset)
+                                            gain_offset=self.qk_gain_offset, **terms)
             return deferred_product(o, self.w_o, self.p_o)
         q = torch.empty((N, nh * hd), dtype=act, device=h.device)
         ops.qk_norm_rope_kv_write(qkv, q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos,
@@ -126,13 +138,13 @@ class GqaAttention(Mixer):
                                   write_kv=owner, gain_offset=self.qk_gain_offset)
         if act == torch.float32:
             ops.attention_f32(q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos, o, self.scale, window,
-                              nh, nkv, hd)
+                              nh, nkv, hd, **terms)
         elif ctx.one_token_each:
             splits = ctx.decode_splits(nkv, cache.group)
             work = ctx.scratch("attention_decode", N * nh * splits * (hd + 2))
             ops.attention_decode_bf16(q, cache.k_pages, cache.v_pages, table, ctx.seq_len, o, work, splits,
-                                      self.scale, window, nh, nkv, hd)
+                                      self.scale, window, nh, nkv, hd, **terms)
         else:
             ops.attention_prefill_bf16(q, cache.k_pages, cache.v_pages, table, ctx.seq_start, ctx.seq_past, o,
-                                       self.scale, window, nh, nkv, hd)
+                                       self.scale, window, nh, nkv, hd, **terms)
         return deferred_product(o, self.w_o, self.p_o)

@@ -18,6 +18,12 @@ class Position(Part):
         """(cos, sin) float [capacity, rotary_dim / 2] on `device`, or (None, None) for no rotation."""
         return None, None
 
+    def score_slopes(self, n_heads: int, device):
+        """A scheme that acts on the attention scores instead of on q and k: float [n_heads] on `device`, the
+        score of query position p and key position j <= p then gets - slope[head] * (p - j) (the linear bias of
+        crates/synaptix-ops/src/pos/alibi.rs:47-66); None (the default): nothing is added."""
+        return None
+
     capacity = None  # positions at and beyond it cannot be encoded; None: no limit
 
 

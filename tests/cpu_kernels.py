@@ -149,7 +149,7 @@ def qk_norm_rope_kv_write(qkv, q_out, k_pages, v_pages, page_table, tok_seq, tok
         v_pages[page, :, :, p % PAGE] = v[n].to(v_pages.dtype)
 
 
-def _attend(qrow, k_pages, v_pages, table_row, pos, scale, window, nh, nkv, hd):
+def _attend(qrow, k_pages, v_pages, table_row, pos, scale, window, nh, nkv, hd, slopes=None, softcap=0.0):
     T = pos + 1
     pages = table_row[:(T + PAGE - 1) // PAGE].long()
     K = k_pages[pages].to(F32).permute(1, 0, 2, 3).reshape(nkv, -1, hd)[:, :T]          # [nkv, T, hd]
@@ -159,29 +159,34 @@ def _attend(qrow, k_pages, v_pages, table_row, pos, scale, window, nh, nkv, hd):
     out = torch.empty(nh, hd)
     for h in range(nh):
         s = (K[h // g, lo:] @ qrow[h]) * scale
+        if softcap:                      # a soft cap on the scaled scores, then a penalty in the distance to the query
+            s = softcap * torch.tanh(s / softcap)
+        if slopes is not None:
+            s = s - float(slopes[h]) * (pos - torch.arange(lo, T, dtype=F32))
         p = torch.softmax(s, 0)
         out[h] = V[h // g][:, lo:] @ p
     return out
 
 
 def attention_f32(q, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale, window, n_heads, n_kv_heads,
-                  head_dim):
+                  head_dim, slopes=None, softcap=0.0):
     N = q.shape[0]
     qf = q.to(F32).view(N, n_heads, head_dim)
     for n in range(N):
         o = _attend(qf[n], k_pages, v_pages, page_table[int(tok_seq[n])], int(tok_pos[n]), scale, window,
-                    n_heads, n_kv_heads, head_dim)
+                    n_heads, n_kv_heads, head_dim, slopes, softcap)
         out[n] = o.reshape(-1).to(out.dtype)
 
 
 def attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, seq_past, out, scale, window, n_heads,
-                           n_kv_heads, head_dim):
+                           n_kv_heads, head_dim, variant=0, slopes=None, softcap=0.0):
     N = q.shape[0]
     qf = q.to(F32).view(N, n_heads, head_dim)
     for b in range(seq_past.shape[0]):
         for n in range(int(seq_start[b]), int(seq_start[b + 1])):
             pos = int(seq_past[b]) + n - int(seq_start[b])
-            o = _attend(qf[n], k_pages, v_pages, page_table[b], pos, scale, window, n_heads, n_kv_heads, head_dim)
+            o = _attend(qf[n], k_pages, v_pages, page_table[b], pos, scale, window, n_heads, n_kv_heads, head_dim,
+                        slopes, softcap)
             out[n] = o.reshape(-1).to(out.dtype)
 
 
@@ -190,18 +195,18 @@ def decode_splits(n_seqs, n_kv_heads, max_pages):
 
 
 def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
-                          n_heads, n_kv_heads, head_dim):
+                          n_heads, n_kv_heads, head_dim, slopes=None, softcap=0.0):
     B = q.shape[0]
     qf = q.to(F32).view(B, n_heads, head_dim)
     for b in range(B):
         o = _attend(qf[b], k_pages, v_pages, page_table[b], int(seq_len[b]) - 1, scale, window, n_heads,
-                    n_kv_heads, head_dim)
+                    n_kv_heads, head_dim, slopes, softcap)
         out[b] = o.reshape(-1).to(out.dtype)
 
 
 def attention_decode_fused_bf16(qkv, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
                                 n_heads, n_kv_heads, head_dim, q_gain, k_gain, eps, cos, sin, write_kv=True,
-                                gain_offset=0.0):
+                                gain_offset=0.0, slopes=None, softcap=0.0):
     B = qkv.shape[-2]
     q = torch.empty((B, n_heads * head_dim), dtype=torch.bfloat16)
     tok_seq = torch.arange(B, dtype=torch.int32)
@@ -209,7 +214,7 @@ def attention_decode_fused_bf16(qkv, k_pages, v_pages, page_table, seq_len, out,
     qk_norm_rope_kv_write(qkv, q, k_pages, v_pages, page_table, tok_seq, tok_pos, q_gain, k_gain, eps, cos, sin,
                           n_heads, n_kv_heads, head_dim, write_kv=write_kv, gain_offset=gain_offset)
     attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
-                          n_heads, n_kv_heads, head_dim)
+                          n_heads, n_kv_heads, head_dim, slopes, softcap)
 
 
 def sample_rows(logits, temperature, uniform, out):

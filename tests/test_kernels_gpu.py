@@ -331,8 +331,8 @@ def test_gated_product_over_weights_in_fragment_order(ops, M, I, K):
 
 
 @pytest.mark.parametrize("gain_dtype,gain_offset", [(BF16, 0.0), (F32, 1.0)])
-@pytest.mark.parametrize("M,H,K,N2", [(1, 64, 96, 48), (8, 4096, 4096, 6144), (5, 208, 1120, 80), (8, 4096, 12288, 24576),
-                                      (3, 10240, 64, 32), (16, 48, 32, 16400)])
+@pytest.mark.parametrize("M,H,K,N2", [(1, 64, 96, 48), (8, 4096, 4096, 6144), (5, 224, 1120, 80), (8, 4096, 12288, 24576),
+                                      (3, 10240, 64, 32), (16, 96, 32, 16400)])
 def test_norm_carried_between_two_products_over_packed_weights(ops, gain_dtype, gain_offset, M, H, K, N2):
     """The two halves of an RMSNorm between two products for few rows.  First half, as the epilogue of the product
     before it: resid += x . W^T, xs = gain * resid, ss = sums of resid^2 over groups of 16 columns.  Second half, as
@@ -610,6 +610,58 @@ def test_attention_prefill(ops, dtype, nh, nkv, hd, past, new, window):
             ops.attention_prefill_bf16(d(q), d(k), dv(v), d(table), d(starts), d(past_t), out, scale, window, nh, nkv,
                                        hd, variant=variant)
             close(out, want, 2e-2, 1e-2, what=f"attention prefill bf16, variant {variant}")
+
+
+@pytest.mark.parametrize("nh,nkv,hd,past,new,window,softcap,sloped", [
+    (4, 2, 16, [0, 0], [40, 130], 0, 0.0, True),          # a penalty in the distance alone
+    (8, 2, 64, [100, 0], [70, 129], 0, 2.0, False),       # a soft cap alone (head size 64: the kernel with 16 rows a wave takes it)
+    (32, 8, 128, [30], [300], 0, 1.0, True),              # both, at the head size and group of the large models
+    (6, 3, 48, [10, 0], [40, 200], 50, 3.0, True),        # with a window
+])
+def test_attention_with_terms_on_the_scores(ops, nh, nkv, hd, past, new, window, softcap, sloped):
+    """score = cap * tanh(score / cap) - slope[head] * (query position - key position) before mask and softmax, in
+    every attention kernel: 32-bit, prompt (bf16), single tokens in splits (bf16), against the plain statement."""
+    B = len(past)
+    lens = [p + n for p, n in zip(past, new)]
+    width = max((T + 63) // 64 for T in lens) + 1
+    table = shuffled_table(B, width, 5)
+    slopes = torch.tensor([0.5 ** (1 + h % 5) for h in range(nh)], dtype=F32) if sloped else None
+    tok_seq, tok_pos, starts, past_t, len_t = step_arrays(past, new)
+    N = len(tok_seq)
+    scale = 1 / math.sqrt(hd)
+    d = lambda t: None if t is None else t.to(DEV)
+    for dtype in (F32, BF16):
+        k, v = make_cache(B * width, nkv, hd, dtype, 50)
+        fill_sequences(k, v, table, lens, nkv, hd, dtype, 51)
+        q = rnd((N, nh * hd), 52, dtype, 2.0)              # scores large enough that the cap bends them
+        want = torch.empty((N, nh * hd), dtype=F32)
+        ref.attention_f32(q.float(), torch.nan_to_num(k.float()), torch.nan_to_num(v.float()), table, tok_seq, tok_pos, want,
+                          scale, window, nh, nkv, hd, slopes, softcap)
+        plain = torch.empty_like(want)
+        ref.attention_f32(q.float(), torch.nan_to_num(k.float()), torch.nan_to_num(v.float()), table, tok_seq, tok_pos, plain,
+                          scale, window, nh, nkv, hd)
+        assert float((want - plain).abs().max()) > 0.1     # the terms matter at these sizes
+        out = torch.empty((N, nh * hd), dtype=dtype, device=DEV)
+        if dtype == F32:
+            ops.attention_f32(d(q), d(k), dv(v), d(table), d(tok_seq), d(tok_pos), out, scale, window, nh, nkv, hd,
+                              slopes=d(slopes), softcap=softcap)
+            close(out, want, 2e-4, what="attention f32 with terms")
+            continue
+        ops.attention_prefill_bf16(d(q), d(k), dv(v), d(table), d(starts), d(past_t), out, scale, window, nh, nkv, hd,
+                                   slopes=d(slopes), softcap=softcap)
+        close(out, want, 2e-2, 1e-2, what="attention prefill bf16 with terms")
+        if hd in (64, 128):
+            with pytest.raises(Exception, match="no terms on the scores"):
+                ops.attention_prefill_bf16(d(q), d(k), dv(v), d(table), d(starts), d(past_t), out, scale, window, nh, nkv,
+                                           hd, variant=2, slopes=d(slopes), softcap=softcap)
+        # single tokens: the last token of each sequence as a decode step over the same cache
+        last = torch.tensor([int(starts[b + 1]) - 1 for b in range(B)])
+        outd = torch.empty((B, nh * hd), dtype=BF16, device=DEV)
+        for splits in (1, 3):
+            work = torch.empty(B * nh * splits * (hd + 2), dtype=F32, device=DEV)
+            ops.attention_decode_bf16(d(q[last].contiguous()), d(k), dv(v), d(table), d(torch.tensor(lens, dtype=I32)), outd,
+                                      work, splits, scale, window, nh, nkv, hd, slopes=d(slopes), softcap=softcap)
+            close(outd, want[last], 2e-2, 1e-2, what=f"attention decode bf16 with terms, {splits} splits")
 
 
 @pytest.mark.parametrize("nh,nkv,hd,lens,window,splits", [

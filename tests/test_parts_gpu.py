@@ -78,7 +78,7 @@ def test_rotary_part_tables():
 def test_attention_part_alone(dtype, nh, nkv, hd, rot, qk_norm, window):
     """GqaAttention with its own sizes and options (partial rotation, no q/k norm, a window, no
     rotation at all), a prompt and then single tokens, against the plain functions."""
-    from synaptix_amd.parts import GqaAttention, RotaryHalfSplit, NoPosition
+    from synaptix_amd.parts import GqaAttention, RotaryHalfSplit, NoPosition, as_delta
     from synaptix_amd.cache import SequenceCache
     H, S, eps = 40, 90, 1e-5
     pos = RotaryHalfSplit(1e4, rot, 256) if rot else NoPosition()
@@ -107,7 +107,7 @@ def test_attention_part_alone(dtype, nh, nkv, hd, rot, qk_norm, window):
     got = []
     for lo, hi in [(0, 70)] + [(i, i + 1) for i in range(70, S)]:
         ctx = one_sequence_ctx(cache, slot, hi - lo, dtype)
-        got.append(att.forward(x[lo:hi].to(DEV), ctx, cache.layer_view(0)))
+        got.append(as_delta(att.forward(x[lo:hi].to(DEV), ctx, cache.layer_view(0))))   # few rows: the product may come unrun
         cache.commit(slot, hi - lo)
     got = torch.cat(got).cpu()
     assert got.dtype == F32
@@ -119,12 +119,12 @@ def test_attention_part_alone(dtype, nh, nkv, hd, rot, qk_norm, window):
 def test_gated_mlp_part_alone(dtype, inter):
     """With 2048 intermediate values and few rows the last product comes as partial sums over
     slices of K, which the norm that follows adds up."""
-    from synaptix_amd.parts import GatedMlp, RmsNorm
+    from synaptix_amd.parts import GatedMlp, RmsNorm, as_delta
     ff = GatedMlp("m.", 56, inter)
     w = {n: rnd(s.shape, 40 + i, 0.2).to(dtype) for i, (n, s) in enumerate(ff.tensor_specs().items())}
     ff.load(lambda name: w[name].to(DEV))
     x = rnd((9, 56), 50).to(dtype)
-    got = ff.forward(x.to(DEV), None)
+    got = as_delta(ff.forward(x.to(DEV), None))
     if inter >= 2048 and dtype == BF16:
         assert got.dim() == 3 and got.shape[0] > 1
     if got.dim() == 3:
@@ -255,7 +255,7 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
 def test_toy_position_encoding_plugs_into_attention():
     """Another position encoding, defined here: angles that grow linearly with the index of the
     pair, on the first 8 of 16 dims.  The mixer only asks its position part for tables."""
-    from synaptix_amd.parts import GqaAttention, Position
+    from synaptix_amd.parts import GqaAttention, Position, as_delta
     from synaptix_amd.cache import SequenceCache
 
     class LinearFrequencies(Position):
@@ -292,7 +292,61 @@ def test_toy_position_encoding_plugs_into_attention():
         got = []
         for lo, hi in [(0, 33)] + [(i, i + 1) for i in range(33, S)]:
             ctx = one_sequence_ctx(cache, slot, hi - lo, dtype)
-            d = att.forward(x[lo:hi].to(DEV), ctx, cache.layer_view(0))
+            d = as_delta(att.forward(x[lo:hi].to(DEV), ctx, cache.layer_view(0)))
+            got.append(d.sum(0) if d.dim() == 3 else d)
+            cache.commit(slot, hi - lo)
+        err = (torch.cat(got).cpu() - want).abs().max()
+        assert err <= (2e-4 if dtype == F32 else 4e-2) * max(1.0, float(want.abs().max())), float(err)
+
+
+@pytest.mark.parametrize("softcap", [None, 1.5])
+def test_toy_position_scheme_that_acts_on_the_scores(softcap):
+    """A position scheme that is no rotation, defined here: a penalty on the scores that grows with the distance
+    between query and key, one slope a head (the reference's linear bias, crates/synaptix-ops/src/pos/alibi.rs:5-66),
+    with and without a soft cap on the scores.  The mixer asks its position part for the slopes and hands them to
+    whichever attention kernel runs: the prompt (whole and in a second chunk), then single tokens, in both types.
+    The slopes are steep enough that dropping them changes the result by far more than the tolerance."""
+    from synaptix_amd.parts import GqaAttention, Position, as_delta
+    from synaptix_amd.cache import SequenceCache
+
+    class DistancePenalty(Position):
+        def score_slopes(self, n_heads, device):
+            return torch.tensor([2.0 ** (-(h + 1) * 8.0 / n_heads) for h in range(n_heads)], dtype=F32).to(device)
+
+    H, S, nh, nkv, hd = 24, 150, 4, 2, 32
+    pos = DistancePenalty()
+    slopes = pos.score_slopes(nh, "cpu")
+    for dtype in (F32, BF16):
+        att = GqaAttention("a.", H, nh, nkv, hd, position=pos, score_softcap=softcap)
+        w = {n: rnd(s_.shape, 60 + i, 0.5).to(dtype) for i, (n, s_) in enumerate(att.tensor_specs().items())}
+        att.load(lambda name: w[name].to(DEV))
+        x = rnd((S, H), 70).to(dtype)
+        xf = x.float()
+        q = (xf @ w["a.q_proj.weight"].float().T).view(S, nh, hd)
+        k = (xf @ w["a.k_proj.weight"].float().T).view(S, nkv, hd)
+        v = (xf @ w["a.v_proj.weight"].float().T).view(S, nkv, hd)
+
+        def dense(with_terms):
+            out = torch.empty(S, nh, hd)
+            dist = (torch.arange(S)[:, None] - torch.arange(S)[None, :]).float()
+            for h in range(nh):
+                sc = (q[:, h] @ k[:, h // (nh // nkv)].T) / math.sqrt(hd)
+                if with_terms:
+                    if softcap:
+                        sc = softcap * torch.tanh(sc / softcap)
+                    sc = sc - slopes[h] * dist
+                sc = sc.masked_fill(dist < 0, float("-inf"))
+                out[:, h] = torch.softmax(sc, -1) @ v[:, h // (nh // nkv)]
+            return out.reshape(S, nh * hd) @ w["a.o_proj.weight"].float().T
+
+        want = dense(True)
+        assert float((want - dense(False)).abs().max()) > 0.2 * float(want.abs().max())      # the terms matter
+        cache = SequenceCache([att.cache_need()], 256, 1, dtype, DEV)
+        slot = cache.acquire()
+        got = []
+        for lo, hi in [(0, 70), (70, 140)] + [(i, i + 1) for i in range(140, S)]:
+            ctx = one_sequence_ctx(cache, slot, hi - lo, dtype)
+            d = as_delta(att.forward(x[lo:hi].to(DEV), ctx, cache.layer_view(0)))
             got.append(d.sum(0) if d.dim() == 3 else d)
             cache.commit(slot, hi - lo)
         err = (torch.cat(got).cpu() - want).abs().max()
