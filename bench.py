@@ -176,6 +176,8 @@ def main() -> int:
                     help="fewer layers than the model has (same layer sizes); both numbers are reported")
     ap.add_argument("--prompt", type=int, default=PROMPT,
                     help="tokens of every prompt (the contract's run has 2,048; the cache holds 8,192 a sequence)")
+    ap.add_argument("--context", type=int, default=8192,
+                    help="the longest sequence (positions and cache a sequence; the contract's run has 8,192)")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
     ap.add_argument("--no-packed-copies", action="store_true",
@@ -192,8 +194,11 @@ def main() -> int:
             return 2
         return unequal_prompts_through_generate(args, shape)
     prompt_len = args.prompt
-    if prompt_len < 1 or prompt_len + args.warmup + args.steps + 8 > 8192:
-        print(f"bench.py: --prompt {prompt_len} plus {args.warmup} + {args.steps} + 8 new tokens exceed the context of 8192")
+    if args.context < 64:
+        print(f"bench.py: --context {args.context} is too short")
+        return 2
+    if prompt_len < 1 or prompt_len + args.warmup + args.steps + 8 > args.context:
+        print(f"bench.py: --prompt {prompt_len} plus {args.warmup} + {args.steps} + 8 new tokens exceed the context of {args.context}")
         return 2
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -207,11 +212,11 @@ def main() -> int:
         from synaptix_amd.parts import keep_packed_copies
         keep_packed_copies(False)
     torch.manual_seed(0)
-    cfg = Qwen3Config.from_dict({**shape, "num_hidden_layers": args.layers})
+    cfg = Qwen3Config.from_dict({**shape, "num_hidden_layers": args.layers, "max_position_embeddings": args.context})
     batches = [args.batch] if args.no_points else sorted({args.batch, *POINTS[args.shape]})
     new_tokens = args.warmup + args.steps + 8
     per_seq = (prompt_len + new_tokens + 63) // 64 * 64
-    eng = Engine.from_config(cfg, seed=0, dtype="bfloat16", max_tokens=max(batches) * per_seq + 64, max_seq=8192)
+    eng = Engine.from_config(cfg, seed=0, dtype="bfloat16", max_tokens=max(batches) * per_seq + 64, max_seq=args.context)
     g = torch.Generator().manual_seed(0)
 
     def prompt():
@@ -241,8 +246,9 @@ def main() -> int:
     # ---- decode
     def decode(batch: int, warmup: int, steps: int):
         slots = [eng.acquire() for _ in range(batch)]
-        for lo in range(0, batch, 8):                       # prompts go in steps of 8 sequences
-            part = slots[lo:lo + 8]
+        group = max(1, min(8, 65536 // prompt_len))         # prompts go in steps of up to 8 sequences and 65,536 tokens
+        for lo in range(0, batch, group):
+            part = slots[lo:lo + group]
             lg = eng.step([(s, prompt()) for s in part], want="last")
             first = eng.sample(lg).cpu().tolist()
             if lo == 0:
@@ -311,7 +317,7 @@ def main() -> int:
         "dtype": "bf16", "data": "synthetic: seeded uniform token ids, random-init weights N(0, 0.02)",
         "config": {"model": f"Qwen3-{args.shape.upper()} shape", "layers": L, "model_layers": shape["num_hidden_layers"],
                    "hidden": H, "heads": nh, "kv_heads": nkv, "head_dim": hd, "intermediate": I, "vocab": V,
-                   "global_batch": args.batch, "seq_len": prompt_len, "context": 8192, "new_tokens": args.steps,
+                   "global_batch": args.batch, "seq_len": prompt_len, "context": args.context, "new_tokens": args.steps,
                    "tie_word_embeddings": cfg.tie_word_embeddings, "rope_theta": 1e6, "rms_norm_eps": 1e-6,
                    "parallelism": "single GPU", "graph": not args.no_graph},
         "prefill": prefill,
