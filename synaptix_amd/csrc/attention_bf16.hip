@@ -601,9 +601,30 @@ SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, co
 // the keys, in units of half a block); its waves take the split's units in turn and their states are
 // combined in LDS.
 // With one split the workgroup writes the output itself; else it writes a partial
-//   partial[(seq * nh + head) * n_splits + split] = { m, l, o[HD] }   (float)
-// and a second kernel merges the splits.
+//   partial[((first + split) * nh + head)] = { m, l, o[HD] }   (float; first: where the sequence's splits begin)
+// and the splits are merged, in their order: by the workgroup of the sequence that finishes last
+// (DecodeWork::counters given), or by a second kernel.
 constexpr int PART = HD + 2;
+
+// How the keys of a step's sequences are handed to workgroups.  Without `items` every sequence is cut
+// into the same n_splits (grid.x sequences, grid.z splits).  With `items` the grid's x counts items
+// {sequence, split, splits of the sequence, first} that the host has laid out, more splits for longer
+// sequences, the longest pieces first; an item with sequence -1 is spare and its workgroups leave at once.
+// counters: one int for each (sequence, grid.y), zero before the launch and zero again after it.
+struct DecodeWork {
+  float* partial;
+  int* counters;
+  const int4* items;
+};
+
+// A value that another workgroup, possibly on another XCD with a second-level cache of its own, reads
+// within the same launch: stored through to memory, and read from there.
+__device__ __forceinline__ void store_through(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_through(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 constexpr int DEC_MAX_WAVES = HD > 128 ? 4 : 8;  // as many as keep their registers (144 at a head size of 128, about twice that at 256) without spilling
 
 // The unit of a wave's work is half a block: 32 keys, whose K rows and whose V fragments are each one
@@ -774,8 +795,8 @@ template <bool FUSED>
 __global__ void __launch_bounds__(DEC_MAX_WAVES * SYN_WAVE)
 attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages, bf16* __restrict__ v_pages,
                          const int* __restrict__ page_table, int table_stride, const int* __restrict__ seq_len,
-                         float* __restrict__ partial, bf16* __restrict__ out, float scale, int window, int nh, int nkv,
-                         int n_splits, int cols_alloc, QkvIntake in, ScoreTerms terms) {
+                         DecodeWork work, bf16* __restrict__ out, float scale, int window, int nh, int nkv,
+                         int n_splits_all, int cols_alloc, QkvIntake in, ScoreTerms terms) {
   // LDS: with STAGED first a piece of STAGE_BYTES for each wave; then
   //      sm[waves][16] running maxima, sl[waves][16] sums, so[waves][cols_alloc][HD + 4] outputs;
   // FUSED: then xs[waves][HD] floats, snew[16] scores of the new key, qs[cols_alloc][HD], knew[HD], vnew[HD] bf16
@@ -787,7 +808,18 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
   constexpr int SO_LD = HD + 4;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / SYN_WAVE), lane = threadIdx.x % SYN_WAVE;
   char* stage = (char*)dec_lds + (size_t)wave * STAGE_BYTES;
-  const int seq = blockIdx.x, split = blockIdx.z;
+  int seq = blockIdx.x, split = blockIdx.z, n_splits = n_splits_all, first = blockIdx.x * n_splits_all;
+  if (work.items) {
+    const int4 item = work.items[blockIdx.x];
+    seq = __builtin_amdgcn_readfirstlane(item.x), split = __builtin_amdgcn_readfirstlane(item.y);
+    n_splits = __builtin_amdgcn_readfirstlane(item.z), first = __builtin_amdgcn_readfirstlane(item.w);
+    // (a spare item, or one that does not fit the launch: nothing is read or written for it)
+    const int n_seqs = gridDim.x / n_splits_all;
+    if (seq < 0 || seq >= n_seqs || n_splits < 1 || split < 0 || split >= n_splits || first < 0 ||
+        first + n_splits > (int)gridDim.x)
+      return;
+  }
+  float* const partial = work.partial;
   const int g = nh / nkv, chunks = (g + 15) / 16;
   const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
   const int kv_len = seq_len[seq], pos = kv_len - 1;
@@ -987,34 +1019,86 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
     if (n_splits == 1) {
       out[((size_t)seq * nh + head) * HD + d] = (bf16)(acc / lsum);
     } else {
-      float* p = partial + ((size_t)(seq * nh + head) * n_splits + split) * PART;
-      p[2 + d] = acc;
+      float* p = partial + (((size_t)first + split) * nh + head) * PART;
+      store_through(p + 2 + d, acc);
       if (d == 0) {
-        p[0] = m;
-        p[1] = lsum;
+        store_through(p, m);
+        store_through(p + 1, lsum);
       }
     }
+  }
+  if (n_splits == 1 || work.counters == nullptr) return;
+
+  // The workgroup of this (sequence, kv head, chunk) that finishes last merges the splits, in their
+  // order whatever the order of arrival.  Every wave's stores have been acknowledged by memory before
+  // its workgroup counts itself in; the one that counts last finds all of them there.
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+  __syncthreads();
+  int* const is_last = (int*)sm;        // (the loop above has finished reading sm)
+  if (threadIdx.x == 0) {
+    int* cnt = work.counters + (size_t)seq * gridDim.y + blockIdx.y;
+    const int before = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int last = before == n_splits - 1;
+    if (last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+    *is_last = last;
+  }
+  __syncthreads();
+  if (!*is_last) return;
+  for (int idx = threadIdx.x; idx < n_cols * HD; idx += blockDim.x) {
+    const int c = idx / HD, d = idx % HD;
+    const int head = kvh * g + chunk * 16 + c;
+    const float* p = partial + ((size_t)first * nh + head) * PART;
+    const size_t step = (size_t)nh * PART;   // from one split of the head to the next
+    float m = -INFINITY;
+    for (int s0 = 0; s0 < n_splits; s0 += 8) {
+      float ms[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) ms[u] = s0 + u < n_splits ? load_through(p + (s0 + u) * step) : -INFINITY;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) m = fmaxf(m, ms[u]);
+    }
+    float acc = 0.f, lsum = 0.f;
+    for (int s0 = 0; s0 < n_splits; s0 += 8) {   // eight splits' values in flight together, added in their order
+      float ms[8], ls[8], vs[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const bool on = s0 + u < n_splits;
+        ms[u] = on ? load_through(p + (s0 + u) * step) : -INFINITY;
+        ls[u] = on ? load_through(p + (s0 + u) * step + 1) : 0.f;
+        vs[u] = on ? load_through(p + (s0 + u) * step + 2 + d) : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (ms[u] == -INFINITY) continue;   // a split that had no keys weighs nothing and may hold anything
+        const float f = __expf(ms[u] - m);
+        acc += f * vs[u];
+        lsum += f * ls[u];
+      }
+    }
+    out[((size_t)seq * nh + head) * HD + d] = (bf16)(acc / lsum);
   }
 }
 
 // one wave a (sequence, head): lanes first share the splits' maxima and sums, then each takes output dims
 __global__ void __launch_bounds__(SYN_WAVE)
-attn_decode_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out, int n_splits) {
+attn_decode_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out, int n_splits, int nh) {
   const int row = blockIdx.x, lane = threadIdx.x;  // row = seq * nh + head
-  const float* p = partial + (size_t)row * n_splits * PART;
+  const int seq = row / nh, head = row % nh;
+  const size_t STEP = (size_t)nh * PART;           // from one split of the head to the next
+  const float* p = partial + ((size_t)seq * n_splits * nh + head) * PART;
   float wsum[(HD + SYN_WAVE - 1) / SYN_WAVE] = {};
   float l = 0.f;
   float m = -INFINITY;
   for (int s0 = 0; s0 < n_splits; s0 += SYN_WAVE) {  // maximum over all splits
     const int s = s0 + lane;
-    m = fmaxf(m, s < n_splits ? p[(size_t)s * PART] : -INFINITY);
+    m = fmaxf(m, s < n_splits ? p[(size_t)s * STEP] : -INFINITY);
   }
   m = wave_max(m);
   for (int s0 = 0; s0 < n_splits; s0 += SYN_WAVE) {
     const int s = s0 + lane;
-    const float ms = s < n_splits ? p[(size_t)s * PART] : -INFINITY;
+    const float ms = s < n_splits ? p[(size_t)s * STEP] : -INFINITY;
     const float w = ms == -INFINITY ? 0.f : __expf(ms - m);  // a split that had no keys weighs nothing
-    l += s < n_splits ? w * p[(size_t)s * PART + 1] : 0.f;
+    l += s < n_splits ? w * p[(size_t)s * STEP + 1] : 0.f;
     const int cnt = min(SYN_WAVE, n_splits - s0);
     for (int j0 = 0; j0 < cnt; j0 += 8) {  // eight splits' values in flight together, added in their order
       constexpr int NI = (HD + SYN_WAVE - 1) / SYN_WAVE;
@@ -1024,7 +1108,7 @@ attn_decode_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ o
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
           const int d = lane + i * SYN_WAVE;
-          vals[u][i] = (j0 + u < cnt && d < HD) ? p[(size_t)(s0 + j0 + u) * PART + 2 + d] : 0.f;
+          vals[u][i] = (j0 + u < cnt && d < HD) ? p[(size_t)(s0 + j0 + u) * STEP + 2 + d] : 0.f;
         }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
@@ -1058,17 +1142,24 @@ static hipError_t raise_decode_lds() {
   });
 }
 
-// workspace: n_seqs * nh * n_splits * (HD + 2) floats (unused with one split)
+// workspace: n_seqs * nh * n_splits * (HD + 2) floats (unused with one split).
+// counters (may be null: then a second kernel merges the splits): n_seqs * kv heads * ceil(group / 16) ints, zero.
+// items (may be null: every sequence in n_splits splits): n_items x {sequence, split, splits of the sequence, first},
+// `first` + split < n_seqs * n_splits being the place of the split's partial results; they need the counters.
 static int launch_decode(const void* q, const QkvIntake* in, void* k_pages, void* v_pages, const int* page_table,
                          int table_stride, const int* seq_len, int n_seqs, void* out, float* workspace, int n_splits,
                          float scale, int window, int nh, int nkv, int hd, hipStream_t stream,
-                         ScoreTerms terms = ScoreTerms{nullptr, 0.f}) {
+                         ScoreTerms terms = ScoreTerms{nullptr, 0.f}, int* counters = nullptr,
+                         const int* items = nullptr, int n_items = 0) {
   SYN_CHECK(terms.softcap >= 0.f, "attention_decode: a soft cap of %g", (double)terms.softcap);
   SYN_CHECK(hd == HD, "attention_decode: library built for head size %d, called with %d", HD, hd);
   SYN_CHECK(n_seqs > 0 && nh > 0 && nkv > 0 && n_splits > 0, "attention_decode: empty input");
   SYN_CHECK(nh % nkv == 0, "attention_decode: %d heads do not divide into %d kv heads", nh, nkv);
   const int chunks = (nh / nkv + 15) / 16;
   SYN_CHECK(nkv * chunks <= 65535 && n_splits <= 65535, "attention_decode: grid too large");
+  SYN_CHECK(items == nullptr || (counters != nullptr && n_items == n_seqs * n_splits),
+            "attention_decode: a list of %d items for %d sequences x %d splits, counters %s", n_items, n_seqs, n_splits,
+            counters ? "given" : "missing");
   // waves a workgroup: as many as the LDS for their states allows (up to 8), but no more than make
   // about 2,048 waves in all: at large batches four waves a workgroup are plenty
   const int cols_alloc = nh / nkv < 16 ? nh / nkv : 16;
@@ -1085,18 +1176,19 @@ static int launch_decode(const void* q, const QkvIntake* in, void* k_pages, void
   SYN_CHECK(lds <= LDS_MAX, "attention_decode: %zu bytes of LDS for %d heads a group", lds, nh / nkv);
   const hipError_t raised = raise_decode_lds();
   SYN_CHECK(raised == hipSuccess, "attention_decode: %zu bytes of LDS refused: %s", LDS_MAX, hipGetErrorString(raised));
-  const dim3 grid(n_seqs, nkv * chunks, n_splits);
+  const dim3 grid = items ? dim3(n_items, nkv * chunks, 1) : dim3(n_seqs, nkv * chunks, n_splits);
+  const DecodeWork work{workspace, counters, (const int4*)items};
   if (in)
     attn_decode_split_kernel<true><<<grid, waves * SYN_WAVE, lds, stream>>>(
-        nullptr, (bf16*)k_pages, (bf16*)v_pages, page_table, table_stride, seq_len, workspace, (bf16*)out, scale,
+        nullptr, (bf16*)k_pages, (bf16*)v_pages, page_table, table_stride, seq_len, work, (bf16*)out, scale,
         window, nh, nkv, n_splits, cols_alloc, *in, terms);
   else
     attn_decode_split_kernel<false><<<grid, waves * SYN_WAVE, lds, stream>>>(
-        (const bf16*)q, (bf16*)k_pages, (bf16*)v_pages, page_table, table_stride, seq_len, workspace, (bf16*)out,
+        (const bf16*)q, (bf16*)k_pages, (bf16*)v_pages, page_table, table_stride, seq_len, work, (bf16*)out,
         scale, window, nh, nkv, n_splits, cols_alloc, QkvIntake{}, terms);
   SYN_LAUNCH_CHECK("attention_decode_split");
-  if (n_splits > 1) {
-    attn_decode_merge_kernel<<<n_seqs * nh, SYN_WAVE, 0, stream>>>(workspace, (bf16*)out, n_splits);
+  if (n_splits > 1 && counters == nullptr) {
+    attn_decode_merge_kernel<<<n_seqs * nh, SYN_WAVE, 0, stream>>>(workspace, (bf16*)out, n_splits, nh);
     SYN_LAUNCH_CHECK("attention_decode_merge");
   }
   return 0;
@@ -1110,14 +1202,16 @@ SYN_EXPORT int syn_attention_decode_bf16(const void* q, const void* k_pages, con
                        workspace, n_splits, scale, window, nh, nkv, hd, stream);
 }
 
-// the same with terms on the scores: slopes [nh] float or null, softcap (0: none), see ScoreTerms
+// the same with terms on the scores (slopes [nh] float or null, softcap (0: none), see ScoreTerms) and with
+// the merge of the splits inside the one launch (counters, items: see launch_decode; both may be null)
 SYN_EXPORT int syn_attention_decode_terms_bf16(const void* q, const void* k_pages, const void* v_pages,
                                                const int* page_table, int table_stride, const int* seq_len, int n_seqs,
                                                void* out, float* workspace, int n_splits, float scale, int window,
                                                int nh, int nkv, int hd, const float* slopes, float softcap,
-                                               hipStream_t stream) {
+                                               int* counters, const int* items, int n_items, hipStream_t stream) {
   return launch_decode(q, nullptr, (void*)k_pages, (void*)v_pages, page_table, table_stride, seq_len, n_seqs, out,
-                       workspace, n_splits, scale, window, nh, nkv, hd, stream, ScoreTerms{slopes, softcap});
+                       workspace, n_splits, scale, window, nh, nkv, hd, stream, ScoreTerms{slopes, softcap}, counters,
+                       items, n_items);
 }
 
 // ---- the same without a workspace argument: see no_alloc.h ----
@@ -1182,7 +1276,8 @@ SYN_EXPORT int syn_attention_decode_fused_bf16(const void* qkv, int n_parts, voi
                                                const void* k_gain, int gain_is_f32, float gain_offset, float eps,
                                                const float* cos_t,
                                                const float* sin_t, int rot, int own_kv, const float* slopes,
-                                               float softcap, hipStream_t stream) {
+                                               float softcap, int* counters, const int* items, int n_items,
+                                               hipStream_t stream) {
   SYN_CHECK(rot % 2 == 0 && rot >= 0 && rot <= hd, "attention_decode_fused: rotary size %d does not fit head size %d",
             rot, hd);
   SYN_CHECK((cos_t == nullptr) == (sin_t == nullptr), "attention_decode_fused: cos and sin come together");
@@ -1194,5 +1289,6 @@ SYN_EXPORT int syn_attention_decode_fused_bf16(const void* qkv, int n_parts, voi
   in.q_gain = q_gain, in.k_gain = k_gain, in.gain_is_f32 = gain_is_f32, in.gain_offset = gain_offset, in.eps = eps;
   in.cos_t = cos_t, in.sin_t = sin_t, in.rot = rot, in.own_kv = own_kv;
   return launch_decode(nullptr, &in, k_pages, v_pages, page_table, table_stride, seq_len, n_seqs, out, workspace,
-                       n_splits, scale, window, nh, nkv, hd, stream, ScoreTerms{slopes, softcap});
+                       n_splits, scale, window, nh, nkv, hd, stream, ScoreTerms{slopes, softcap}, counters, items,
+                       n_items);
 }

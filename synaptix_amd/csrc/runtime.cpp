@@ -14,6 +14,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <queue>
 #include <vector>
 
 #define RT_API extern "C" __attribute__((visibility("default")))
@@ -452,12 +453,66 @@ RT_API int syn_step_fill(void* h, int B, const int* sids, const long* counts, co
   return OK;
 }
 
+// The work list of a decode step's attention over one group of layers: rows * n_splits items
+// {sequence, split, splits of the sequence, first}, where `first` + split is the place of the split's
+// partial result.  Every sequence gets one split; the others go one by one to the sequence whose splits
+// are longest, while a split keeps at least MIN_UNITS units of 32 keys (a window bounds the keys that
+// count); sequences of one length get equal shares.  The items lie sequence by sequence, the longest pieces
+// first, spare items {-1, 0, 0, 0} last.
+RT_API int syn_decode_items(const int* seq_len, int rows, int n_splits, long window, int* items) {
+  if (rows <= 0 || n_splits <= 0) return fail(MISUSE, "a work list for %d rows x %d splits", rows, n_splits);
+  constexpr long UNIT = 32, MIN_UNITS = 8;
+  constexpr int MAX_SPLITS = 64;
+  const long T = (long)rows * n_splits;
+  std::vector<long> units(rows);
+  std::vector<int> splits(rows, 1);
+  for (int i = 0; i < rows; ++i) {
+    long keys = std::max(1, seq_len[i]);
+    if (window > 0) keys = std::min(keys, window);
+    units[i] = (keys + UNIT - 1) / UNIT;
+  }
+  // (units * other splits compared, not quotients: exact, and ties go to the earlier row)
+  auto longer = [&](int a, int b) {
+    const long l = units[a] * splits[b], r = units[b] * splits[a];
+    return l != r ? l < r : a > b;   // priority_queue keeps the greatest on top
+  };
+  auto may_grow = [&](int i) { return splits[i] < MAX_SPLITS && units[i] >= MIN_UNITS * (splits[i] + 1); };
+  std::priority_queue<int, std::vector<int>, decltype(longer)> heap(longer);
+  for (int i = 0; i < rows; ++i)
+    if (may_grow(i)) heap.push(i);
+  for (long left = T - rows; left > 0 && !heap.empty(); --left) {
+    const int i = heap.top();
+    heap.pop();
+    ++splits[i];
+    if (may_grow(i)) heap.push(i);
+  }
+  std::vector<int> order(rows);
+  for (int i = 0; i < rows; ++i) order[i] = i;
+  auto piece = [&](int i) { return (units[i] + splits[i] - 1) / splits[i]; };
+  std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return piece(a) > piece(b); });
+  long at = 0;
+  for (int i : order) {
+    const long first = at;
+    for (int sp = 0; sp < splits[i]; ++sp, ++at) {
+      int* it = items + 4 * at;
+      it[0] = i, it[1] = sp, it[2] = splits[i], it[3] = (int)first;
+    }
+  }
+  for (; at < T; ++at) {
+    int* it = items + 4 * at;
+    it[0] = -1, it[1] = 0, it[2] = 0, it[3] = 0;
+  }
+  return OK;
+}
+
 // A decode step of `rows` rows of which the first B are sequences (one token each) and the rest
 // padding: token 0 at position 0 against a spare page that no sequence owns.  After the integer
-// tables lie 2 * rows floats: temperatures and uniform numbers (0 where none are given).
+// tables lie 2 * rows floats: temperatures and uniform numbers (0 where none are given); after
+// them, for each group with item_splits[g] > 0 (item_splits may be null), the work list of the
+// group's attention: rows * item_splits[g] items of four ints (syn_decode_items).
 RT_API int syn_decode_fill(void* h, int rows, int B, const int* sids, const int* tokens, int n_groups,
                            const int* widths, const int* spare_pages, const float* temps, const float* uniforms,
-                           int* host) {
+                           const int* item_splits, int* host) {
   Cache* c = (Cache*)h;
   if (B > rows) return fail(MISUSE, "%d sequences for a table of %d rows", B, rows);
   const Layout l = make_layout(rows, rows, rows, n_groups, widths);
@@ -489,6 +544,13 @@ RT_API int syn_decode_fill(void* h, int rows, int B, const int* sids, const int*
   for (int i = 0; i < 2 * rows; ++i) f[i] = 0.f;
   if (temps)
     for (int i = 0; i < B; ++i) f[i] = temps[i], f[rows + i] = uniforms[i];
+  int* items = host + l.total + 2 * rows;
+  for (int g = 0; g < n_groups && item_splits; ++g) {
+    if (item_splits[g] <= 0) continue;
+    const int rc = syn_decode_items(host + l.seq_len, rows, item_splits[g], c->windows[g], items);
+    if (rc) return rc;
+    items += 4L * rows * item_splits[g];
+  }
   return OK;
 }
 

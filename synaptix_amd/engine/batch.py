@@ -58,6 +58,16 @@ class ScratchPool:
             self.tensors[name] = t
         return t
 
+    def counters(self, name: str, numel: int) -> torch.Tensor:
+        """int32 counters that are zero when handed out first; their users leave them zero."""
+        t = self.tensors.get(name)
+        if t is None or t.numel() < numel:
+            if self.frozen:
+                raise RuntimeError(f"counters {name!r} of a captured step would have to grow to {numel}")
+            t = torch.zeros(max(numel, 1), dtype=torch.int32, device=self.device)
+            self.tensors[name] = t
+        return t
+
 
 class StepContext:
     """What parts see of a step.  Device arrays are views into one buffer."""
@@ -73,6 +83,7 @@ class StepContext:
         for name, (o, n) in layout.off.items():
             setattr(self, name, buffer[o:o + n])
         self._tables = [buffer[o:o + n].view(layout.B, w) for (o, n), w in zip(layout.table_off, layout.widths)]
+        self.items = None       # a work list of decode attention for each group, where the step's owner keeps them
 
     def page_table(self, group: int) -> torch.Tensor:
         return self._tables[group]
@@ -80,9 +91,17 @@ class StepContext:
     def decode_splits(self, n_kv_heads: int, group: int) -> int:
         return ops.decode_splits(self.n_seqs, n_kv_heads, self.layout.widths[group])
 
+    def decode_items(self, group: int):
+        """The group's work list for decode attention (int32 [n_seqs * decode_splits, 4]) or None."""
+        return None if self.items is None else self.items[group]
+
     def scratch(self, name: str, numel: int) -> torch.Tensor:
         """Float scratch memory that lives as long as its pool's owner; contents are undefined."""
         return self._scratch.get(name, numel)
+
+    def counters(self, name: str, numel: int) -> torch.Tensor:
+        """Zeroed int32 counters that live as long as the pool's owner; whoever counts with them leaves them zero."""
+        return self._scratch.counters(name, numel)
 
 
 def fill_host_buffer(layout: StepLayout, host: np.ndarray, cache, slots, tokens_flat: np.ndarray, counts,

@@ -41,7 +41,14 @@ class DecodeRunner:
         self.engine, self.rows, self.widths = engine, rows, list(widths)
         self.layout = StepLayout(rows, rows, rows, widths)
         n_int = self.layout.total
-        self.total = n_int + 2 * rows                          # + temperatures and uniforms as float bits
+        # the work lists of decode attention, one for each group of layers whose keys are split: longer sequences
+        # get more of the group's rows * splits workgroups (per kv head), refreshed with the step's other tables
+        groups = engine.cache.groups
+        self.item_splits = [ops.decode_splits(rows, g.need.kv_heads, w) if engine.dtype == torch.bfloat16 else 0
+                            for g, w in zip(groups, self.widths)]
+        self.item_splits = [s if s > 1 else 0 for s in self.item_splits]
+        n_items = [rows * s for s in self.item_splits]
+        self.total = n_int + 2 * rows + 4 * sum(n_items)       # + temperatures and uniforms as float bits + items
         dev = engine.device
         self.dev = torch.zeros(self.total, dtype=torch.int32, device=dev)
         self.host = [torch.zeros(self.total, dtype=torch.int32, pin_memory=True) for _ in range(2)]
@@ -49,6 +56,10 @@ class DecodeRunner:
         self.turn = 0
         self.temps = self.dev[n_int:n_int + rows].view(torch.float32)
         self.uniforms = self.dev[n_int + rows:n_int + 2 * rows].view(torch.float32)
+        self.items, at = [], n_int + 2 * rows
+        for n in n_items:
+            self.items.append(self.dev[at:at + 4 * n].view(n, 4) if n else None)
+            at += 4 * n
         self.out_tokens = torch.zeros(rows, dtype=torch.int32, device=dev)
         self.logits = None
         self.graph = None
@@ -67,7 +78,7 @@ class DecodeRunner:
             u = (C.c_float * B)(*[float(x) for x in uniforms])
         rt.check(rt.lib().syn_decode_fill(self.engine.cache._h, self.rows, B, rt.ints([int(s) for s in slots]),
                                           rt.ints([int(x) for x in tokens]), len(self.widths), rt.ints(self.widths),
-                                          rt.ints(self.spare), t, u, host.ctypes.data))
+                                          rt.ints(self.spare), t, u, rt.ints(self.item_splits), host.ctypes.data))
 
     def _forward(self, ctx):
         eng = self.engine
@@ -96,6 +107,7 @@ class DecodeRunner:
             ctx = StepContext(self.layout, self.dev, eng.dtype, [-1] * self.rows, [0] * self.rows, [1] * self.rows,
                               self.scratch)
             ctx.max_position = eng.max_positions - 1 if eng.max_positions else 0   # checked on the host each step
+            ctx.items = self.items
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side), torch.no_grad():

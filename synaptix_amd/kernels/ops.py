@@ -562,10 +562,30 @@ def decode_splits(n_seqs, n_kv_heads, max_pages):
     return int(splits)
 
 
+def _decode_work(name, counters, items, B, n_splits, n_heads, n_kv_heads):
+    """The optional arguments of the decode kernels that put the merge of the splits into the one
+    launch.  counters: int32, at least B * kv heads * ceil(group / 16), zero (the kernel leaves them
+    zero); items: int32 [B * n_splits, 4] rows {sequence, split, splits of the sequence, first}
+    that hand longer sequences more splits (runtime.decode_items lays them out), needs counters."""
+    if counters is None:
+        if items is not None:
+            raise KernelError(f"{name}: a list of items needs counters")
+        return None, None, 0
+    chunks = -(-(n_heads // n_kv_heads) // 16)
+    _need(counters, f"{name}.counters", _I32)
+    if counters.numel() < B * n_kv_heads * chunks:
+        raise KernelError(f"{name}: {counters.numel()} counters for {B} sequences x {n_kv_heads * chunks}")
+    if items is None:
+        return _ptr(counters), None, 0
+    _need(items, f"{name}.items", _I32, (B * n_splits, 4))
+    return _ptr(counters), _ptr(items), B * n_splits
+
+
 def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
-                          n_heads, n_kv_heads, head_dim, slopes=None, softcap=0.0):
+                          n_heads, n_kv_heads, head_dim, slopes=None, softcap=0.0, counters=None, items=None):
     """One query for each sequence (its last token, already in the cache); seq_len [B] counts it.
-    workspace: float [B * nh * n_splits * (hd + 2)].  slopes, softcap: see _score_terms."""
+    workspace: float [B * nh * n_splits * (hd + 2)].  slopes, softcap: see _score_terms; counters,
+    items: see _decode_work."""
     nh, nkv, hd = n_heads, n_kv_heads, head_dim
     _need(q, "attention_decode.q", _BF16, (None, nh * hd))
     B = q.shape[0]
@@ -578,24 +598,25 @@ def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspa
     _need(workspace, "attention_decode.workspace", _F32)
     if workspace.numel() < B * nh * n_splits * (hd + 2):
         raise KernelError(f"attention_decode: workspace of {workspace.numel()} floats is too small")
-    if slopes is None and not softcap:
+    if slopes is None and not softcap and counters is None:
         _call(_attn_lib(hd), "syn_attention_decode_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
               page_table.shape[1], _ptr(seq_len), B, _ptr(out), _ptr(workspace), int(n_splits), ctypes.c_float(scale),
               int(window or 0), nh, nkv, hd, _stream())
         return
     _call(_attn_lib(hd), "syn_attention_decode_terms_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
           page_table.shape[1], _ptr(seq_len), B, _ptr(out), _ptr(workspace), int(n_splits), ctypes.c_float(scale),
-          int(window or 0), nh, nkv, hd, *_score_terms("attention_decode", slopes, softcap, nh), _stream())
+          int(window or 0), nh, nkv, hd, *_score_terms("attention_decode", slopes, softcap, nh),
+          *_decode_work("attention_decode", counters, items, B, n_splits, nh, nkv), _stream())
 
 
 def attention_decode_fused_bf16(qkv, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
                                 n_heads, n_kv_heads, head_dim, q_gain, k_gain, eps, cos, sin, write_kv=True,
-                                gain_offset=0.0, slopes=None, softcap=0.0):
+                                gain_offset=0.0, slopes=None, softcap=0.0, counters=None, items=None):
     """attention_decode_bf16 for one new token a sequence whose q, k and v come straight from the
     fused projection: qkv [B, (nh + 2 nkv) * hd] in bf16, or float partial sums [S, B, ...] that are
     added first.  The q/k RMSNorm (if gains are given), the rotation at position seq_len - 1 (if
     tables are given) and, with write_kv, the write of the new k and v into the cache pages happen
-    inside the attention kernel; seq_len [B] counts the new token."""
+    inside the attention kernel; seq_len [B] counts the new token.  counters, items: see _decode_work."""
     nh, nkv, hd = n_heads, n_kv_heads, head_dim
     width = (nh + 2 * nkv) * hd
     n_parts = 0
@@ -633,7 +654,8 @@ def attention_decode_fused_bf16(qkv, k_pages, v_pages, page_table, seq_len, out,
           _ptr(page_table), page_table.shape[1], _ptr(seq_len), B, _ptr(out), _ptr(workspace), int(n_splits),
           ctypes.c_float(scale), int(window or 0), nh, nkv, hd, _ptr(q_gain), _ptr(k_gain), gain_f32,
           ctypes.c_float(gain_offset), ctypes.c_float(eps), _ptr(cos), _ptr(sin), rot, 1 if write_kv else 0,
-          *_score_terms("attention_decode_fused", slopes, softcap, nh), _stream())
+          *_score_terms("attention_decode_fused", slopes, softcap, nh),
+          *_decode_work("attention_decode_fused", counters, items, B, n_splits, nh, nkv), _stream())
 
 
 # ----------------------------------------------------------------------------- sampling

@@ -40,7 +40,8 @@ _SIGNATURES = {
     "syn_cache_check": (_I, [_P]),
     "syn_step_layout": (_L, [_L, _L, _L, _I, _IP, _LP]),
     "syn_step_fill": (_I, [_P, _I, _IP, _LP, _P, _L, _P, _I, _IP, _P]),
-    "syn_decode_fill": (_I, [_P, _I, _I, _IP, _IP, _I, _IP, _IP, _FP, _FP, _P]),
+    "syn_decode_fill": (_I, [_P, _I, _I, _IP, _IP, _I, _IP, _IP, _FP, _FP, _IP, _P]),
+    "syn_decode_items": (_I, [_IP, _I, _I, _L, _IP]),
     "syn_philox_block": (None, [_UP, _UP, _UP]),
     "syn_philox_new": (_P, [C.c_uint64]),
     "syn_philox_delete": (None, [_P]),
@@ -82,3 +83,14 @@ def ints(values):
 
 def longs(values):
     return (C.c_long * len(values))(*values)
+
+
+def decode_items(seq_len, n_splits: int, window=None) -> list:
+    """The work list of a decode step's attention as the runtime lays it out: for sequences of the
+    lengths `seq_len`, len(seq_len) * n_splits items (sequence, split, splits of the sequence, first);
+    spare items have sequence -1."""
+    rows = len(seq_len)
+    out = (C.c_int * (4 * rows * n_splits))()
+    check(lib().syn_decode_items(ints([int(x) for x in seq_len]), rows, int(n_splits),
+                                 -1 if window is None else int(window), out))
+    return [tuple(out[4 * i:4 * i + 4]) for i in range(rows * n_splits)]

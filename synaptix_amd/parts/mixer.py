@@ -101,6 +101,20 @@ class GqaAttention(Mixer):
             self._slopes[key] = None if sl is None else sl.to(device=device, dtype=torch.float32).contiguous()
         return dict(slopes=self._slopes[key], softcap=self.score_softcap)
 
+    def _decode_work(self, ctx, cache, n_seqs):
+        """For single tokens: the workspace of the splits' partial results, the number of splits, and
+        what merges them inside the attention kernel (counters, and the step's work list if it keeps one)."""
+        splits = ctx.decode_splits(self.nkv, cache.group)
+        work = ctx.scratch("attention_decode", n_seqs * self.nh * splits * (self.hd + 2))
+        merge = {}
+        if splits > 1:
+            chunks = -(-(self.nh // self.nkv) // 16)
+            items = ctx.decode_items(cache.group)
+            if items is not None and items.shape[0] != n_seqs * splits:
+                items = None
+            merge = dict(counters=ctx.counters("attention_decode_arrivals", n_seqs * self.nkv * chunks), items=items)
+        return work, splits, merge
+
     def forward(self, h, ctx, cache, owner=True):
         nh, nkv, hd = self.nh, self.nkv, self.hd
         N, act = h.shape[0], h.dtype
@@ -125,12 +139,11 @@ class GqaAttention(Mixer):
         window = self.window or 0
         if act == torch.bfloat16 and ctx.one_token_each:
             # single tokens: the attention kernel takes q, k and v from the projection itself
-            splits = ctx.decode_splits(nkv, cache.group)
-            work = ctx.scratch("attention_decode", N * nh * splits * (hd + 2))
+            work, splits, merge = self._decode_work(ctx, cache, N)
             ops.attention_decode_fused_bf16(qkv, cache.k_pages, cache.v_pages, table, ctx.seq_len, o, work, splits,
                                             self.scale, window, nh, nkv, hd, self.q_gain, self.k_gain,
                                             self.qk_norm_eps or 0.0, cos, sin, write_kv=owner,
-                                            gain_offset=self.qk_gain_offset, **terms)
+                                            gain_offset=self.qk_gain_offset, **terms, **merge)
             return deferred_product(o, self.w_o, self.p_o)
         q = torch.empty((N, nh * hd), dtype=act, device=h.device)
         ops.qk_norm_rope_kv_write(qkv, q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos,
@@ -140,10 +153,9 @@ class GqaAttention(Mixer):
             ops.attention_f32(q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos, o, self.scale, window,
                               nh, nkv, hd, **terms)
         elif ctx.one_token_each:
-            splits = ctx.decode_splits(nkv, cache.group)
-            work = ctx.scratch("attention_decode", N * nh * splits * (hd + 2))
+            work, splits, merge = self._decode_work(ctx, cache, N)
             ops.attention_decode_bf16(q, cache.k_pages, cache.v_pages, table, ctx.seq_len, o, work, splits,
-                                      self.scale, window, nh, nkv, hd, **terms)
+                                      self.scale, window, nh, nkv, hd, **terms, **merge)
         else:
             ops.attention_prefill_bf16(q, cache.k_pages, cache.v_pages, table, ctx.seq_start, ctx.seq_past, o,
                                        self.scale, window, nh, nkv, hd, **terms)

@@ -195,7 +195,7 @@ def decode_splits(n_seqs, n_kv_heads, max_pages):
 
 
 def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
-                          n_heads, n_kv_heads, head_dim, slopes=None, softcap=0.0):
+                          n_heads, n_kv_heads, head_dim, slopes=None, softcap=0.0, counters=None, items=None):
     B = q.shape[0]
     qf = q.to(F32).view(B, n_heads, head_dim)
     for b in range(B):
@@ -206,7 +206,7 @@ def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspa
 
 def attention_decode_fused_bf16(qkv, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
                                 n_heads, n_kv_heads, head_dim, q_gain, k_gain, eps, cos, sin, write_kv=True,
-                                gain_offset=0.0, slopes=None, softcap=0.0):
+                                gain_offset=0.0, slopes=None, softcap=0.0, counters=None, items=None):
     B = qkv.shape[-2]
     q = torch.empty((B, n_heads * head_dim), dtype=torch.bfloat16)
     tok_seq = torch.arange(B, dtype=torch.int32)

@@ -8,6 +8,7 @@ import pytest
 import torch
 
 import cpu_kernels as ref
+from synaptix_amd.kernels import runtime as rt
 
 pytestmark = pytest.mark.gpu
 
@@ -664,6 +665,31 @@ def test_attention_with_terms_on_the_scores(ops, nh, nkv, hd, past, new, window,
             close(outd, want[last], 2e-2, 1e-2, what=f"attention decode bf16 with terms, {splits} splits")
 
 
+def merged_in_kernel(run, two_kernels, want, lens, splits, window, nh, nkv):
+    """The same call with the merge of the splits inside the one launch, by the workgroup that finishes last:
+    first with every sequence in `splits` splits, then with the host's work list, which gives long sequences
+    more of them; twice each with the same counters, which the kernel has to leave at zero."""
+    if splits == 1:
+        return
+    chunks = -(-(nh // nkv) // 16)
+    counters = torch.zeros(len(lens) * nkv * chunks, dtype=I32, device=DEV)
+    items = torch.tensor(rt.decode_items(lens, splits, window or None), dtype=I32, device=DEV)
+    for what, kw in (("merged in the kernel", dict(counters=counters)),
+                     ("with a work list", dict(counters=counters, items=items))):
+        outs = []
+        for _ in range(2):
+            got = torch.full_like(two_kernels, float("nan"))
+            run(got, **kw)
+            close(got, want, 2e-2, 1e-2, what=f"decode attention {what}")
+            outs.append(got.cpu())
+            assert int(counters.abs().sum()) == 0, f"{what}: counters are not back at zero"
+        assert torch.equal(outs[0], outs[1]), f"{what}: two runs differ"
+    # the same splits merged by either way: the same sums in another order
+    got = torch.empty_like(two_kernels)
+    run(got, counters=counters)
+    close(got, two_kernels.float().cpu(), 1e-2, 1e-2, what="merge in the kernel against the merge kernel")
+
+
 @pytest.mark.parametrize("nh,nkv,hd,lens,window,splits", [
     (8, 2, 64, [600, 3], 0, 4),                 # crates/synaptix-kernels-cuda/tests/cuda_flash_decode.rs:101 GQA, Tkv=600
     (4, 4, 128, [40], 0, 8),                    # more splits than pages (empty splits), ibid. 130-183
@@ -699,6 +725,9 @@ def test_attention_decode_bf16(ops, nh, nkv, hd, lens, window, splits):
     ops.attention_decode_bf16(d(q), d(k), dv(v), d(table), d(torch.tensor(lens, dtype=I32)), out, work, splits, scale,
                               window, nh, nkv, hd)
     close(out, want, 2e-2, 1e-2, what="attention decode bf16")
+    merged_in_kernel(lambda out2, **kw: ops.attention_decode_bf16(
+        d(q), d(k), dv(v), d(table), d(torch.tensor(lens, dtype=I32)), out2, work, splits, scale, window, nh, nkv, hd, **kw),
+        out, want, lens, splits, window, nh, nkv)
 
 
 @pytest.mark.parametrize("nh,nkv,hd,rot,norm,lens,window,splits,parts,own", [
@@ -748,6 +777,9 @@ def test_attention_decode_with_qkv_intake(ops, nh, nkv, hd, rot, norm, lens, win
     ops.attention_decode_fused_bf16(d(qkv), kd, vd, d(table), d(seq_len), out, work, splits, scale, window, nh, nkv, hd,
                                     d(qg), d(kg), 1e-5, d(cos), d(sin), write_kv=own)
     close(out, want, 2e-2, 1e-2, what="decode attention with q/k/v intake")
+    merged_in_kernel(lambda out2, **kw: ops.attention_decode_fused_bf16(
+        d(qkv), kd, vd, d(table), d(seq_len), out2, work, splits, scale, window, nh, nkv, hd, d(qg), d(kg), 1e-5, d(cos),
+        d(sin), write_kv=own, **kw), out, want, lens, splits, window, nh, nkv)
     # the cache afterwards: the new rows written (or nothing touched)
     close(kd, k_ref.float(), 2e-2, 1e-2, what="k pages after the step")
     close(hv(vd), v_ref.float(), 2e-2, 1e-2, what="v pages after the step")

@@ -60,10 +60,11 @@ def test_decode_tables_pad_with_a_spare_page():
     c.reserve(a, 1), c.reserve(b, 1)
     rows, widths, spare = 4, [4, 4], [12, 12]
     lay = StepLayout(rows, rows, rows, widths)
-    host = np.zeros(lay.total + 2 * rows, dtype=np.int32)
+    item_splits = [0, 3]                       # the second group keeps a work list for its attention: 4 x 3 items
+    host = np.zeros(lay.total + 2 * rows + 4 * rows * 3, dtype=np.int32)
     temps, unis = (C.c_float * 2)(0.5, 0.0), (C.c_float * 2)(0.25, 0.75)
     rt.check(rt.lib().syn_decode_fill(c._h, rows, 2, rt.ints([a, b]), rt.ints([9, 8]), 2, rt.ints(widths),
-                                      rt.ints(spare), temps, unis, host.ctypes.data))
+                                      rt.ints(spare), temps, unis, rt.ints(item_splits), host.ctypes.data))
 
     def arr(name):
         o, n = lay.off[name]
@@ -77,14 +78,17 @@ def test_decode_tables_pad_with_a_spare_page():
     own = c.page_table(0, [a, b], width=4)
     assert full[0, :3].tolist() == own[0, :3].tolist() and full[1, 0] == own[1, 0]
     assert full[0, 3] == 12 and full[1, 1:].tolist() == [12, 12, 12] and (full[2:] == 12).all()
-    f = host[lay.total:].view(np.float32)
+    f = host[lay.total:lay.total + 2 * rows].view(np.float32)
     assert f.tolist() == [0.5, 0.0, 0.0, 0.0, 0.25, 0.75, 0.0, 0.0]
+    items = host[lay.total + 2 * rows:].reshape(12, 4).tolist()
+    assert [tuple(i) for i in items] == rt.decode_items([131, 6, 1, 1], 3)      # from the lengths that the step has
+    assert sorted(i[0] for i in items[:4]) == [0, 1, 2, 3] and all(i[0] == -1 for i in items[4:])   # too short to split
     with pytest.raises(CacheError, match="width"):
         rt.check(rt.lib().syn_decode_fill(c._h, rows, 2, rt.ints([a, b]), rt.ints([9, 8]), 2, rt.ints([2, 4]),
-                                          rt.ints(spare), None, None, host.ctypes.data))
+                                          rt.ints(spare), None, None, None, host.ctypes.data))
     with pytest.raises(CacheError, match="rows"):
         rt.check(rt.lib().syn_decode_fill(c._h, 1, 2, rt.ints([a, b]), rt.ints([9, 8]), 2, rt.ints(widths),
-                                          rt.ints(spare), None, None, host.ctypes.data))
+                                          rt.ints(spare), None, None, None, host.ctypes.data))
 
 
 def test_host_side_rules_of_the_kernels_stay_within_their_kernels_limits():
