@@ -608,8 +608,9 @@ constexpr int PART = HD + 2;
 
 // How the keys of a step's sequences are handed to workgroups.  Without `items` every sequence is cut
 // into the same n_splits (grid.x sequences, grid.z splits).  With `items` the grid's x counts items
-// {sequence, split, splits of the sequence, first} that the host has laid out, more splits for longer
-// sequences, the longest pieces first; an item with sequence -1 is spare and its workgroups leave at once.
+// {sequence, split | splits of the sequence << 16, first, the sequence's length} that the host has laid out,
+// more splits for longer sequences, the longest pieces first; an item with sequence -1 is spare and its
+// workgroups leave at once.
 // counters: one int for each (sequence, grid.y), zero before the launch and zero again after it.
 struct DecodeWork {
   float* partial;
@@ -808,21 +809,22 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
   constexpr int SO_LD = HD + 4;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / SYN_WAVE), lane = threadIdx.x % SYN_WAVE;
   char* stage = (char*)dec_lds + (size_t)wave * STAGE_BYTES;
-  int seq = blockIdx.x, split = blockIdx.z, n_splits = n_splits_all, first = blockIdx.x * n_splits_all;
+  int seq = blockIdx.x, split = blockIdx.z, n_splits = n_splits_all, first = blockIdx.x * n_splits_all, item_len = -1;
   if (work.items) {
     const int4 item = work.items[blockIdx.x];
-    seq = __builtin_amdgcn_readfirstlane(item.x), split = __builtin_amdgcn_readfirstlane(item.y);
-    n_splits = __builtin_amdgcn_readfirstlane(item.z), first = __builtin_amdgcn_readfirstlane(item.w);
+    seq = __builtin_amdgcn_readfirstlane(item.x), first = __builtin_amdgcn_readfirstlane(item.z);
+    split = __builtin_amdgcn_readfirstlane(item.y) & 0xFFFF, n_splits = __builtin_amdgcn_readfirstlane(item.y) >> 16;
+    item_len = __builtin_amdgcn_readfirstlane(item.w);   // (with the item: one trip to memory less than through seq_len)
     // (a spare item, or one that does not fit the launch: nothing is read or written for it)
     const int n_seqs = gridDim.x / n_splits_all;
-    if (seq < 0 || seq >= n_seqs || n_splits < 1 || split < 0 || split >= n_splits || first < 0 ||
-        first + n_splits > (int)gridDim.x)
+    if (seq < 0 || seq >= n_seqs || n_splits < 1 || split >= n_splits || first < 0 || first + n_splits > (int)gridDim.x ||
+        item_len < 1)
       return;
   }
   float* const partial = work.partial;
   const int g = nh / nkv, chunks = (g + 15) / 16;
   const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
-  const int kv_len = seq_len[seq], pos = kv_len - 1;
+  const int kv_len = item_len > 0 ? item_len : seq_len[seq], pos = kv_len - 1;
   const int col = lane % 16;
   const int hg = chunk * 16 + col;  // head inside the group
   const bool valid = hg < g;
@@ -1144,8 +1146,9 @@ static hipError_t raise_decode_lds() {
 
 // workspace: n_seqs * nh * n_splits * (HD + 2) floats (unused with one split).
 // counters (may be null: then a second kernel merges the splits): n_seqs * kv heads * ceil(group / 16) ints, zero.
-// items (may be null: every sequence in n_splits splits): n_items x {sequence, split, splits of the sequence, first},
-// `first` + split < n_seqs * n_splits being the place of the split's partial results; they need the counters.
+// items (may be null: every sequence in n_splits splits): n_items x {sequence, split | splits of the sequence << 16,
+// first, length}, `first` + split < n_seqs * n_splits being the place of the split's partial results and length
+// what seq_len holds for the sequence; they need the counters.
 static int launch_decode(const void* q, const QkvIntake* in, void* k_pages, void* v_pages, const int* page_table,
                          int table_stride, const int* seq_len, int n_seqs, void* out, float* workspace, int n_splits,
                          float scale, int window, int nh, int nkv, int hd, hipStream_t stream,

@@ -454,8 +454,8 @@ RT_API int syn_step_fill(void* h, int B, const int* sids, const long* counts, co
 }
 
 // The work list of a decode step's attention over one group of layers: rows * n_splits items
-// {sequence, split, splits of the sequence, first}, where `first` + split is the place of the split's
-// partial result.  Every sequence gets one split; the others go one by one to the sequence whose splits
+// {sequence, split | splits of the sequence << 16, first, the sequence's length}, where `first` + split is
+// the place of the split's partial result.  Every sequence gets one split; the others go one by one to the sequence whose splits
 // are longest, while a split keeps at least MIN_UNITS units of 32 keys (a window bounds the keys that
 // count); sequences of one length get equal shares.  The items lie sequence by sequence, the longest pieces
 // first, spare items {-1, 0, 0, 0} last.
@@ -495,7 +495,7 @@ RT_API int syn_decode_items(const int* seq_len, int rows, int n_splits, long win
     const long first = at;
     for (int sp = 0; sp < splits[i]; ++sp, ++at) {
       int* it = items + 4 * at;
-      it[0] = i, it[1] = sp, it[2] = splits[i], it[3] = (int)first;
+      it[0] = i, it[1] = sp | (splits[i] << 16), it[2] = (int)first, it[3] = seq_len[i];
     }
   }
   for (; at < T; ++at) {

@@ -565,8 +565,8 @@ def decode_splits(n_seqs, n_kv_heads, max_pages):
 def _decode_work(name, counters, items, B, n_splits, n_heads, n_kv_heads):
     """The optional arguments of the decode kernels that put the merge of the splits into the one
     launch.  counters: int32, at least B * kv heads * ceil(group / 16), zero (the kernel leaves them
-    zero); items: int32 [B * n_splits, 4] rows {sequence, split, splits of the sequence, first}
-    that hand longer sequences more splits (runtime.decode_items lays them out), needs counters."""
+    zero); items: int32 [B * n_splits, 4], the work list that hands longer sequences more splits
+    (runtime.decode_items lays it out), needs counters."""
     if counters is None:
         if items is not None:
             raise KernelError(f"{name}: a list of items needs counters")

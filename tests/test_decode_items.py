@@ -9,6 +9,15 @@ from synaptix_amd.kernels import runtime as rt
 UNIT, MIN_UNITS = 32, 8
 
 
+def _unpacked(lengths, n_splits, window=None):
+    """(sequence, split, splits of the sequence, first) of every item; the length that an item carries is checked here."""
+    out = []
+    for seq, split_and_n, first, length in rt.decode_items(lengths, n_splits, window):
+        assert seq < 0 or length == lengths[seq]
+        out.append((seq, split_and_n & 0xFFFF, split_and_n >> 16, first))
+    return out
+
+
 def _by_sequence(items):
     seqs = {}
     for at, (seq, split, n, first) in enumerate(items):
@@ -19,7 +28,7 @@ def _by_sequence(items):
 
 
 def _check(lengths, n_splits, window=None):
-    items = rt.decode_items(lengths, n_splits, window)
+    items = _unpacked(lengths, n_splits, window)
     assert len(items) == len(lengths) * n_splits
     seqs = _by_sequence(items)
     assert sorted(seqs) == list(range(len(lengths)))          # every sequence is there

@@ -83,6 +83,7 @@ def test_decode_tables_pad_with_a_spare_page():
     items = host[lay.total + 2 * rows:].reshape(12, 4).tolist()
     assert [tuple(i) for i in items] == rt.decode_items([131, 6, 1, 1], 3)      # from the lengths that the step has
     assert sorted(i[0] for i in items[:4]) == [0, 1, 2, 3] and all(i[0] == -1 for i in items[4:])   # too short to split
+    assert all(i[1] == 1 << 16 for i in items[:4]) and sorted(i[3] for i in items[:4]) == [1, 1, 6, 131]
     with pytest.raises(CacheError, match="width"):
         rt.check(rt.lib().syn_decode_fill(c._h, rows, 2, rt.ints([a, b]), rt.ints([9, 8]), 2, rt.ints([2, 4]),
                                           rt.ints(spare), None, None, None, host.ctypes.data))
