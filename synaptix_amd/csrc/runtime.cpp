@@ -453,6 +453,57 @@ RT_API int syn_step_fill(void* h, int B, const int* sids, const long* counts, co
   return OK;
 }
 
+// The same for a step that is replayed from a captured graph and therefore has fixed counts: N_pad tokens,
+// B_pad sequences, want_pad wanted rows.  The step's own B sequences and N tokens come first; the tokens up
+// to N_pad are padding (token 0 at positions 0, 1, ... of sequence B, which owns no slot and whose table
+// row names only a spare page that no sequence owns); sequences beyond it are empty; wanted rows beyond the
+// step's own name row 0.  B < B_pad unless N == N_pad; a table row of widths[g] pages must hold N_pad - N tokens.
+RT_API int syn_step_fill_padded(void* h, int B, const int* sids, const long* counts, const int* tokens, long n_want,
+                                const int* want_rows, int n_groups, const int* widths, const int* spare_pages,
+                                long N_pad, int B_pad, long want_pad, int* host) {
+  Cache* c = (Cache*)h;
+  long N = 0;
+  for (int i = 0; i < B; ++i) N += counts[i];
+  if (N > N_pad || B > B_pad || n_want > want_pad || (N < N_pad && B == B_pad))
+    return fail(MISUSE, "a step of %ld tokens, %d sequences, %ld wanted rows for a table of %ld, %d, %ld", N, B, n_want,
+                N_pad, B_pad, want_pad);
+  for (int g = 0; g < n_groups; ++g)
+    if ((N_pad - N + PAGE_TOKENS - 1) / PAGE_TOKENS > widths[g])
+      return fail(MISUSE, "page table width %d of group %d is less than the %ld padding tokens need", widths[g], g, N_pad - N);
+  const Layout l = make_layout(N_pad, B_pad, want_pad, n_groups, widths);
+  long pos = 0;
+  for (int i = 0; i < B_pad; ++i) {
+    long past = 0, n = 0;
+    int sid = -1;
+    if (i < B) {
+      Slot* s = c->live_slot(sids[i]);
+      if (!s) return MISUSE;
+      past = s->length, n = counts[i], sid = sids[i];
+    } else if (i == B) {
+      n = N_pad - N;
+    }
+    host[l.seq_start + i] = (int)pos;
+    host[l.seq_past + i] = (int)past;
+    host[l.seq_len + i] = (int)(past + n);
+    host[l.seq_slot + i] = sid;
+    for (long t = 0; t < n; ++t) {
+      host[l.tokens + pos + t] = i < B ? tokens[pos + t] : 0;
+      host[l.tok_seq + pos + t] = i;
+      host[l.tok_pos + pos + t] = (int)(past + t);
+    }
+    pos += n;
+  }
+  host[l.seq_start + B_pad] = (int)pos;
+  for (long i = 0; i < want_pad; ++i) host[l.want + i] = i < n_want ? want_rows[i] : 0;
+  for (int g = 0; g < n_groups; ++g) {
+    int* tab = host + l.tables[g];
+    const int rc = fill_table(c, g, sids, B, widths[g], spare_pages[g], tab);
+    if (rc) return rc;
+    for (long j = (long)B * widths[g]; j < (long)B_pad * widths[g]; ++j) tab[j] = spare_pages[g];
+  }
+  return OK;
+}
+
 // The work list of a decode step's attention over one group of layers: rows * n_splits items
 // {sequence, split | splits of the sequence << 16, first, the sequence's length}, where `first` + split is
 // the place of the split's partial result.  Every sequence gets one split; the others go one by one to the sequence whose splits

@@ -63,6 +63,7 @@ class Engine:
         # same values again may be captured, which a mixer with a running state is not
         self.has_states = any(isinstance(n, StateNeed) for n in model.cache_needs())
         self.graph_ok = not self.has_states
+        self.prompt_graphs = True        # short prompt steps are replayed from graphs (see _prompt_runner)
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -124,8 +125,8 @@ class Engine:
             self._copied[i].synchronize()
         return i, self._host[i], self._dev[i]
 
-    def prepare(self, entries, want) -> tuple:
-        """Check a step, hold its pages, and write its arrays to the device.  Returns (ctx, n_want)."""
+    def _checked(self, entries, want) -> tuple:
+        """A step's entries and wanted places, checked: (slots, token arrays, tokens cached before, counts, wanted rows)."""
         if not entries:
             raise StepError("a step needs at least one sequence")
         slots = [e[0] for e in entries]
@@ -159,12 +160,19 @@ class Engine:
                         raise StepError(f"slot {slots[i]}: wanted place {p} is outside its {token_lists[i].size} tokens")
                     want_rows.append(int(starts[i]) + int(p))
         counts = [int(t.size) for t in token_lists]
+        return slots, token_lists, past, counts, want_rows
+
+    def prepare(self, entries, want) -> tuple:
+        """Check a step, hold its pages, and write its arrays to the device.  Returns (ctx, n_want)."""
+        slots, token_lists, past, counts, want_rows = self._checked(entries, want)
         self.cache.reserve_step(slots, counts)            # all pages of the step, or none
+        return self._context(slots, token_lists, past, counts, want_rows), len(want_rows)
+
+    def _context(self, slots, token_lists, past, counts, want_rows):
         widths = [self.cache.table_width(gi, slots) for gi in range(len(self.cache.groups))]
-        layout = StepLayout(int(starts[-1]), len(entries), len(want_rows), widths)
+        layout = StepLayout(sum(counts), len(slots), len(want_rows), widths)
         dev = self._upload(layout, slots, np.concatenate(token_lists), counts, want_rows)
-        ctx = StepContext(layout, dev, self.dtype, slots, past, counts, self._scratch)
-        return ctx, len(want_rows)
+        return StepContext(layout, dev, self.dtype, slots, past, counts, self._scratch)
 
     def _upload(self, layout, slots, tokens_flat, counts, want_rows) -> torch.Tensor:
         """The step's arrays on the device, through a pinned buffer and one asynchronous copy."""
@@ -179,14 +187,45 @@ class Engine:
         """entries: [(slot, tokens), ...]; want: "last", "all", None or a list of places for each
         entry.  Returns float logits [wanted, vocab] on the device, in the order of the entries and
         of their places."""
-        ctx, n_want = self.prepare(entries, want)
-        with torch.no_grad():
-            logits = self.model.forward(ctx, ctx.tokens, ctx.want if n_want else None, self.cache)
-        for s, n in zip(ctx.slots, ctx.new_counts):
+        slots, token_lists, past, counts, want_rows = self._checked(entries, want)
+        self.cache.reserve_step(slots, counts)            # all pages of the step, or none
+        runner = self._prompt_runner(slots, counts, want_rows)
+        if runner is not None:
+            logits = runner.step(slots, token_lists, counts, want_rows)
+        else:
+            ctx = self._context(slots, token_lists, past, counts, want_rows)
+            with torch.no_grad():
+                logits = self.model.forward(ctx, ctx.tokens, ctx.want if want_rows else None, self.cache)
+        for s, n in zip(slots, counts):
             self.cache.commit(s, n)
         if logits is None:
             logits = torch.empty((0, self.vocab), dtype=torch.float32, device=self.device)
         return logits
+
+    def _prompt_runner(self, slots, counts, want_rows):
+        """The captured step for a short prompt step with one wanted row a sequence, or None: launched one by
+        one, the kernels of a few dozen tokens take the host longer than the GPU."""
+        if not (self.prompt_graphs and self.graph_ok and self.dtype == torch.bfloat16) or ops.timing_active():
+            return None
+        if len(want_rows) != len(slots) or all(c == 1 for c in counts):
+            return None
+        starts = np.concatenate([[0], np.cumsum(counts)])
+        if any(not (starts[i] <= r < starts[i + 1]) for i, r in enumerate(want_rows)):
+            return None
+        from .graph import PromptRunner, prompt_bucket
+        bucket = prompt_bucket(int(starts[-1]), len(slots))
+        if bucket is None or (self.max_positions is not None and self.max_positions < bucket[0]):
+            return None
+        widths = []
+        for gi in range(len(self.cache.groups)):
+            width = 1                                  # few distinct widths, so that graphs are shared; the
+            while width < max(self.cache.table_width(gi, slots), pages_for(bucket[0])):   # padding tokens fit a row
+                width *= 2
+            widths.append(width)
+        key = ("prompt",) + bucket + tuple(widths)
+        if key not in self._runners:
+            self._runners[key] = PromptRunner(self, bucket[0], bucket[1], widths)
+        return self._runners[key]
 
     def decode_runner(self, n_seqs: int, max_len: int):
         """The captured decode step for up to n_seqs sequences of at most max_len tokens."""

@@ -40,6 +40,7 @@ _SIGNATURES = {
     "syn_cache_check": (_I, [_P]),
     "syn_step_layout": (_L, [_L, _L, _L, _I, _IP, _LP]),
     "syn_step_fill": (_I, [_P, _I, _IP, _LP, _P, _L, _P, _I, _IP, _P]),
+    "syn_step_fill_padded": (_I, [_P, _I, _IP, _LP, _P, _L, _P, _I, _IP, _IP, _L, _I, _L, _P]),
     "syn_decode_fill": (_I, [_P, _I, _I, _IP, _IP, _I, _IP, _IP, _FP, _FP, _IP, _P]),
     "syn_decode_items": (_I, [_IP, _I, _I, _L, _IP]),
     "syn_philox_block": (None, [_UP, _UP, _UP]),

@@ -272,6 +272,64 @@ def test_graph_replays_equal_eager_steps(dtype):
         e.cache.check()
 
 
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_captured_prompt_steps_equal_eager_ones(name):
+    """Short prompt steps are replayed from graphs with padding rows behind their own: every replay against
+    the eager step of an engine that has the graphs switched off and against the plain implementation;
+    several steps through one graph with eager work between them, sequences that go on with a second piece
+    of their prompt, a wanted place that is not the last, a slot that is used again, and decode steps after."""
+    dtype = "bfloat16"
+    V = CONFIGS[name]["vocab_size"]
+    eager, graph = make_engine(name, dtype, 4096), make_engine(name, dtype, 4096)
+    eager.prompt_graphs = False
+
+    def both(entries_of, want):
+        got = graph.step(entries_of(graph), want=want)
+        ref = eager.step(entries_of(eager), want=want)
+        torch.cuda.synchronize()
+        assert got.shape == ref.shape
+        err = float((got - ref).abs().max())
+        assert err <= 3e-2 * max(1.0, float(ref.abs().max())), f"replayed prompt step differs from the eager one by {err}"
+        return got
+
+    slots = {id(e): [] for e in (eager, graph)}
+
+    def acquire(n):
+        for e in (eager, graph):
+            slots[id(e)] += [e.acquire() for _ in range(n)]
+
+    acquire(3)
+    prompts = [random_tokens(V, n, 900 + n) for n in (5, 33, 20)]
+    got = both(lambda e: list(zip(slots[id(e)][:3], prompts)), "last")              # 58 tokens: the graph of 64 rows, 4 + 1 sequences
+    assert any(k[0] == "prompt" and k[1] == 64 and k[2] == 5 for k in graph._runners if isinstance(k[0], str))
+    for i, p in enumerate(prompts):
+        assert_logits_close(got[i:i + 1], plain_logits(name, p)[-1:], dtype, f"captured prompt step, sequence {i}")
+    # the same graph again with other lengths, and a wanted place in the middle of the first sequence
+    acquire(2)
+    more = [random_tokens(V, n, 950 + n) for n in (40, 9)]
+    got = both(lambda e: list(zip(slots[id(e)][3:5], more)), [[17], [8]])
+    assert_logits_close(got[0:1], plain_logits(name, more[0])[17:18], dtype, "a wanted place that is not the last")
+    # second pieces of two prompts (tokens cached before), beside a fresh one-token sequence
+    acquire(1)
+    tails = [random_tokens(V, n, 970 + n) for n in (30, 12)]
+    got = both(lambda e: [(slots[id(e)][0], tails[0]), (slots[id(e)][3], tails[1]), (slots[id(e)][5], [7])], "last")
+    assert_logits_close(got[0:1], plain_logits(name, prompts[0] + tails[0])[-1:], dtype, "second piece of a prompt")
+    assert_logits_close(got[1:2], plain_logits(name, more[0] + tails[1])[-1:], dtype, "second piece of a prompt")
+    # a slot that is given back and used again; exactly as many tokens as the graph has rows (no padding rows)
+    for e in (eager, graph):
+        e.release(slots[id(e)][1])
+        slots[id(e)][1] = e.acquire()
+    full = random_tokens(V, 16, 990)
+    got = both(lambda e: [(slots[id(e)][1], full)], "last")
+    assert_logits_close(got, plain_logits(name, full)[-1:], dtype, "a step without padding rows")
+    # decode steps after the replayed prompts read what they wrote
+    got = both(lambda e: [(slots[id(e)][0], [3]), (slots[id(e)][1], [4])], "last")
+    assert_logits_close(got[1:2], plain_logits(name, full + [4])[-1:], dtype, "decode after a captured prompt step")
+    for e in (eager, graph):
+        e.cache.check()
+    assert not any(isinstance(k[0], str) for k in eager._runners)
+
+
 def test_a_captured_step_keeps_its_own_scratch_memory():
     """A graph holds the addresses of the scratch memory it was captured with.  Larger steps
     afterwards (eager ones and larger captured ones) need more of it; the small runner's must stay

@@ -84,6 +84,7 @@ def test_per_op_times_of_eager_steps_and_their_refusal_under_capture():
     from synaptix_amd import Engine
     from synaptix_amd.kernels import ops
     eng = Engine.load(model_folder("B"), dtype="bfloat16", max_tokens=512)
+    eng.prompt_graphs = False                                  # (op by op means launched one by one, both times)
     s = eng.acquire()
     plain = eng.step([(s, [1, 2, 3, 4, 5])], want="last").clone()
     eng.release(s)
