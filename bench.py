@@ -85,9 +85,6 @@ def unequal_prompts_through_generate(args, shape, emit=True):
     from synaptix_amd import Qwen3Config, Engine
     from synaptix_amd.engine.generate import generate, GenerationConfig
 
-    if args.no_packed_copies:
-        from synaptix_amd.parts import keep_packed_copies
-        keep_packed_copies(False)
     n_prompts, lo, hi = 16, 64, 4096
     new_tokens = args.steps + 1                    # the first token of each sequence comes from the prompts' step
     if new_tokens < 2 or hi + new_tokens > 8192:
@@ -180,8 +177,6 @@ def main() -> int:
                     help="the longest sequence (positions and cache a sequence; the contract's run has 8,192)")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a decode step from the host")
-    ap.add_argument("--no-packed-copies", action="store_true",
-                    help="keep no second copy of the weights in MFMA fragment order: steps of up to 64 rows read the plain matrices")
     args = ap.parse_args()
     shape = SHAPES[args.shape]
     if args.steps is None:
@@ -208,9 +203,6 @@ def main() -> int:
     from synaptix_amd import Qwen3Config, Engine
     from synaptix_amd.kernels import ops
 
-    if args.no_packed_copies:
-        from synaptix_amd.parts import keep_packed_copies
-        keep_packed_copies(False)
     torch.manual_seed(0)
     cfg = Qwen3Config.from_dict({**shape, "num_hidden_layers": args.layers, "max_position_embeddings": args.context})
     batches = [args.batch] if args.no_points else sorted({args.batch, *POINTS[args.shape]})

@@ -22,13 +22,33 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
   for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = to_f32<T>(row[i]);
 }
 
-SYN_EXPORT int syn_embed(const void* table, int table_is_f32, const int* ids, float* resid, int n_tokens, int H,
+// the same from a bf16 table in fragment order ([V / 16][H / 32][64 lanes][8], as the products read the tied
+// output head): eight consecutive values of a row are one lane's 16 bytes
+__global__ void embed_packed_kernel(const bf16* __restrict__ table, const int* __restrict__ ids, float* __restrict__ resid,
+                                    int H) {
+  const int n = blockIdx.x, id = ids[n];
+  const bf16* group = table + (size_t)(id / 16) * H * 16;   // the 16 rows around row id: H / 32 fragments of 512 values
+  float* out = resid + (size_t)n * H;
+  for (int c = threadIdx.x; c < H / 8; c += blockDim.x) {   // chunk c: values 8 c .. 8 c + 7 of the row
+    const bf16x8 v = *(const bf16x8*)(group + (size_t)(c / 4) * 512 + ((c % 4) * 16 + id % 16) * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[c * 8 + e] = (float)v[e];
+  }
+}
+
+// table_kind: 0 = bf16 rows, 1 = float rows, 2 = bf16 in fragment order (V a multiple of 16, H of 32)
+SYN_EXPORT int syn_embed(const void* table, int table_kind, const int* ids, float* resid, int n_tokens, int H,
                          hipStream_t stream) {
   SYN_CHECK(n_tokens > 0 && H > 0, "embed: empty input (%d tokens, width %d)", n_tokens, H);
-  if (table_is_f32)
+  SYN_CHECK(table_kind >= 0 && table_kind <= 2, "embed: unknown kind of table %d", table_kind);
+  if (table_kind == 1) {
     embed_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)table, ids, resid, H);
-  else
+  } else if (table_kind == 2) {
+    SYN_CHECK(H % 32 == 0, "embed: a table in fragment order has a width that is a multiple of 32, not %d", H);
+    embed_packed_kernel<<<n_tokens, 256, 0, stream>>>((const bf16*)table, ids, resid, H);
+  } else {
     embed_kernel<bf16><<<n_tokens, 256, 0, stream>>>((const bf16*)table, ids, resid, H);
+  }
   SYN_LAUNCH_CHECK("embed");
   return 0;
 }

@@ -639,7 +639,11 @@ __device__ __forceinline__ int direct_swizzle(int row) {
   return BK == 64 ? (row >> 1) & 7 : row & (BK / 8 - 1);
 }
 
-template <int BM, int BN, int BK, int WM, int WN, bool PAIRED, int STAGES>
+// WP: w is the weight in fragment order (pack_weight: [N / 16][K / 32][64 lanes][8], N a multiple of 16).  A load of a
+// wave then moves one fragment (16 rows x 32 k-values, 1 KB of consecutive bytes) into the slot that a load of
+// plain rows fills, and a lane's fragment of an MFMA 32x32x16 lies in two of them: rows fr % 16 of fragment
+// fr / 16, chunks 2 (ks % 2) + fh of k-fragment ks / 2; 16 lanes read 256 consecutive bytes, without a swizzle.
+template <int BM, int BN, int BK, int WM, int WN, bool PAIRED, int STAGES, bool WP>
 __global__ void __launch_bounds__(64 * WM * WN)
 gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, Epilogue ep,
                    int M, int N, int K, int k_slice) {
@@ -670,14 +674,21 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
   static_assert(BM % (RPI * WAVES) == 0, "a pass lies in x or in W as a whole, for all waves alike");
   const size_t row_bytes = (size_t)K * sizeof(bf16);
   const BufferView vx = buffer_view(x + (size_t)m0 * K, (size_t)(M - m0) * row_bytes);
+  // (in fragment order 16 rows of W are K / 32 fragments of 1 KB one after another: as many bytes as 16 plain rows)
   const BufferView vw = buffer_view(w + (size_t)n0 * K, (size_t)(N - n0) * row_bytes);
+  constexpr int KF = BK / 32;                    // fragments of a k-tile along K
   unsigned src[PASSES];
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
     const int row0 = (p * WAVES + wave) * RPI, row = row0 + lane / CPR;
     const int chunk = (lane % CPR) ^ direct_swizzle<BK>(row);
-    const int in_tile = row0 < BM ? row : row - BM;
-    src[p] = (unsigned)((size_t)in_tile * row_bytes + chunk * 16);
+    if (WP && row0 >= BM) {
+      const int slot = (row0 - BM) / RPI;        // which fragment of the tile: 16 rows slot / KF, k-fragment slot % KF
+      src[p] = (unsigned)((size_t)(slot / KF) * 16 * row_bytes + (size_t)(slot % KF) * 1024 + lane * 16);
+    } else {
+      const int in_tile = row0 < BM ? row : row - BM;
+      src[p] = (unsigned)((size_t)in_tile * row_bytes + chunk * 16);
+    }
   }
   auto fetch = [&](int kt, int buf) {
 #pragma unroll
@@ -688,7 +699,7 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
       if (p * WAVES * RPI < BM)
         buffer_to_lds16(vx, dst, src[p], (k_begin + kt * BK) * (int)sizeof(bf16));
       else
-        buffer_to_lds16<true>(vw, dst, src[p], (k_begin + kt * BK) * (int)sizeof(bf16));
+        buffer_to_lds16<true>(vw, dst, src[p], (k_begin + kt * BK) * (int)sizeof(bf16) * (WP ? 16 : 1));
     }
   };
   // Tile kt lies in buffer kt % STAGES; while it is multiplied the STAGES - 1 tiles after it are on their
@@ -733,7 +744,10 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         const int row = wn + j * 32 + fr;
-        b[j] = *(const bf16x8*)(ws + row * BK + (c ^ direct_swizzle<BK>(row + BM)) * 8);
+        if constexpr (WP)
+          b[j] = *(const bf16x8*)(ws + ((row / 16) * KF + ks / 2) * 512 + ((2 * (ks % 2) + fh) * 16 + row % 16) * 8);
+        else
+          b[j] = *(const bf16x8*)(ws + row * BK + (c ^ direct_swizzle<BK>(row + BM)) * 8);
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -746,9 +760,15 @@ gemm_direct_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void*
   store_tiles<TM, TN, PAIRED>(acc, out, ep, blockIdx.y, M, N, m0 + wm, n0 + wn, lane);
 }
 
+// A weight [N, K] as a product is handed it: plain rows, or in fragment order (pack_weight)
+struct Weight {
+  const bf16* p;
+  bool packed;
+};
+
 // slices > 1 only with a float output [slices, M, N]; K must be a multiple of BK
 template <int BM, int BN, int BK, int WM, int WN, bool PAIRED = false, int STAGES = 3>
-static int launch_direct(const bf16* x, const bf16* w, void* out, Epilogue ep, int M, int N, int K,
+static int launch_direct(const bf16* x, Weight w, void* out, Epilogue ep, int M, int N, int K,
                          hipStream_t stream, int slices = 1) {
   SYN_CHECK(K % BK == 0, "gemm: K = %d is no multiple of the k-tile %d", K, BK);
   const int step = BK > 128 ? BK : 128;
@@ -757,13 +777,20 @@ static int launch_direct(const bf16* x, const bf16* w, void* out, Epilogue ep, i
   static OncePerDevice raised;
   if (lds > 65536) {
     const hipError_t e = once_per_device(raised, [&] {
-      return hipFuncSetAttribute((const void*)gemm_direct_kernel<BM, BN, BK, WM, WN, PAIRED, STAGES>,
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      hipError_t r = hipFuncSetAttribute((const void*)gemm_direct_kernel<BM, BN, BK, WM, WN, PAIRED, STAGES, false>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (r == hipSuccess)
+        r = hipFuncSetAttribute((const void*)gemm_direct_kernel<BM, BN, BK, WM, WN, PAIRED, STAGES, true>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      return r;
     });
     SYN_CHECK(e == hipSuccess, "gemm: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
   }
-  gemm_direct_kernel<BM, BN, BK, WM, WN, PAIRED, STAGES>
-      <<<dim3(tile_grid(M, N, BM, BN), slices), 64 * WM * WN, lds, stream>>>(x, w, out, ep, M, N, K, k_slice);
+  const dim3 grid(tile_grid(M, N, BM, BN), slices);
+  if (w.packed)
+    gemm_direct_kernel<BM, BN, BK, WM, WN, PAIRED, STAGES, true><<<grid, 64 * WM * WN, lds, stream>>>(x, w.p, out, ep, M, N, K, k_slice);
+  else
+    gemm_direct_kernel<BM, BN, BK, WM, WN, PAIRED, STAGES, false><<<grid, 64 * WM * WN, lds, stream>>>(x, w.p, out, ep, M, N, K, k_slice);
   return 0;
 }
 
@@ -781,7 +808,8 @@ static int launch_direct(const bf16* x, const bf16* w, void* out, Epilogue ep, i
 // Counters showed the texture addresser busy about 25 cycles for each 1 KB load of 8 rows x 128 bytes,
 // 1,600 of the 2,048 cycles that the MFMAs of a 256x256x64 tile take: loads that arrive in a burst
 // hold up the waves that issue them, so their spread matters more than their number.
-template <int BM, int BN, int WM, int WN, bool PAIRED>
+// WP: w in fragment order, as in gemm_direct_kernel.
+template <int BM, int BN, int WM, int WN, bool PAIRED, bool WP>
 __global__ void __launch_bounds__(64 * WM * WN)
 gemm_pipelined_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, void* __restrict__ out, Epilogue ep,
                       int M, int N, int K, int k_slice) {
@@ -808,7 +836,8 @@ gemm_pipelined_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, vo
   // below 2^32 for any M and N
   const size_t row_bytes = (size_t)K * sizeof(bf16);
   const BufferView vx = buffer_view(x + (size_t)m0 * K + k_begin, (size_t)(M - m0) * row_bytes - k_begin * sizeof(bf16));
-  const BufferView vw = buffer_view(w + (size_t)n0 * K + k_begin, (size_t)(N - n0) * row_bytes - k_begin * sizeof(bf16));
+  const BufferView vw = buffer_view(w + (size_t)n0 * K + (size_t)k_begin * (WP ? 16 : 1),
+                                    (size_t)(N - n0) * row_bytes - (size_t)k_begin * sizeof(bf16) * (WP ? 16 : 1));
   // pass p: the wave fills tile rows (p * WAVES + wave) * 8 .. + 8 (x rows first, then W rows; rows beyond M or
   // N repeat the last valid one and their results are never stored)
   unsigned src[PASSES];
@@ -816,12 +845,20 @@ gemm_pipelined_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, vo
   for (int p = 0; p < PASSES; ++p) {
     const int row0 = (p * WAVES + wave) * RPI, row = row0 + lane / 8;
     const int chunk = (lane % 8) ^ direct_swizzle<BK>(row);
-    const int in_tile = row0 < BM ? min(row, M - 1 - m0) : min(row - BM, N - 1 - n0);
-    src[p] = (unsigned)((size_t)in_tile * row_bytes + chunk * 16);
+    if (WP && row0 >= BM) {
+      // fragment slot of the tile: 16 rows slot / 2 (groups beyond N repeat the last one), k-fragment slot % 2
+      const int slot = (row0 - BM) / RPI, group = min(slot / 2, (N - n0) / 16 - 1);
+      src[p] = (unsigned)((size_t)group * 16 * row_bytes + (size_t)(slot % 2) * 1024 + lane * 16);
+    } else {
+      const int in_tile = row0 < BM ? min(row, M - 1 - m0) : min(row - BM, N - 1 - n0);
+      src[p] = (unsigned)((size_t)in_tile * row_bytes + chunk * 16);
+    }
   }
   auto fetch_pass = [&](int kt, int buf, int p) {
     bf16* dst = smem + (size_t)buf * ROWS * BK + (size_t)(p * WAVES + wave) * RPI * BK;
-    buffer_to_lds16((p * WAVES + wave) * RPI < BM ? vx : vw, dst, src[p], kt * (BK * (int)sizeof(bf16)));
+    const bool of_x = (p * WAVES + wave) * RPI < BM;
+    // (a k-tile of 64 is 128 bytes further on in a plain row, two fragments of 1 KB further on in fragment order)
+    buffer_to_lds16(of_x ? vx : vw, dst, src[p], kt * (BK * (int)sizeof(bf16)) * (WP && !of_x ? 16 : 1));
   };
 
   f32x16 acc[TM][TN];
@@ -837,12 +874,18 @@ gemm_pipelined_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, vo
 #pragma unroll
   for (int i = 0; i < TM; ++i) arow[i] = (wm + i * 32 + fr) * BK, asw[i] = direct_swizzle<BK>(wm + i * 32 + fr);
 #pragma unroll
-  for (int j = 0; j < TN; ++j) brow[j] = (BM + wn + j * 32 + fr) * BK, bsw[j] = direct_swizzle<BK>(BM + wn + j * 32 + fr);
+  for (int j = 0; j < TN; ++j) {
+    const int row = wn + j * 32 + fr;
+    // (in fragment order: the two fragments of rows row / 16 begin at 1,024 elements a group; k-step ks lies 256 further on)
+    brow[j] = WP ? BM * BK + (row / 16) * 1024 + (fh * 16 + row % 16) * 8 : (BM + row) * BK;
+    bsw[j] = direct_swizzle<BK>(BM + row);
+  }
   bf16x8 a[2][TM], b[2][TN];   // two sets of fragments: one is multiplied while the other is read
   auto read_one = [&](int buf, int ks, int set, int idx) {
     const bf16* base = smem + (size_t)buf * ROWS * BK;
     const int c = 2 * ks + fh;  // the 16-byte chunk of a row that this lane multiplies
     if (idx < TM) a[set][idx] = *(const bf16x8*)(base + arow[idx] + (c ^ asw[idx]) * 8);
+    else if constexpr (WP) b[set][idx - TM] = *(const bf16x8*)(base + brow[idx - TM] + ks * 256);
     else b[set][idx - TM] = *(const bf16x8*)(base + brow[idx - TM] + (c ^ bsw[idx - TM]) * 8);
   };
   auto mfmas = [&](int set) {
@@ -911,7 +954,7 @@ gemm_pipelined_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, vo
 }
 
 template <int BM, int BN, int WM, int WN, bool PAIRED = false>
-static int launch_pipelined(const bf16* x, const bf16* w, void* out, Epilogue ep, int M, int N, int K,
+static int launch_pipelined(const bf16* x, Weight w, void* out, Epilogue ep, int M, int N, int K,
                             hipStream_t stream, int slices = 1) {
   SYN_CHECK(K % 64 == 0, "gemm: K = %d is no multiple of the k-tile 64", K);
   const int k_slice = ((K + slices - 1) / slices + 127) / 128 * 128;  // the same cut as the tiles for few rows make
@@ -920,19 +963,26 @@ static int launch_pipelined(const bf16* x, const bf16* w, void* out, Epilogue ep
   static OncePerDevice raised;
   if (lds > 65536) {
     const hipError_t e = once_per_device(raised, [&] {
-      return hipFuncSetAttribute((const void*)gemm_pipelined_kernel<BM, BN, WM, WN, PAIRED>,
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      hipError_t r = hipFuncSetAttribute((const void*)gemm_pipelined_kernel<BM, BN, WM, WN, PAIRED, false>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (r == hipSuccess)
+        r = hipFuncSetAttribute((const void*)gemm_pipelined_kernel<BM, BN, WM, WN, PAIRED, true>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      return r;
     });
     SYN_CHECK(e == hipSuccess, "gemm: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
   }
-  gemm_pipelined_kernel<BM, BN, WM, WN, PAIRED>
-      <<<dim3(tile_grid(M, N, BM, BN), slices), 64 * WM * WN, lds, stream>>>(x, w, out, ep, M, N, K, k_slice);
+  const dim3 grid(tile_grid(M, N, BM, BN), slices);
+  if (w.packed)
+    gemm_pipelined_kernel<BM, BN, WM, WN, PAIRED, true><<<grid, 64 * WM * WN, lds, stream>>>(x, w.p, out, ep, M, N, K, k_slice);
+  else
+    gemm_pipelined_kernel<BM, BN, WM, WN, PAIRED, false><<<grid, 64 * WM * WN, lds, stream>>>(x, w.p, out, ep, M, N, K, k_slice);
   return 0;
 }
 
 // M > 64: the tile shape by pick_large_tile; loads straight into LDS where K allows it
 template <bool PAIRED>
-static int launch_large(const bf16* x, const bf16* w, void* out, Epilogue ep, int M, int N, int K,
+static int launch_large(const bf16* x, Weight w, void* out, Epilogue ep, int M, int N, int K,
                         hipStream_t stream, int slices = 1);
 
 // Compute units of the current device (256 on an MI355X), asked once a device: what the rules for tiles fill.
@@ -974,7 +1024,7 @@ static int pick_large_tile(int M, int N) {
 }
 
 template <bool PAIRED>
-static int launch_large(const bf16* x, const bf16* w, void* out, Epilogue ep, int M, int N, int K,
+static int launch_large(const bf16* x, Weight w, void* out, Epilogue ep, int M, int N, int K,
                         hipStream_t stream, int slices) {
   // cut along K (the reader adds the partial sums): the largest tile, which the slices multiply
   if (slices > 1) return launch_pipelined<256, 256, 2, 4, PAIRED>(x, w, out, ep, M, N, K, stream, slices);
@@ -985,18 +1035,23 @@ static int launch_large(const bf16* x, const bf16* w, void* out, Epilogue ep, in
     if (shape == 3) return launch_pipelined<256, 160, 4, 1, PAIRED>(x, w, out, ep, M, N, K, stream);
     return launch_pipelined<128, 128, 2, 2, PAIRED>(x, w, out, ep, M, N, K, stream);
   }
-  if (shape == 0) return launch_tiled<256, 256, 64, 4, 2, PAIRED>(x, w, out, ep, M, N, K, stream);
-  if (shape == 1 || shape == 3) return launch_tiled<256, 192, 64, 4, 2, PAIRED>(x, w, out, ep, M, N, K, stream);
-  return launch_tiled<128, 128, 64, 2, 2, PAIRED>(x, w, out, ep, M, N, K, stream);
+  SYN_CHECK(!w.packed, "gemm: a weight in fragment order needs a K that is a multiple of 64 (K = %d)", K);
+  if (shape == 0) return launch_tiled<256, 256, 64, 4, 2, PAIRED>(x, w.p, out, ep, M, N, K, stream);
+  if (shape == 1 || shape == 3) return launch_tiled<256, 192, 64, 4, 2, PAIRED>(x, w.p, out, ep, M, N, K, stream);
+  return launch_tiled<128, 128, 64, 2, 2, PAIRED>(x, w.p, out, ep, M, N, K, stream);
 }
 
 // ------------------------------------------------------------------ entry point
 // dtype: 0 = float in, float out; 1 = bf16 in, bf16 out; 2 = bf16 in, float out.
 // slices > 1 (bf16 in, float out): out is [slices, M, N], slice s holds the sum over its part of K; the
 // reader adds the slices.
+// w_packed: w is the weight in fragment order (pack_weight; bf16, N a multiple of 16, K of 128): for the tiles that
+// load straight into LDS; the other kernels read plain rows only.
 SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int M, int N, int K, int force_simt,
-                        int slices, hipStream_t stream) {
+                        int slices, int w_packed, hipStream_t stream) {
   SYN_CHECK(M > 0 && N > 0 && K > 0, "gemm: empty shape M=%d N=%d K=%d", M, N, K);
+  SYN_CHECK(!w_packed || (dtype != 0 && !force_simt && N % 16 == 0 && K % 128 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0),
+            "gemm: a weight in fragment order needs bf16 operands, N = %d a multiple of 16 and K = %d of 128", N, K);
   SYN_CHECK(dtype >= 0 && dtype <= 2, "gemm: unknown dtype code %d", dtype);
   SYN_CHECK(slices >= 1 && (slices == 1 || (dtype == 2 && !force_simt && K % 8 == 0 && slices <= 64 && (M <= 64 || K % 64 == 0))),
             "gemm: %d slices of K need bf16 operands and a float output (and beyond 64 rows a K that is a multiple of 64; K = %d)", slices, K);
@@ -1020,6 +1075,7 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   }
   const bf16* xb = (const bf16*)x;
   const bf16* wb = (const bf16*)w;
+  const Weight wt = {wb, w_packed != 0};
   // From sweeps at the shapes of an 8B model (N = 4096 .. 151936, K = 4096 and 12288).
   // Short prompts (65 to 512 rows) of a narrow product: even the smallest of the large tiles would leave
   // most compute units without work (q/k/v at 128 rows: 48 tiles of 128 x 128), and the product is still
@@ -1031,41 +1087,41 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   const long tiles_cut = (long)(M <= 256 ? (M + 127) / 128 : (M + 255) / 256) * ((N + 127) / 128);
   const bool few_large_tiles = M > 64 && M <= 512 && K % 128 == 0 && (slices > 1 ? tiles_cut : tiles128) * slices <= compute_units();
   int rc = 0;
-  if (M == 1 && slices == 1) {
+  if (M == 1 && slices == 1 && !w_packed) {
     // one row: fragments of W straight from memory, K split over the waves
     if (N <= 8192) launch_skinny<1, 16, 4>(xb, wb, out, ep, M, N, K, stream);
     else launch_skinny<1, 8, 4>(xb, wb, out, ep, M, N, K, stream);
   } else if (M <= 32) {
     // few rows: memory-bound; small tiles (many workgroups), deep in K (long pieces of each row), three
     // k-tiles in flight, straight into LDS where K allows it
-    if (N >= 65536 && K % 256 == 0) rc = launch_direct<32, 64, 256, 1, 2>(xb, wb, out, ep, M, N, K, stream, slices);
-    else if (N >= 65536) rc = launch_tiled<32, 32, 256, 1, 1>(xb, wb, out, ep, M, N, K, stream, slices);
-    else if (K % 128 == 0) rc = launch_direct<32, 64, 128, 1, 2>(xb, wb, out, ep, M, N, K, stream, slices);
+    if (N >= 65536 && K % 256 == 0) rc = launch_direct<32, 64, 256, 1, 2>(xb, wt, out, ep, M, N, K, stream, slices);
+    else if (N >= 65536 && !w_packed) rc = launch_tiled<32, 32, 256, 1, 1>(xb, wb, out, ep, M, N, K, stream, slices);
+    else if (K % 128 == 0) rc = launch_direct<32, 64, 128, 1, 2>(xb, wt, out, ep, M, N, K, stream, slices);
     else rc = launch_tiled<32, 64, 128, 1, 2>(xb, wb, out, ep, M, N, K, stream, slices);
   } else if (M <= 64 && K % 128 == 0) {
     // 33 to 64 rows: 128 rows of W a workgroup, so that the rows of x are fetched half as often (every
     // workgroup reads all of x), three k-tiles in a ring, one workgroup a compute unit.  A decode step of 64
     // sequences: 7.70 -> 7.51 ms with this tile for q/k/v, o_proj and down_proj, 7.26 with it for gate+up
     // as well (though that product then has only 192 workgroups); 64 x 64 tiles in a ring of four: 8.08.
-    rc = launch_direct<64, 128, 128, 2, 4, false, 3>(xb, wb, out, ep, M, N, K, stream, slices);
+    rc = launch_direct<64, 128, 128, 2, 4, false, 3>(xb, wt, out, ep, M, N, K, stream, slices);
   } else if (few_large_tiles && slices > 1) {
     // short prompts of a narrow product whose reader adds partial sums: k-tiles of 64 in a ring of three, 128 rows
     // of W a workgroup, and as many slices of K as fill the compute units (ops.gemm_slices).  Measured at the
     // shapes of an 8B layer against the tiles of the branch below: 128 rows: q/k/v in 4 slices 17 us (31 uncut),
     // down_proj in 8 slices 26 (30 in 4); 256 rows: q/k/v 26 (32), down_proj 39 (50); 512 rows (256 rows of x a
     // tile): q/k/v in 2 slices 36 (51), o_proj in 4 slices 29 (30), down_proj 57 (55).
-    if (M <= 256) rc = launch_direct<128, 128, 64, 2, 4, false, 3>(xb, wb, out, ep, M, N, K, stream, slices);
-    else rc = launch_direct<256, 128, 64, 4, 2, false, 3>(xb, wb, out, ep, M, N, K, stream, slices);
+    if (M <= 256) rc = launch_direct<128, 128, 64, 2, 4, false, 3>(xb, wt, out, ep, M, N, K, stream, slices);
+    else rc = launch_direct<256, 128, 64, 4, 2, false, 3>(xb, wt, out, ep, M, N, K, stream, slices);
   } else if (few_large_tiles && K % 128 == 0) {
     // the same uncut: 64 x 128 up to 256 rows, 128 x 128 beyond (a prompt of 256 tokens
     // 8.91 -> 8.24 ms, of 512 tokens 12.63 -> 11.59 ms against 64 x 64 tiles)
-    if (M <= 256) rc = launch_direct<64, 128, 128, 2, 4, false, 3>(xb, wb, out, ep, M, N, K, stream, slices);
-    else rc = launch_direct<128, 128, 128, 2, 4, false, 2>(xb, wb, out, ep, M, N, K, stream, slices);
+    if (M <= 256) rc = launch_direct<64, 128, 128, 2, 4, false, 3>(xb, wt, out, ep, M, N, K, stream, slices);
+    else rc = launch_direct<128, 128, 128, 2, 4, false, 2>(xb, wt, out, ep, M, N, K, stream, slices);
   } else if (M <= 64 || few_large_tiles) {
-    if (K % 128 == 0) rc = launch_direct<64, 64, 128, 2, 2, false, 2>(xb, wb, out, ep, M, N, K, stream, slices);
+    if (K % 128 == 0) rc = launch_direct<64, 64, 128, 2, 2, false, 2>(xb, wt, out, ep, M, N, K, stream, slices);
     else rc = launch_tiled<64, 64, 128, 2, 2>(xb, wb, out, ep, M, N, K, stream, slices);
   } else {
-    rc = launch_large<false>(xb, wb, out, ep, M, N, K, stream, slices);
+    rc = launch_large<false>(xb, wt, out, ep, M, N, K, stream, slices);
   }
   if (rc) return rc;
   SYN_LAUNCH_CHECK("gemm");
@@ -1075,8 +1131,11 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
 // out[M, N/2] = silu(x . Wg^T) * (x . Wu^T), bf16, where w [N, K] holds the rows of Wg and of Wu in
 // turns of 16: rows 32b .. 32b+15 are rows 16b .. 16b+15 of Wg, rows 32b+16 .. 32b+31 those of Wu.
 // The activation is applied to the 32-bit sums and rounded once.
-SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, int N, int K, int act, hipStream_t stream) {
+// w_packed: as for syn_gemm
+SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, int N, int K, int act, int w_packed,
+                               hipStream_t stream) {
   SYN_CHECK(M > 0 && N > 0 && K > 0, "gemm_swiglu: empty shape M=%d N=%d K=%d", M, N, K);
+  SYN_CHECK(!w_packed || K % 128 == 0, "gemm_swiglu: a weight in fragment order needs K = %d a multiple of 128", K);
   SYN_CHECK(act >= 0 && act < SYN_ACT_COUNT, "gemm_swiglu: unknown activation code %d", act);
   const Epilogue ep = {0, act};
   SYN_CHECK(N % 32 == 0, "gemm_swiglu: %d paired rows are no multiple of 32", N);
@@ -1085,15 +1144,16 @@ SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, i
   const bf16* xb = (const bf16*)x;
   const bf16* wb = (const bf16*)w;
   int rc = 0;
-  if (M == 1) {
+  const Weight wt = {wb, w_packed != 0};
+  if (M == 1 && !w_packed) {
     // one row: fragments of W straight from memory; eight waves on the gate rows, eight on the up rows
     launch_skinny<2, 8, 4, true>(xb, wb, out, ep, M, N, K, stream);
   } else if (M <= 32) {
-    if (N >= 65536) rc = launch_tiled<32, 32, 256, 1, 1, true>(xb, wb, out, ep, M, N, K, stream);
-    else if (K % 128 == 0) rc = launch_direct<32, 64, 128, 1, 2, true>(xb, wb, out, ep, M, N, K, stream);
+    if (N >= 65536 && !w_packed) rc = launch_tiled<32, 32, 256, 1, 1, true>(xb, wb, out, ep, M, N, K, stream);
+    else if (K % 128 == 0) rc = launch_direct<32, 64, 128, 1, 2, true>(xb, wt, out, ep, M, N, K, stream);
     else rc = launch_tiled<32, 64, 128, 1, 2, true>(xb, wb, out, ep, M, N, K, stream);
   } else if (M <= 64) {
-    if (K % 128 == 0) rc = launch_direct<64, 128, 128, 2, 2, true, 3>(xb, wb, out, ep, M, N, K, stream);
+    if (K % 128 == 0) rc = launch_direct<64, 128, 128, 2, 2, true, 3>(xb, wt, out, ep, M, N, K, stream);
     else rc = launch_tiled<64, 64, 128, 2, 2, true>(xb, wb, out, ep, M, N, K, stream);
   } else if (M <= 256 && K % 64 == 0) {
     // 65 to 256 rows: still bound by reading W.  All of x in one tile, so that W is read once; k-tiles of 64 in a
@@ -1101,11 +1161,11 @@ SYN_EXPORT int syn_gemm_swiglu(const void* x, const void* w, void* out, int M, i
     // (N = 24576, K = 4096) against the smallest of the large tiles: 128 rows 66 -> 46 us (96 rows of W a
     // workgroup: 256 workgroups), 192 rows 72 -> 57, 256 rows 80 -> 62; from 320 rows on the large tiles win
     // (98 against 110 us and more).
-    if (M <= 128) rc = launch_direct<128, 96, 64, 4, 1, true, 4>(xb, wb, out, ep, M, N, K, stream);
-    else if (M <= 192) rc = launch_direct<192, 128, 64, 2, 2, true, 3>(xb, wb, out, ep, M, N, K, stream);
-    else rc = launch_direct<256, 128, 64, 4, 2, true, 3>(xb, wb, out, ep, M, N, K, stream);
+    if (M <= 128) rc = launch_direct<128, 96, 64, 4, 1, true, 4>(xb, wt, out, ep, M, N, K, stream);
+    else if (M <= 192) rc = launch_direct<192, 128, 64, 2, 2, true, 3>(xb, wt, out, ep, M, N, K, stream);
+    else rc = launch_direct<256, 128, 64, 4, 2, true, 3>(xb, wt, out, ep, M, N, K, stream);
   } else {
-    rc = launch_large<true>(xb, wb, out, ep, M, N, K, stream);
+    rc = launch_large<true>(xb, wt, out, ep, M, N, K, stream);
   }
   if (rc) return rc;
   SYN_LAUNCH_CHECK("gemm_swiglu");

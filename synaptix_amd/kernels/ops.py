@@ -151,13 +151,17 @@ def activation_code(name) -> int:
 # ----------------------------------------------------------------------------- rows
 
 def embed(table, ids, resid):
-    """resid[n, :] = table[ids[n], :] as float.  table [V, H] bf16|f32, ids [N] int32, resid [N, H] f32."""
-    _need(table, "embed.table", (_BF16, _F32), (None, None))
-    V, H = table.shape
+    """resid[n, :] = table[ids[n], :] as float.  table [V, H] bf16|f32 (or bf16 in fragment order, pack_weight: four
+    dimensions), ids [N] int32, resid [N, H] f32."""
+    if isinstance(table, torch.Tensor) and table.dim() == 4:
+        _need(table, "embed.table", _BF16, (None, None, 64, 8))
+        H, kind = table.shape[1] * 32, 2
+    else:
+        _need(table, "embed.table", (_BF16, _F32), (None, None))
+        H, kind = table.shape[1], _is_f32(table)
     _need(ids, "embed.ids", _I32, (None,))
     _need(resid, "embed.resid", _F32, (ids.shape[0], H))
-    _call(load_library("core"), "syn_embed", _ptr(table), _is_f32(table), _ptr(ids), _ptr(resid),
-          ids.shape[0], H, _stream())
+    _call(load_library("core"), "syn_embed", _ptr(table), kind, _ptr(ids), _ptr(resid), ids.shape[0], H, _stream())
 
 
 def add_rmsnorm(resid, delta, gain, eps, out, rows=None, gain_offset=0.0):
@@ -206,15 +210,36 @@ def swiglu(gate_up, out, activation="silu"):
 
 # ----------------------------------------------------------------------------- matrix product
 
+def _packed_shape(w, name, K):
+    """(N, K) of a weight in fragment order (pack_weight), checked against the rows' width."""
+    _need(w, name, _BF16, (None, K // 32 if K % 32 == 0 else -1, 64, 8))
+    return w.shape[0] * 16
+
+
 def gemm(x, w, out, force_simt=False):
     """out[M, N] = x[M, K] . w[N, K]^T with 32-bit accumulation.
     float x float -> float (plain FMA); bf16 x bf16 -> bf16 or float (MFMA).
     A float out of shape [S, M, N] (bf16 operands) receives S partial sums over slices of K
-    instead; their sum over S is the product."""
+    instead; their sum over S is the product.
+    w may be the weight in fragment order (pack_weight: four dimensions): the tiles for 9 rows and more read it
+    where K is a multiple of 128; for other K the product runs in blocks of 16 rows through gemm_packed."""
     _need(x, "gemm.x", (_BF16, _F32), (None, None))
     M, K = x.shape
-    _need(w, "gemm.w", x.dtype, (None, K))
-    N = w.shape[0]
+    packed = isinstance(w, torch.Tensor) and w.dim() == 4
+    if packed:
+        if x.dtype != _BF16 or force_simt:
+            raise KernelError("gemm: a weight in fragment order takes bf16 rows and the MFMA kernels")
+        N = _packed_shape(w, "gemm.w", K)
+        if K % 128:
+            if out.dim() == 3 and out.shape[0] != 1:
+                raise KernelError(f"gemm: no slices of K = {K} over a weight in fragment order")
+            rows = out[0] if out.dim() == 3 else out
+            for m0 in range(0, M, PACKED_BLOCK_ROWS):
+                gemm_packed(x[m0:m0 + PACKED_BLOCK_ROWS], w, rows[m0:m0 + PACKED_BLOCK_ROWS])
+            return
+    else:
+        _need(w, "gemm.w", x.dtype, (None, K))
+        N = w.shape[0]
     slices = 1
     if out.dim() == 3:
         slices = out.shape[0]
@@ -230,7 +255,7 @@ def gemm(x, w, out, force_simt=False):
         _need(out, "gemm.out", (_BF16, _F32), (M, N))
         code = 2 if out.dtype == _F32 else 1
     _call(load_library("core"), "syn_gemm", _ptr(x), _ptr(w), _ptr(out), code, M, N, K, 1 if force_simt else 0,
-          slices, _stream())
+          slices, 1 if packed else 0, _stream())
 
 
 PAIR = 16   # rows of the gate and of the up projection alternate in turns of this many
@@ -246,18 +271,29 @@ def pair_rows(gate, up):
 
 def gemm_swiglu(x, w_paired, out, activation="silu"):
     """out[M, I] = act(x . Wg^T) * (x . Wu^T) in bf16 with w_paired = pair_rows(Wg, Wu): the
-    activation on the 32-bit sums inside the product, so that the two products are never stored."""
+    activation on the 32-bit sums inside the product, so that the two products are never stored.
+    w_paired may be in fragment order (pack_weight of the paired rows), as for gemm."""
     _need(x, "gemm_swiglu.x", _BF16, (None, None))
     M, K = x.shape
-    _need(w_paired, "gemm_swiglu.w", _BF16, (None, K))
-    N = w_paired.shape[0]
+    packed = isinstance(w_paired, torch.Tensor) and w_paired.dim() == 4
+    if packed:
+        N = _packed_shape(w_paired, "gemm_swiglu.w", K)
+    else:
+        _need(w_paired, "gemm_swiglu.w", _BF16, (None, K))
+        N = w_paired.shape[0]
     if N % (2 * PAIR) or K % 8:
         raise KernelError(f"gemm_swiglu: {N} paired rows, K = {K} (multiples of {2 * PAIR} and of 8)")
     _need(out, "gemm_swiglu.out", _BF16, (M, N // 2))
+    if packed and K % 128:
+        for m0 in range(0, M, PACKED_BLOCK_ROWS):
+            gemm_packed(x[m0:m0 + PACKED_BLOCK_ROWS], w_paired, out[m0:m0 + PACKED_BLOCK_ROWS], paired=True,
+                        activation=activation)
+        return
     _call(load_library("core"), "syn_gemm_swiglu", _ptr(x), _ptr(w_paired), _ptr(out), M, N, K,
-          activation_code(activation), _stream())
+          activation_code(activation), 1 if packed else 0, _stream())
 
 
+PACKED_BLOCK_ROWS = 16   # the most rows that a product of gemm_packed takes
 PACKED_MAX_ROWS = 8   # up to this many rows of x the products over packed weights are the faster ones
 PACKED_MAX_ROWS_GATED = 16   # the gated product, whose waves take two groups of rows of W for every fragment of x
 

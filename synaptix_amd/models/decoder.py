@@ -19,7 +19,7 @@ import torch
 
 from ..kernels import ops
 from ..parts.base import Part
-from ..parts.linear import linear, packed_copy, as_delta, as_rows
+from ..parts.linear import Matrix, linear, as_delta, as_rows
 from ..weights.source import TensorSpec
 
 
@@ -40,11 +40,11 @@ class TokenEmbedding(Part):
         return {self.name: TensorSpec((self.vocab, self.hidden), "table")}
 
     def load(self, get):
-        self.table = get(self.name)
+        self.table = Matrix(get(self.name))       # (a tied output head multiplies with the same matrix)
 
     def forward(self, ids):
         resid = torch.empty((ids.shape[0], self.hidden), dtype=torch.float32, device=ids.device)
-        ops.embed(self.table, ids, resid)
+        ops.embed(self.table.data, ids, resid)
         return resid
 
 
@@ -54,7 +54,7 @@ class OutputHead(Part):
 
     def __init__(self, name: str, vocab: int, hidden: int, tied_to: TokenEmbedding | None = None):
         self.name, self.vocab, self.hidden, self.tied_to = name, vocab, hidden, tied_to
-        self.weight = self.packed = None
+        self.weight = None
 
     def tensor_specs(self):
         return {} if self.tied_to is not None else {self.name: TensorSpec((self.vocab, self.hidden))}
@@ -64,11 +64,10 @@ class OutputHead(Part):
         return [self.name] if self.tied_to is not None else []
 
     def load(self, get):
-        self.weight = self.tied_to.table if self.tied_to is not None else get(self.name)
-        self.packed = packed_copy(self.weight)   # in fragment order, for single tokens
+        self.weight = self.tied_to.table if self.tied_to is not None else Matrix(get(self.name))
 
     def forward(self, h):
-        return linear(h, self.weight, torch.float32, self.packed)
+        return linear(h, self.weight, torch.float32)
 
 
 class DecoderModel:

@@ -4,8 +4,8 @@ from .position import Position, NoPosition, RotaryHalfSplit
 from .mixer import Mixer, GqaAttention
 from .feedforward import FeedForward, GatedMlp
 from .block import Block, PreNormBlock
-from .linear import (keep_packed_copies, linear, linear_for_sum, deferred_product, DeferredProduct, ScaledRows,
+from .linear import (Matrix, linear, linear_for_sum, deferred_product, DeferredProduct, ScaledRows,
                      as_rows, as_delta)
 
 __all__ = ["Part", "KvNeed", "StateNeed", "RmsNorm", "Position", "NoPosition", "RotaryHalfSplit", "Mixer",
-           "GqaAttention", "FeedForward", "GatedMlp", "Block", "PreNormBlock", "linear", "keep_packed_copies"]
+           "GqaAttention", "FeedForward", "GatedMlp", "Block", "PreNormBlock", "linear", "Matrix"]

@@ -10,7 +10,7 @@ import torch
 from ..kernels import ops
 from ..weights.source import TensorSpec
 from .base import Part
-from .linear import linear, linear_for_sum, deferred_product, as_rows, ScaledRows, packed_copy
+from .linear import Matrix, linear, linear_for_sum, deferred_product, as_rows, ScaledRows
 
 
 class FeedForward(Part):
@@ -32,7 +32,6 @@ class GatedMlp(FeedForward):
             raise ValueError(f"{prefix}: {e}") from None
         self.prefix, self.hidden, self.intermediate, self.activation = prefix, hidden, intermediate, activation
         self.w_gate_up = self.w_down = None
-        self.p_gate_up = self.p_down = None   # copies in fragment order for single tokens
         self.paired = False      # gate and up rows in turns of 16: the activation runs inside the product
 
     def tensor_specs(self):
@@ -48,22 +47,21 @@ class GatedMlp(FeedForward):
         gate, up = get(p + "gate_proj.weight"), get(p + "up_proj.weight")
         self.paired = (gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16
                        and self.intermediate % ops.PAIR == 0 and self.hidden % 8 == 0)
-        self.w_gate_up = ops.pair_rows(gate, up) if self.paired else torch.cat([gate, up], 0)
-        self.w_down = get(p + "down_proj.weight")
-        self.p_gate_up = packed_copy(self.w_gate_up) if self.paired and self.intermediate % 16 == 0 else None
-        self.p_down = packed_copy(self.w_down)
+        self.w_gate_up = Matrix(ops.pair_rows(gate, up) if self.paired else torch.cat([gate, up], 0))
+        self.w_down = Matrix(get(p + "down_proj.weight"))
 
     def forward(self, h, ctx):
         m = torch.empty((h.shape[0], self.intermediate), dtype=h.dtype, device=h.device)
         if self.paired and h.dtype == torch.bfloat16:
-            if self.p_gate_up is not None and h.shape[0] <= ops.PACKED_MAX_ROWS_GATED:
+            if self.w_gate_up.packed is not None and h.shape[0] <= ops.PACKED_MAX_ROWS_GATED:
                 if isinstance(h, ScaledRows):      # the norm's last step is the product's epilogue
-                    ops.gemm_packed(h.rows, self.p_gate_up, m, paired=True, activation=self.activation, row_scale=h.row_scale)
+                    ops.gemm_packed(h.rows, self.w_gate_up.packed, m, paired=True, activation=self.activation,
+                                    row_scale=h.row_scale)
                 else:
-                    ops.gemm_packed(h, self.p_gate_up, m, paired=True, activation=self.activation)
+                    ops.gemm_packed(h, self.w_gate_up.packed, m, paired=True, activation=self.activation)
             else:
-                ops.gemm_swiglu(as_rows(h), self.w_gate_up, m, self.activation)
+                ops.gemm_swiglu(as_rows(h), self.w_gate_up.data, m, self.activation)
         else:
             h = as_rows(h)
             ops.swiglu(linear(h, self.w_gate_up, h.dtype), m, self.activation)
-        return deferred_product(m, self.w_down, self.p_down)
+        return deferred_product(m, self.w_down)

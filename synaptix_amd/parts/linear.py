@@ -10,25 +10,38 @@ import torch
 from ..kernels import ops
 
 
-_KEEP_PACKED_COPIES = True
+class Matrix:
+    """A weight [N, K] as the products read it, kept once: a bf16 matrix whose sizes allow it (N a multiple of
+    16, K of 32) lies in the order of the MFMA fragments (ops.pack_weight), which the products for single tokens
+    need and the tiles for prompts read as well; any other lies in plain rows (`plain`)."""
+
+    def __init__(self, w, keep_rows: bool = False):
+        """keep_rows: leave w in plain rows whatever its sizes (a small matrix that only ever meets many rows)."""
+        self.shape, self.dtype, self.device = tuple(w.shape), w.dtype, w.device
+        self.packed = None if keep_rows else ops.pack_weight(w)
+        self.plain = w if self.packed is None else None
+
+    @property
+    def data(self):
+        """What ops.gemm, ops.gemm_swiglu and ops.embed take for this weight."""
+        return self.plain if self.packed is None else self.packed
+
+    def rows(self):
+        """The matrix in plain rows (a copy, if it is kept in fragment order): for tests and tools."""
+        return self.plain if self.packed is None else ops.unpack_weight(self.packed)
+
+    def nbytes(self):
+        t = self.data
+        return t.numel() * t.element_size()
 
 
-def keep_packed_copies(flag: bool) -> None:
-    """Whether models loaded from now on keep the second copy of their bf16 weights (packed_copy).
-    Without it single tokens read the plain matrices through the slower kernels."""
-    global _KEEP_PACKED_COPIES
-    _KEEP_PACKED_COPIES = bool(flag)
+def _use_packed(x, m):
+    return m.packed is not None and x.dtype == torch.bfloat16 and x.shape[0] <= ops.PACKED_MAX_ROWS
 
 
-def packed_copy(w):
-    """What a part keeps beside a bf16 weight for single tokens: the same matrix in the order of the MFMA
-    fragments (ops.pack_weight), or None.  It doubles the memory of the weight; a step of up to
-    ops.PACKED_MAX_ROWS rows reads it instead of w."""
-    return ops.pack_weight(w) if _KEEP_PACKED_COPIES and w.dtype == torch.bfloat16 else None
-
-
-def _use_packed(x, packed):
-    return packed is not None and x.dtype == torch.bfloat16 and x.shape[0] <= ops.PACKED_MAX_ROWS
+def _matrix(w):
+    """The products below take a Matrix; a tensor [N, K] in plain rows is taken as it is."""
+    return w if isinstance(w, Matrix) else Matrix(w, keep_rows=True)
 
 
 class ScaledRows:
@@ -62,12 +75,12 @@ class DeferredProduct:
     the residual rows runs it with the residual sum and its own first half as the epilogue (ops.gemm_packed,
     resid_norm), or asks for `run()`, the float product itself."""
 
-    def __init__(self, x, w, packed):
-        self.x, self.w, self.packed = x, w, packed
+    def __init__(self, x, w):
+        self.x, self.w, self.packed = x, w, w.packed
         self.shape = (x.shape[0], w.shape[0])
 
     def run(self):
-        return linear_for_sum(self.x, self.w, self.packed)
+        return linear_for_sum(self.x, self.w)
 
 
 def as_delta(d):
@@ -75,24 +88,25 @@ def as_delta(d):
     return d.run() if isinstance(d, DeferredProduct) else d
 
 
-def deferred_product(x, w, packed=None):
-    """linear_for_sum, but where the product would run over packed weights in one slice it is only described:
+def deferred_product(x, w):
+    """linear_for_sum, but where the product would run over few rows in one slice it is only described:
     the caller's result is the delta that a following norm adds to the residual rows, and that norm can take the
     product in (RmsNorm.add_apply)."""
-    if isinstance(x, torch.Tensor) and _use_packed(x, packed) and ops.packed_slices(w.shape[0], w.shape[1]) <= 1:
-        return DeferredProduct(x, w, packed)
-    return linear_for_sum(x, w, packed)
+    w = _matrix(w)
+    if isinstance(x, torch.Tensor) and _use_packed(x, w) and ops.packed_slices(w.shape[0], w.shape[1]) <= 1:
+        return DeferredProduct(x, w)
+    return linear_for_sum(x, w)
 
 
-def linear(x, w, out_dtype, packed=None):
-    """x [M, K] in the activation type, w [N, K]; a weight kept in 32-bit takes the 32-bit product.
-    packed: packed_copy(w), taken for few rows."""
-    if _use_packed(x, packed) and out_dtype in (torch.bfloat16, torch.float32):
+def linear(x, w, out_dtype):
+    """x [M, K] in the activation type, w a Matrix [N, K]; a weight kept in 32-bit takes the 32-bit product."""
+    w = _matrix(w)
+    if _use_packed(x, w) and out_dtype in (torch.bfloat16, torch.float32):
         out = torch.empty((x.shape[0], w.shape[0]), dtype=out_dtype, device=x.device)
         if isinstance(x, ScaledRows):
-            ops.gemm_packed(x.rows, packed, out, row_scale=x.row_scale)
+            ops.gemm_packed(x.rows, w.packed, out, row_scale=x.row_scale)
         else:
-            ops.gemm_packed(x, packed, out)
+            ops.gemm_packed(x, w.packed, out)
         return out
     x = as_rows(x)
     if w.dtype != x.dtype:
@@ -102,31 +116,37 @@ def linear(x, w, out_dtype, packed=None):
             raise TypeError(f"linear: activation {x.dtype} with weight {w.dtype}")
     out = torch.empty((x.shape[0], w.shape[0]), dtype=torch.float32 if x.dtype == torch.float32 else out_dtype,
                       device=x.device)
-    ops.gemm(x, w, out)
+    ops.gemm(x, w.data, out)
     return out if out.dtype == out_dtype else out.to(out_dtype)
 
 
-def linear_for_sum(x, w, packed=None):
+def product_slices(n_rows, w, dtype) -> int:
+    """Into how many slices of K the product of n_rows rows with w is cut for a reader that adds partial sums."""
+    if w.dtype != dtype or (w.packed is not None and w.shape[1] % 128):
+        return 1            # (in fragment order the tiles for many rows take a K that is a multiple of 128 only)
+    return ops.gemm_slices(n_rows, w.shape[0], w.shape[1], dtype)
+
+
+def linear_for_sum(x, w):
     """The product as float partial sums for a consumer that adds them up (the residual sum fused
     into the next norm): [S, M, N] when cutting K into S slices gives a small product more
     workgroups, else [M, N]."""
-    if _use_packed(x, packed):
+    w = _matrix(w)
+    if _use_packed(x, w):
         slices = ops.packed_slices(w.shape[0], w.shape[1])
         if slices <= 1:
-            return linear(x, w, torch.float32, packed)
+            return linear(x, w, torch.float32)
         out = torch.empty((slices, x.shape[0], w.shape[0]), dtype=torch.float32, device=x.device)
         if isinstance(x, ScaledRows):
-            ops.gemm_packed(x.rows, packed, out, row_scale=x.row_scale)
+            ops.gemm_packed(x.rows, w.packed, out, row_scale=x.row_scale)
         else:
-            ops.gemm_packed(x, packed, out)
+            ops.gemm_packed(x, w.packed, out)
         return out
     x = as_rows(x)
-    M, K = x.shape
-    N = w.shape[0]
-    slices = ops.gemm_slices(M, N, K, x.dtype) if w.dtype == x.dtype else 1
+    M = x.shape[0]
+    slices = product_slices(M, w, x.dtype)
     if slices <= 1:
         return linear(x, w, torch.float32)
-    out = torch.empty((slices, M, N), dtype=torch.float32, device=x.device)
-    ops.gemm(x, w, out)
+    out = torch.empty((slices, M, w.shape[0]), dtype=torch.float32, device=x.device)
+    ops.gemm(x, w.data, out)
     return out
-

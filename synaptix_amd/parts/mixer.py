@@ -15,7 +15,7 @@ import torch
 from ..kernels import ops
 from ..weights.source import TensorSpec
 from .base import Part, KvNeed
-from .linear import linear, linear_for_sum, deferred_product, as_rows, ScaledRows, packed_copy
+from .linear import Matrix, linear, linear_for_sum, product_slices, deferred_product, as_rows, ScaledRows
 from .position import Position, NoPosition
 
 
@@ -77,9 +77,8 @@ class GqaAttention(Mixer):
     def load(self, get):
         p = self.prefix
         # one product for q, k and v: rows of the three matrices one after another
-        self.w_qkv = torch.cat([get(p + "q_proj.weight"), get(p + "k_proj.weight"), get(p + "v_proj.weight")], 0)
-        self.w_o = get(p + "o_proj.weight")
-        self.p_qkv, self.p_o = packed_copy(self.w_qkv), packed_copy(self.w_o)   # in fragment order, for single tokens
+        self.w_qkv = Matrix(torch.cat([get(p + "q_proj.weight"), get(p + "k_proj.weight"), get(p + "v_proj.weight")], 0))
+        self.w_o = Matrix(get(p + "o_proj.weight"))
         if self.qk_norm_eps is not None:
             self.q_gain = get(p + "q_norm.weight")
             self.k_gain = get(p + "k_norm.weight").to(self.q_gain.dtype)
@@ -123,15 +122,15 @@ class GqaAttention(Mixer):
         if cap is not None and ctx.max_position >= cap:
             raise ValueError(f"position {ctx.max_position} is beyond the position encoding's capacity {cap}")
         # single tokens: partial sums over slices of K, which the attention kernel adds; prompts: the plain product
-        if self.p_qkv is not None and N <= ops.PACKED_MAX_ROWS and act == torch.bfloat16:
-            qkv = linear_for_sum(h, self.w_qkv, self.p_qkv)       # float partial sums [S, N, width]
+        if self.w_qkv.packed is not None and N <= ops.PACKED_MAX_ROWS and act == torch.bfloat16:
+            qkv = linear_for_sum(h, self.w_qkv)       # float partial sums [S, N, width]
             if qkv.dim() == 2:
                 qkv = qkv.unsqueeze(0)
         else:
             h = as_rows(h)
             # (every kernel behind it adds partial sums itself; ops.gemm_slices cuts where the product would
             # otherwise leave compute units without work: single tokens and prompts up to about 1,200 tokens)
-            sliced = ops.gemm_slices(N, self.w_qkv.shape[0], self.hidden, act) > 1
+            sliced = product_slices(N, self.w_qkv, act) > 1
             qkv = linear_for_sum(h, self.w_qkv) if sliced else linear(h, self.w_qkv, act)
         cos, sin = self.position.tables(h.device)
         table = ctx.page_table(cache.group)
@@ -144,7 +143,7 @@ class GqaAttention(Mixer):
                                             self.scale, window, nh, nkv, hd, self.q_gain, self.k_gain,
                                             self.qk_norm_eps or 0.0, cos, sin, write_kv=owner,
                                             gain_offset=self.qk_gain_offset, **terms, **merge)
-            return deferred_product(o, self.w_o, self.p_o)
+            return deferred_product(o, self.w_o)
         q = torch.empty((N, nh * hd), dtype=act, device=h.device)
         ops.qk_norm_rope_kv_write(qkv, q, cache.k_pages, cache.v_pages, table, ctx.tok_seq, ctx.tok_pos,
                                   self.q_gain, self.k_gain, self.qk_norm_eps or 0.0, cos, sin, nh, nkv, hd,
@@ -159,4 +158,4 @@ class GqaAttention(Mixer):
         else:
             ops.attention_prefill_bf16(q, cache.k_pages, cache.v_pages, table, ctx.seq_start, ctx.seq_past, o,
                                        self.scale, window, nh, nkv, hd, **terms)
-        return deferred_product(o, self.w_o, self.p_o)
+        return deferred_product(o, self.w_o)

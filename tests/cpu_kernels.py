@@ -18,8 +18,16 @@ PAGE = 64
 F32 = torch.float32
 
 
+def _rows(w):
+    """A weight in plain rows, whether it comes so or in fragment order (pack_weight: four dimensions)."""
+    if w.dim() == 4:
+        from synaptix_amd.kernels import ops
+        return ops.unpack_weight(w)
+    return w
+
+
 def embed(table, ids, resid):
-    resid.copy_(table[ids.long()].to(F32))
+    resid.copy_(_rows(table)[ids.long()].to(F32))
 
 
 def add_rmsnorm(resid, delta, gain, eps, out, rows=None, gain_offset=0.0):
@@ -51,6 +59,7 @@ def swiglu(gate_up, out, activation="silu"):
 
 
 def gemm(x, w, out, force_simt=False):
+    w = _rows(w)
     if out.dim() == 3:                      # partial sums over slices of K
         S, K = out.shape[0], x.shape[1]
         step = ((K + S - 1) // S + 127) // 128 * 128
@@ -65,6 +74,7 @@ PAIR = 16
 
 def gemm_swiglu(x, w_paired, out, activation="silu"):
     assert activation in ("silu", "swish")
+    w_paired = _rows(w_paired)
     N, K = w_paired.shape
     w = w_paired.view(N // (2 * PAIR), 2, PAIR, K)
     g = x.to(F32) @ w[:, 0].reshape(N // 2, K).to(F32).T

@@ -108,24 +108,23 @@ def test_a_head_size_without_a_kernel_is_refused_when_the_engine_is_made(tmp_pat
     assert eng.step([(s, [1, 2, 3])], want="last").shape == (1, cfg.vocab_size)
 
 
-def test_single_tokens_give_the_same_logits_with_and_without_packed_weight_copies():
-    """The copy of the weights in fragment order is a layout, not another model."""
-    from synaptix_amd.parts import keep_packed_copies
-    from helpers import random_tokens
-    toks = random_tokens(CONFIGS["A"]["vocab_size"], 12, 77)
-    got = []
-    for keep in (True, False):
-        keep_packed_copies(keep)
-        try:
-            eng = make_engine("A", "bfloat16", 256)
-        finally:
-            keep_packed_copies(True)
-        has = eng.model.blocks[0].mixer.p_o is not None
-        assert has == keep
-        s = eng.acquire()
-        eng.step([(s, toks[:9])], want=None)
-        got.append(torch.cat([eng.step([(s, [t])], want="last") for t in toks[9:]]))
-    assert float((got[0] - got[1]).abs().max()) <= 2e-2
+def test_every_weight_is_kept_once():
+    """A bf16 matrix whose sizes allow it lies in fragment order and nowhere else; the others in plain rows;
+    both are the matrix of the model's folder (the order is a layout, not another model)."""
+    from safetensors.torch import load_file
+    import os
+    eng = make_engine("A", "bfloat16", 256)
+    stored = load_file(os.path.join(model_folder("A"), "model.safetensors"))
+    mixer, ff = eng.model.blocks[0].mixer, eng.model.blocks[0].feed_forward
+    for m in (mixer.w_qkv, mixer.w_o, ff.w_gate_up, ff.w_down, eng.model.head.weight, eng.model.embedding.table):
+        assert (m.packed is None) != (m.plain is None)
+        N, K = m.shape
+        assert (m.packed is not None) == (N % 16 == 0 and K % 32 == 0)
+        assert m.nbytes() == N * K * 2
+    assert torch.equal(mixer.w_o.rows(), stored["model.layers.0.self_attn.o_proj.weight"])
+    assert torch.equal(eng.model.embedding.table.rows(), stored["model.embed_tokens.weight"])
+    if CONFIGS["A"].get("tie_word_embeddings"):
+        assert eng.model.head.weight is eng.model.embedding.table
 
 
 def test_generation_that_resumes_a_kept_prefix_equals_a_fresh_one():

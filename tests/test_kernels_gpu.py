@@ -446,6 +446,66 @@ def test_slices_fill_the_compute_units(ops):
         assert 1 <= s <= 8
 
 
+@pytest.mark.parametrize("M,N,K,S", [
+    (9, 48, 128, 1), (16, 4096, 4096, 1), (33, 208, 256, 1), (64, 6144, 4096, 1), (64, 144, 384, 3),
+    (100, 4112, 384, 1), (128, 208, 4096, 8), (130, 6144, 1024, 1), (200, 4096, 1024, 2), (256, 1008, 2560, 4),
+    (257, 528, 4096, 8), (300, 96, 128, 1), (512, 4096, 1024, 2), (700, 272, 640, 1),
+    (1700, 5120, 128, 1),               # the 256 x 160 tile
+    (2053, 528, 256, 1), (1000, 12304, 128, 1), (2048, 6144, 512, 1),   # the large tiles, ragged edges
+    (8, 70000 // 16 * 16, 256, 1), (20, 66000 // 16 * 16, 128, 1),      # few rows, very wide
+    (40, 80, 96, 1), (300, 48, 160, 1),                                   # K no multiple of 128: in blocks of 16 rows
+])
+def test_tiled_gemm_reads_weights_in_fragment_order(ops, M, N, K, S):
+    """The tiles for 9 rows and more over pack_weight(W): the same sums in the same order as over plain rows
+    (bit for bit where both run the same tile), for every tile shape, with ragged edges in M and N, and as
+    partial sums over slices of K."""
+    x, w = rnd((M, K), 16, BF16), rnd((N, K), 17, BF16)
+    wd = w.to(DEV)
+    wp = ops.pack_weight(wd)
+    assert wp is not None
+    want = (x.double() @ w.double().T).float()
+    atol = 1e-3 * math.sqrt(K)
+    for out_dtype in ((F32,) if S > 1 else (BF16, F32)):
+        shape = (S, M, N) if S > 1 else (M, N)
+        got = torch.full(shape, float("nan"), dtype=out_dtype, device=DEV)
+        ops.gemm(x.to(DEV), wp, got)
+        total = got.float().sum(0) if S > 1 else got
+        close(total, want, atol if out_dtype == F32 else atol + 0.02, 0 if out_dtype == F32 else 1e-2,
+              f"gemm over fragment order {M}x{N}x{K}")
+        if K % 128 == 0 and not (N >= 65536 and K % 256):   # (very wide and K no multiple of 256: plain rows take another tile)
+            plain = torch.full(shape, float("nan"), dtype=out_dtype, device=DEV)
+            ops.gemm(x.to(DEV), wd, plain)
+            assert torch.equal(plain, got), "the same tiles over both layouts must give the same bits"
+
+
+@pytest.mark.parametrize("M,I,K", [(9, 48, 128), (16, 2560, 4096), (33, 80, 128), (64, 1024, 512), (100, 176, 384),
+                                   (128, 12288, 4096), (192, 1040, 256), (256, 2560, 1024), (300, 112, 128),
+                                   (1000, 6160, 256), (2048, 1024, 512), (20, 40000, 128), (40, 48, 96)])
+def test_tiled_gated_gemm_reads_weights_in_fragment_order(ops, M, I, K):
+    x = rnd((M, K), 18, BF16)
+    wg, wu = rnd((I, K), 19, BF16, 0.5), rnd((I, K), 20, BF16, 0.5)
+    paired = ops.pair_rows(wg.to(DEV), wu.to(DEV))
+    wp = ops.pack_weight(paired)
+    g = x.double() @ wg.double().T
+    want = (g / (1 + torch.exp(-g)) * (x.double() @ wu.double().T)).float()
+    got = torch.full((M, I), float("nan"), dtype=BF16, device=DEV)
+    ops.gemm_swiglu(x.to(DEV), wp, got)
+    close(got, want, 0.03 + 2e-3 * math.sqrt(K), 2e-2, f"gated gemm over fragment order {M}x{I}x{K}")
+    if K % 128 == 0 and 2 * I < 65536:
+        plain = torch.empty((M, I), dtype=BF16, device=DEV)
+        ops.gemm_swiglu(x.to(DEV), paired, plain)
+        assert torch.equal(plain, got)
+
+
+def test_embedding_from_a_table_in_fragment_order(ops):
+    V, H = 1008, 4128
+    table = rnd((V, H), 21, BF16)
+    ids = torch.tensor([0, 15, 16, 17, V - 1, 500, 31], dtype=I32)
+    out = torch.full((ids.numel(), H), float("nan"), dtype=F32, device=DEV)
+    ops.embed(ops.pack_weight(table.to(DEV)), ids.to(DEV), out)
+    assert torch.equal(out.cpu(), table[ids.long()].to(F32))
+
+
 def test_gemm_bf16_paths_agree(ops):
     """The MFMA kernels and the plain kernel compute the same sums."""
     for M in (4, 40, 300):

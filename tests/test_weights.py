@@ -116,20 +116,22 @@ def test_load_hands_parts_their_tensors_in_kept_types():
     assert model.blocks[0].norm1.gain.dtype == torch.bfloat16
     att = model.blocks[1].mixer
     assert att.w_qkv.shape == ((4 + 2 * 2) * 16, 64) and att.w_qkv.dtype == torch.bfloat16
-    assert torch.equal(att.w_qkv[:64], tensors["model.layers.1.self_attn.q_proj.weight"])
-    assert torch.equal(att.w_qkv[64:96], tensors["model.layers.1.self_attn.k_proj.weight"])
+    assert att.w_qkv.packed is not None and att.w_qkv.plain is None            # kept once, in fragment order
+    assert torch.equal(att.w_qkv.rows()[:64], tensors["model.layers.1.self_attn.q_proj.weight"])
+    assert torch.equal(att.w_qkv.rows()[64:96], tensors["model.layers.1.self_attn.k_proj.weight"])
     assert model.head.weight is model.embedding.table        # tied: one buffer
     ff = model.blocks[0].feed_forward
     # bf16: rows of gate and up in turns of 16, for the product that applies the activation itself
     gate, up = tensors["model.layers.0.mlp.gate_proj.weight"], tensors["model.layers.0.mlp.up_proj.weight"]
     assert ff.paired and ff.w_gate_up.shape == (2 * 176, 64)
-    assert torch.equal(ff.w_gate_up[:16], gate[:16]) and torch.equal(ff.w_gate_up[16:32], up[:16])
-    assert torch.equal(ff.w_gate_up[-32:-16], gate[-16:]) and torch.equal(ff.w_gate_up[-16:], up[-16:])
+    gu = ff.w_gate_up.rows()
+    assert torch.equal(gu[:16], gate[:16]) and torch.equal(gu[16:32], up[:16])
+    assert torch.equal(gu[-32:-16], gate[-16:]) and torch.equal(gu[-16:], up[-16:])
     m32 = _model(TINY_A)
     load_weights(m32, DictSource(tensors), torch.float32, "cpu")
     assert m32.blocks[0].mixer.w_o.dtype == torch.float32
     ff32 = m32.blocks[0].feed_forward                          # 32-bit: one after the other
-    assert not ff32.paired and torch.equal(ff32.w_gate_up[176:], up.float())
+    assert not ff32.paired and ff32.w_gate_up.packed is None and torch.equal(ff32.w_gate_up.plain[176:], up.float())
 
 
 def test_random_weights_mode(tmp_path):
