@@ -809,21 +809,25 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
   constexpr int SO_LD = HD + 4;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / SYN_WAVE), lane = threadIdx.x % SYN_WAVE;
   char* stage = (char*)dec_lds + (size_t)wave * STAGE_BYTES;
+  // Without a work list the grid is (sequences, kv heads x chunks, splits); with one it is (kv heads x chunks, items),
+  // the kv heads of an item next to each other (they lie side by side in a page).
   int seq = blockIdx.x, split = blockIdx.z, n_splits = n_splits_all, first = blockIdx.x * n_splits_all, item_len = -1;
+  int group_of_heads = blockIdx.y, n_groups_of_heads = gridDim.y;
   if (work.items) {
-    const int4 item = work.items[blockIdx.x];
+    const int4 item = work.items[blockIdx.y];
+    group_of_heads = blockIdx.x, n_groups_of_heads = gridDim.x;
     seq = __builtin_amdgcn_readfirstlane(item.x), first = __builtin_amdgcn_readfirstlane(item.z);
     split = __builtin_amdgcn_readfirstlane(item.y) & 0xFFFF, n_splits = __builtin_amdgcn_readfirstlane(item.y) >> 16;
     item_len = __builtin_amdgcn_readfirstlane(item.w);   // (with the item: one trip to memory less than through seq_len)
     // (a spare item, or one that does not fit the launch: nothing is read or written for it)
-    const int n_seqs = gridDim.x / n_splits_all;
-    if (seq < 0 || seq >= n_seqs || n_splits < 1 || split >= n_splits || first < 0 || first + n_splits > (int)gridDim.x ||
+    const int n_seqs = gridDim.y / n_splits_all;
+    if (seq < 0 || seq >= n_seqs || n_splits < 1 || split >= n_splits || first < 0 || first + n_splits > (int)gridDim.y ||
         item_len < 1)
       return;
   }
   float* const partial = work.partial;
   const int g = nh / nkv, chunks = (g + 15) / 16;
-  const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+  const int kvh = group_of_heads / chunks, chunk = group_of_heads % chunks;
   const int kv_len = item_len > 0 ? item_len : seq_len[seq], pos = kv_len - 1;
   const int col = lane % 16;
   const int hg = chunk * 16 + col;  // head inside the group
@@ -1038,7 +1042,7 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
   __syncthreads();
   int* const is_last = (int*)sm;        // (the loop above has finished reading sm)
   if (threadIdx.x == 0) {
-    int* cnt = work.counters + (size_t)seq * gridDim.y + blockIdx.y;
+    int* cnt = work.counters + (size_t)seq * n_groups_of_heads + group_of_heads;
     const int before = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const int last = before == n_splits - 1;
     if (last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
@@ -1083,11 +1087,21 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
 
 // one wave a (sequence, head): lanes first share the splits' maxima and sums, then each takes output dims
 __global__ void __launch_bounds__(SYN_WAVE)
-attn_decode_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out, int n_splits, int nh) {
+// of_seq: with a work list, {first, splits} of each sequence (the table behind the list's items); else every
+// sequence has n_splits_all splits, the first at sequence * n_splits_all
+attn_decode_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out, int n_splits_all, int nh,
+                         const int2* __restrict__ of_seq) {
   const int row = blockIdx.x, lane = threadIdx.x;  // row = seq * nh + head
   const int seq = row / nh, head = row % nh;
   const size_t STEP = (size_t)nh * PART;           // from one split of the head to the next
-  const float* p = partial + ((size_t)seq * n_splits * nh + head) * PART;
+  int first = seq * n_splits_all, n_splits = n_splits_all;
+  if (of_seq) {
+    first = __builtin_amdgcn_readfirstlane(of_seq[seq].x), n_splits = __builtin_amdgcn_readfirstlane(of_seq[seq].y);
+    const int n_seqs = gridDim.x / nh;
+    // (one split has written the output itself; a table that does not fit the launch is not followed)
+    if (n_splits <= 1 || first < 0 || first + n_splits > n_seqs * n_splits_all) return;
+  }
+  const float* p = partial + ((size_t)first * nh + head) * PART;
   float wsum[(HD + SYN_WAVE - 1) / SYN_WAVE] = {};
   float l = 0.f;
   float m = -INFINITY;
@@ -1145,10 +1159,13 @@ static hipError_t raise_decode_lds() {
 }
 
 // workspace: n_seqs * nh * n_splits * (HD + 2) floats (unused with one split).
-// counters (may be null: then a second kernel merges the splits): n_seqs * kv heads * ceil(group / 16) ints, zero.
+// counters (may be null): n_seqs * kv heads * ceil(group / 16) ints, zero.  With them the splits are merged inside the
+// one launch where the grid is at most two workgroups a compute unit; where it is larger, and without them, a second
+// kernel merges (a workgroup that waits for its stores and counts itself in holds its place that much longer, which a
+// grid of several rounds pays in every round: 8 sequences of 32,000 tokens 9.3 ms a step against 9.1).
 // items (may be null: every sequence in n_splits splits): n_items x {sequence, split | splits of the sequence << 16,
 // first, length}, `first` + split < n_seqs * n_splits being the place of the split's partial results and length
-// what seq_len holds for the sequence; they need the counters.
+// what seq_len holds for the sequence; behind them n_seqs x {first, splits}, the same by sequence.
 static int launch_decode(const void* q, const QkvIntake* in, void* k_pages, void* v_pages, const int* page_table,
                          int table_stride, const int* seq_len, int n_seqs, void* out, float* workspace, int n_splits,
                          float scale, int window, int nh, int nkv, int hd, hipStream_t stream,
@@ -1159,10 +1176,9 @@ static int launch_decode(const void* q, const QkvIntake* in, void* k_pages, void
   SYN_CHECK(n_seqs > 0 && nh > 0 && nkv > 0 && n_splits > 0, "attention_decode: empty input");
   SYN_CHECK(nh % nkv == 0, "attention_decode: %d heads do not divide into %d kv heads", nh, nkv);
   const int chunks = (nh / nkv + 15) / 16;
-  SYN_CHECK(nkv * chunks <= 65535 && n_splits <= 65535, "attention_decode: grid too large");
-  SYN_CHECK(items == nullptr || (counters != nullptr && n_items == n_seqs * n_splits),
-            "attention_decode: a list of %d items for %d sequences x %d splits, counters %s", n_items, n_seqs, n_splits,
-            counters ? "given" : "missing");
+  SYN_CHECK(nkv * chunks <= 65535 && n_splits <= 65535 && n_items <= 65535, "attention_decode: grid too large");
+  SYN_CHECK(items == nullptr || n_items == n_seqs * n_splits,
+            "attention_decode: a list of %d items for %d sequences x %d splits", n_items, n_seqs, n_splits);
   // waves a workgroup: as many as the LDS for their states allows (up to 8), but no more than make
   // about 2,048 waves in all: at large batches four waves a workgroup are plenty
   const int cols_alloc = nh / nkv < 16 ? nh / nkv : 16;
@@ -1179,8 +1195,9 @@ static int launch_decode(const void* q, const QkvIntake* in, void* k_pages, void
   SYN_CHECK(lds <= LDS_MAX, "attention_decode: %zu bytes of LDS for %d heads a group", lds, nh / nkv);
   const hipError_t raised = raise_decode_lds();
   SYN_CHECK(raised == hipSuccess, "attention_decode: %zu bytes of LDS refused: %s", LDS_MAX, hipGetErrorString(raised));
-  const dim3 grid = items ? dim3(n_items, nkv * chunks, 1) : dim3(n_seqs, nkv * chunks, n_splits);
-  const DecodeWork work{workspace, counters, (const int4*)items};
+  const dim3 grid = items ? dim3(nkv * chunks, n_items, 1) : dim3(n_seqs, nkv * chunks, n_splits);
+  const bool merge_inside = counters != nullptr && (long)n_seqs * nkv * chunks * n_splits <= 2L * syn_compute_units();
+  const DecodeWork work{workspace, merge_inside ? counters : nullptr, (const int4*)items};
   if (in)
     attn_decode_split_kernel<true><<<grid, waves * SYN_WAVE, lds, stream>>>(
         nullptr, (bf16*)k_pages, (bf16*)v_pages, page_table, table_stride, seq_len, work, (bf16*)out, scale,
@@ -1190,8 +1207,9 @@ static int launch_decode(const void* q, const QkvIntake* in, void* k_pages, void
         (const bf16*)q, (bf16*)k_pages, (bf16*)v_pages, page_table, table_stride, seq_len, work, (bf16*)out,
         scale, window, nh, nkv, n_splits, cols_alloc, QkvIntake{}, terms);
   SYN_LAUNCH_CHECK("attention_decode_split");
-  if (n_splits > 1 && counters == nullptr) {
-    attn_decode_merge_kernel<<<n_seqs * nh, SYN_WAVE, 0, stream>>>(workspace, (bf16*)out, n_splits, nh);
+  if (n_splits > 1 && !merge_inside) {
+    attn_decode_merge_kernel<<<n_seqs * nh, SYN_WAVE, 0, stream>>>(workspace, (bf16*)out, n_splits, nh,
+                                                                   items ? (const int2*)(items + 4L * n_items) : nullptr);
     SYN_LAUNCH_CHECK("attention_decode_merge");
   }
   return 0;

@@ -70,6 +70,22 @@ static inline hipError_t once_per_device(OncePerDevice& once, F&& step) {
   return e;
 }
 
+// Compute units of the current device (256 on an MI355X), asked once a device: what the hosts' rules for tiles and
+// splits fill.  (The Python rules ask the same number: kernels/ops.py, compute_units.)
+static inline int syn_compute_units() {
+  static int of_device[SYN_MAX_DEVICES];
+  static OncePerDevice once;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= SYN_MAX_DEVICES) return 256;
+  const hipError_t e = once_per_device(once, [&] {
+    int n = 0;
+    const hipError_t r = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    of_device[dev] = (r == hipSuccess && n > 0) ? n : 256;
+    return hipSuccess;
+  });
+  return e == hipSuccess ? of_device[dev] : 256;
+}
+
 // ---- conversions ----
 template <typename T> __device__ __forceinline__ float to_f32(T v);
 template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }

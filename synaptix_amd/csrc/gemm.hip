@@ -985,22 +985,6 @@ template <bool PAIRED>
 static int launch_large(const bf16* x, Weight w, void* out, Epilogue ep, int M, int N, int K,
                         hipStream_t stream, int slices = 1);
 
-// Compute units of the current device (256 on an MI355X), asked once a device: what the rules for tiles fill.
-// The host's rules for slices of K ask the same number (kernels/ops.py: compute_units).
-static int compute_units() {
-  static int of_device[SYN_MAX_DEVICES];
-  static OncePerDevice once;
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= SYN_MAX_DEVICES) return 256;
-  const hipError_t e = once_per_device(once, [&] {
-    int n = 0;
-    const hipError_t r = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
-    of_device[dev] = (r == hipSuccess && n > 0) ? n : 256;
-    return hipSuccess;
-  });
-  return e == hipSuccess ? of_device[dev] : 256;
-}
-
 // Which of the large tiles for M > 64: 0 = 256 x 256, 1 = 256 x 192 (one workgroup of four waves a compute
 // unit; a fifth less efficient), 2 = 128 x 128 (two workgroups a compute unit, about as much less efficient),
 // 3 = 256 x 160 (four waves of 64 x 160; for N = 5120, which it cuts into 32 where 256 x 192 makes 27).
@@ -1012,7 +996,7 @@ static int compute_units() {
 static int pick_large_tile(int M, int N) {
   auto rounds = [](long tiles, long slots) { return (tiles + slots - 1) / slots; };
   auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-  const long cus = compute_units();
+  const long cus = syn_compute_units();
   const double cost[4] = {(double)rounds(tiles(256, 256), cus) * 256 * 256,
                           (double)rounds(tiles(256, 192), cus) * 256 * 192 * 1.2,
                           (double)rounds(tiles(128, 128), 2 * cus) * 2 * 128 * 128 * 1.2,
@@ -1085,7 +1069,7 @@ SYN_EXPORT int syn_gemm(const void* x, const void* w, void* out, int dtype, int 
   const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
   // (cut along K the tiles are 128 x 128 up to 256 rows and 256 x 128 beyond)
   const long tiles_cut = (long)(M <= 256 ? (M + 127) / 128 : (M + 255) / 256) * ((N + 127) / 128);
-  const bool few_large_tiles = M > 64 && M <= 512 && K % 128 == 0 && (slices > 1 ? tiles_cut : tiles128) * slices <= compute_units();
+  const bool few_large_tiles = M > 64 && M <= 512 && K % 128 == 0 && (slices > 1 ? tiles_cut : tiles128) * slices <= syn_compute_units();
   int rc = 0;
   if (M == 1 && slices == 1 && !w_packed) {
     // one row: fragments of W straight from memory, K split over the waves

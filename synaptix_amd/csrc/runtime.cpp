@@ -508,8 +508,10 @@ RT_API int syn_step_fill_padded(void* h, int B, const int* sids, const long* cou
 // {sequence, split | splits of the sequence << 16, first, the sequence's length}, where `first` + split is
 // the place of the split's partial result.  Every sequence gets one split; the others go one by one to the sequence whose splits
 // are longest, while a split keeps at least MIN_UNITS units of 32 keys (a window bounds the keys that
-// count); sequences of one length get equal shares.  The items lie sequence by sequence, the longest pieces
-// first, spare items {-1, 0, 0, 0} last.
+// count); sequences of one length get equal shares.  The items lie in rounds (every sequence's first split, then
+// the second of those that have one, ...), in each round the longest pieces first; spare items {-1, 0, 0, 0} last.
+// Behind the items lie rows x {first, splits}, the same by sequence, for a kernel that merges the splits afterwards:
+// `items` has room for 4 * rows * n_splits + 2 * rows ints.
 RT_API int syn_decode_items(const int* seq_len, int rows, int n_splits, long window, int* items) {
   if (rows <= 0 || n_splits <= 0) return fail(MISUSE, "a work list for %d rows x %d splits", rows, n_splits);
   constexpr long UNIT = 32, MIN_UNITS = 8;
@@ -541,18 +543,29 @@ RT_API int syn_decode_items(const int* seq_len, int rows, int n_splits, long win
   for (int i = 0; i < rows; ++i) order[i] = i;
   auto piece = [&](int i) { return (units[i] + splits[i] - 1) / splits[i]; };
   std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return piece(a) > piece(b); });
+  // the places of the partial results: a sequence's splits side by side; the items themselves in rounds (split 0 of
+  // every sequence, then split 1 of those that have one, ...), so that the workgroups that run at one time belong
+  // to many sequences, as they do when every sequence has the same number of splits
+  std::vector<long> first(rows);
   long at = 0;
+  int most = 1;
   for (int i : order) {
-    const long first = at;
-    for (int sp = 0; sp < splits[i]; ++sp, ++at) {
-      int* it = items + 4 * at;
-      it[0] = i, it[1] = sp | (splits[i] << 16), it[2] = (int)first, it[3] = seq_len[i];
-    }
+    first[i] = at;
+    at += splits[i];
+    most = std::max(most, splits[i]);
   }
+  at = 0;
+  for (int sp = 0; sp < most; ++sp)
+    for (int i : order) {
+      if (sp >= splits[i]) continue;
+      int* it = items + 4 * at++;
+      it[0] = i, it[1] = sp | (splits[i] << 16), it[2] = (int)first[i], it[3] = seq_len[i];
+    }
   for (; at < T; ++at) {
     int* it = items + 4 * at;
     it[0] = -1, it[1] = 0, it[2] = 0, it[3] = 0;
   }
+  for (int i = 0; i < rows; ++i) items[4 * T + 2 * i] = (int)first[i], items[4 * T + 2 * i + 1] = splits[i];
   return OK;
 }
 
@@ -560,7 +573,7 @@ RT_API int syn_decode_items(const int* seq_len, int rows, int n_splits, long win
 // padding: token 0 at position 0 against a spare page that no sequence owns.  After the integer
 // tables lie 2 * rows floats: temperatures and uniform numbers (0 where none are given); after
 // them, for each group with item_splits[g] > 0 (item_splits may be null), the work list of the
-// group's attention: rows * item_splits[g] items of four ints (syn_decode_items).
+// group's attention: rows * item_splits[g] items of four ints and rows pairs (syn_decode_items).
 RT_API int syn_decode_fill(void* h, int rows, int B, const int* sids, const int* tokens, int n_groups,
                            const int* widths, const int* spare_pages, const float* temps, const float* uniforms,
                            const int* item_splits, int* host) {
@@ -600,7 +613,7 @@ RT_API int syn_decode_fill(void* h, int rows, int B, const int* sids, const int*
     if (item_splits[g] <= 0) continue;
     const int rc = syn_decode_items(host + l.seq_len, rows, item_splits[g], c->windows[g], items);
     if (rc) return rc;
-    items += 4L * rows * item_splits[g];
+    items += 4L * rows * item_splits[g] + 2L * rows;
   }
   return OK;
 }

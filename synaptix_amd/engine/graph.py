@@ -78,8 +78,8 @@ class DecodeRunner:
         self.item_splits = [ops.decode_splits(rows, g.need.kv_heads, w) if engine.dtype == torch.bfloat16 else 0
                             for g, w in zip(groups, self.widths)]
         self.item_splits = [s if s > 1 else 0 for s in self.item_splits]
-        n_items = [rows * s for s in self.item_splits]
-        self.total = n_int + 2 * rows + 4 * sum(n_items)       # + temperatures and uniforms as float bits + items
+        n_items = [4 * rows * s + 2 * rows if s else 0 for s in self.item_splits]       # ints of each list
+        self.total = n_int + 2 * rows + sum(n_items)           # + temperatures and uniforms as float bits + work lists
         dev = engine.device
         self.dev = torch.zeros(self.total, dtype=torch.int32, device=dev)
         self.host = [torch.zeros(self.total, dtype=torch.int32, pin_memory=True) for _ in range(2)]
@@ -89,8 +89,8 @@ class DecodeRunner:
         self.uniforms = self.dev[n_int + rows:n_int + 2 * rows].view(torch.float32)
         self.items, at = [], n_int + 2 * rows
         for n in n_items:
-            self.items.append(self.dev[at:at + 4 * n].view(n, 4) if n else None)
-            at += 4 * n
+            self.items.append(self.dev[at:at + n] if n else None)
+            at += n
         self.out_tokens = torch.zeros(rows, dtype=torch.int32, device=dev)
         self.logits = None
         self.graph = None

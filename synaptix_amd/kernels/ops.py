@@ -599,22 +599,20 @@ def decode_splits(n_seqs, n_kv_heads, max_pages):
 
 
 def _decode_work(name, counters, items, B, n_splits, n_heads, n_kv_heads):
-    """The optional arguments of the decode kernels that put the merge of the splits into the one
-    launch.  counters: int32, at least B * kv heads * ceil(group / 16), zero (the kernel leaves them
-    zero); items: int32 [B * n_splits, 4], the work list that hands longer sequences more splits
-    (runtime.decode_items lays it out), needs counters."""
-    if counters is None:
-        if items is not None:
-            raise KernelError(f"{name}: a list of items needs counters")
-        return None, None, 0
-    chunks = -(-(n_heads // n_kv_heads) // 16)
-    _need(counters, f"{name}.counters", _I32)
-    if counters.numel() < B * n_kv_heads * chunks:
-        raise KernelError(f"{name}: {counters.numel()} counters for {B} sequences x {n_kv_heads * chunks}")
-    if items is None:
-        return _ptr(counters), None, 0
-    _need(items, f"{name}.items", _I32, (B * n_splits, 4))
-    return _ptr(counters), _ptr(items), B * n_splits
+    """The optional arguments of the decode kernels.  counters: int32, at least B * kv heads * ceil(group / 16),
+    zero (the kernel leaves them zero): with them the splits are merged inside the one launch where its grid is
+    small enough for that to pay.  items: int32 [4 * B * n_splits + 2 * B], the work list that hands longer
+    sequences more splits (runtime.decode_items lays it out)."""
+    n_items = 0
+    if items is not None:
+        _need(items, f"{name}.items", _I32, (4 * B * n_splits + 2 * B,))
+        n_items = B * n_splits
+    if counters is not None:
+        chunks = -(-(n_heads // n_kv_heads) // 16)
+        _need(counters, f"{name}.counters", _I32)
+        if counters.numel() < B * n_kv_heads * chunks:
+            raise KernelError(f"{name}: {counters.numel()} counters for {B} sequences x {n_kv_heads * chunks}")
+    return _ptr(counters), _ptr(items), n_items
 
 
 def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspace, n_splits, scale, window,
@@ -634,7 +632,7 @@ def attention_decode_bf16(q, k_pages, v_pages, page_table, seq_len, out, workspa
     _need(workspace, "attention_decode.workspace", _F32)
     if workspace.numel() < B * nh * n_splits * (hd + 2):
         raise KernelError(f"attention_decode: workspace of {workspace.numel()} floats is too small")
-    if slopes is None and not softcap and counters is None:
+    if slopes is None and not softcap and counters is None and items is None:
         _call(_attn_lib(hd), "syn_attention_decode_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
               page_table.shape[1], _ptr(seq_len), B, _ptr(out), _ptr(workspace), int(n_splits), ctypes.c_float(scale),
               int(window or 0), nh, nkv, hd, _stream())

@@ -87,11 +87,12 @@ def longs(values):
 
 
 def decode_items(seq_len, n_splits: int, window=None) -> list:
-    """The work list of a decode step's attention as the runtime lays it out and the kernel reads it:
-    for sequences of the lengths `seq_len`, len(seq_len) * n_splits items (sequence, split | splits of
-    the sequence << 16, first, the sequence's length); spare items have sequence -1."""
+    """The work list of a decode step's attention as the runtime lays it out and the kernel reads it,
+    as a flat list of ints: for sequences of the lengths `seq_len`, len(seq_len) * n_splits items of
+    four (sequence, split | splits of the sequence << 16, first, the sequence's length; spare items have
+    sequence -1), then (first, splits) of every sequence."""
     rows = len(seq_len)
-    out = (C.c_int * (4 * rows * n_splits))()
+    out = (C.c_int * (4 * rows * n_splits + 2 * rows))()
     check(lib().syn_decode_items(ints([int(x) for x in seq_len]), rows, int(n_splits),
                                  -1 if window is None else int(window), out))
-    return [tuple(out[4 * i:4 * i + 4]) for i in range(rows * n_splits)]
+    return list(out)

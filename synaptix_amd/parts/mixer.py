@@ -109,7 +109,7 @@ class GqaAttention(Mixer):
         if splits > 1:
             chunks = -(-(self.nh // self.nkv) // 16)
             items = ctx.decode_items(cache.group)
-            if items is not None and items.shape[0] != n_seqs * splits:
+            if items is not None and items.numel() != 4 * n_seqs * splits + 2 * n_seqs:
                 items = None
             merge = dict(counters=ctx.counters("attention_decode_arrivals", n_seqs * self.nkv * chunks), items=items)
         return work, splits, merge

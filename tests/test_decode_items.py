@@ -10,11 +10,18 @@ UNIT, MIN_UNITS = 32, 8
 
 
 def _unpacked(lengths, n_splits, window=None):
-    """(sequence, split, splits of the sequence, first) of every item; the length that an item carries is checked here."""
+    """(sequence, split, splits of the sequence, first) of every item; the length that an item carries and the
+    table by sequence behind the items are checked here."""
+    flat = rt.decode_items(lengths, n_splits, window)
+    T, rows = len(lengths) * n_splits, len(lengths)
+    assert len(flat) == 4 * T + 2 * rows
     out = []
-    for seq, split_and_n, first, length in rt.decode_items(lengths, n_splits, window):
+    for at in range(T):
+        seq, split_and_n, first, length = flat[4 * at:4 * at + 4]
         assert seq < 0 or length == lengths[seq]
         out.append((seq, split_and_n & 0xFFFF, split_and_n >> 16, first))
+        if seq >= 0:
+            assert flat[4 * T + 2 * seq:4 * T + 2 * seq + 2] == [first, split_and_n >> 16]   # the same by sequence
     return out
 
 
@@ -37,7 +44,7 @@ def _check(lengths, n_splits, window=None):
         n = rows[0][2]
         assert [r[1] for r in rows] == list(range(n)) and all(r[2] == n for r in rows)   # each split once, in order
         first = rows[0][3]
-        assert all(r[3] == first for r in rows) and first == rows[0][0]                  # partial results lie where the items lie
+        assert all(r[3] == first for r in rows) and first >= 0                           # one place for the sequence's partial results
         places = set(range(first, first + n))
         assert not (places & taken) and max(places) < len(items)
         taken |= places
@@ -61,10 +68,15 @@ def test_longer_sequences_get_more_splits_and_lie_first():
     items, n = _check(lengths, 4)
     assert n[1] >= n[6] >= n[4] >= n[2] >= n[0] == 1
     assert sum(n.values()) <= 32 and n[1] > 4                 # what short sequences cannot use goes to long ones
-    pieces = [-(-(-(-lengths[s] // UNIT)) // k) for s, _, k, _ in items if s >= 0]
-    assert pieces == sorted(pieces, reverse=True)
+    # in rounds: every sequence's first split, then the second of those that have one, ...; in a round the longest pieces first
+    rounds = [sp for s, sp, _, _ in items if s >= 0]
+    assert rounds == sorted(rounds)
+    for r in set(rounds):
+        pieces = [-(-(-(-lengths[s] // UNIT)) // k) for s, sp, k, _ in items if s >= 0 and sp == r]
+        assert pieces == sorted(pieces, reverse=True)
+    pieces = [-(-(-(-lengths[s] // UNIT)) // k) for s, sp, k, _ in items if s >= 0]
     # the longest piece of the uneven batch is shorter than with equal shares
-    assert pieces[0] < -(-(-(-4000 // UNIT)) // 4)
+    assert max(pieces) < -(-(-(-4000 // UNIT)) // 4)
 
 
 def test_a_window_bounds_the_keys_that_count():

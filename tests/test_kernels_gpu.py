@@ -735,7 +735,8 @@ def merged_in_kernel(run, two_kernels, want, lens, splits, window, nh, nkv):
     counters = torch.zeros(len(lens) * nkv * chunks, dtype=I32, device=DEV)
     items = torch.tensor(rt.decode_items(lens, splits, window or None), dtype=I32, device=DEV)
     for what, kw in (("merged in the kernel", dict(counters=counters)),
-                     ("with a work list", dict(counters=counters, items=items))):
+                     ("with a work list", dict(counters=counters, items=items)),
+                     ("with a work list, merged by the second kernel", dict(items=items))):
         outs = []
         for _ in range(2):
             got = torch.full_like(two_kernels, float("nan"))
@@ -765,6 +766,7 @@ def merged_in_kernel(run, two_kernels, want, lens, splits, window, nh, nkv):
     (32, 8, 128, [7000, 40], 0, 32),            # long contexts: 32 and 64 splits, most of them empty for the short sequence
     (8, 2, 64, [6500, 130, 7000], 0, 64),
     (4, 1, 32, [4100], 0, 24),
+    (32, 8, 128, [3000, 500, 2600, 100, 1500], 0, 16),   # 640 workgroups: more than two a compute unit, merged by the second kernel
 ])
 def test_attention_decode_bf16(ops, nh, nkv, hd, lens, window, splits):
     B = len(lens)

@@ -61,7 +61,7 @@ def test_decode_tables_pad_with_a_spare_page():
     rows, widths, spare = 4, [4, 4], [12, 12]
     lay = StepLayout(rows, rows, rows, widths)
     item_splits = [0, 3]                       # the second group keeps a work list for its attention: 4 x 3 items
-    host = np.zeros(lay.total + 2 * rows + 4 * rows * 3, dtype=np.int32)
+    host = np.zeros(lay.total + 2 * rows + 4 * rows * 3 + 2 * rows, dtype=np.int32)
     temps, unis = (C.c_float * 2)(0.5, 0.0), (C.c_float * 2)(0.25, 0.75)
     rt.check(rt.lib().syn_decode_fill(c._h, rows, 2, rt.ints([a, b]), rt.ints([9, 8]), 2, rt.ints(widths),
                                       rt.ints(spare), temps, unis, rt.ints(item_splits), host.ctypes.data))
@@ -80,10 +80,12 @@ def test_decode_tables_pad_with_a_spare_page():
     assert full[0, 3] == 12 and full[1, 1:].tolist() == [12, 12, 12] and (full[2:] == 12).all()
     f = host[lay.total:lay.total + 2 * rows].view(np.float32)
     assert f.tolist() == [0.5, 0.0, 0.0, 0.0, 0.25, 0.75, 0.0, 0.0]
-    items = host[lay.total + 2 * rows:].reshape(12, 4).tolist()
-    assert [tuple(i) for i in items] == rt.decode_items([131, 6, 1, 1], 3)      # from the lengths that the step has
+    flat = host[lay.total + 2 * rows:].tolist()
+    assert flat == rt.decode_items([131, 6, 1, 1], 3)                          # from the lengths that the step has
+    items = [flat[4 * i:4 * i + 4] for i in range(12)]
     assert sorted(i[0] for i in items[:4]) == [0, 1, 2, 3] and all(i[0] == -1 for i in items[4:])   # too short to split
     assert all(i[1] == 1 << 16 for i in items[:4]) and sorted(i[3] for i in items[:4]) == [1, 1, 6, 131]
+    assert flat[48:] == [x for i in range(4) for x in (next(it[2] for it in items if it[0] == i), 1)]   # the same by sequence
     with pytest.raises(CacheError, match="width"):
         rt.check(rt.lib().syn_decode_fill(c._h, rows, 2, rt.ints([a, b]), rt.ints([9, 8]), 2, rt.ints([2, 4]),
                                           rt.ints(spare), None, None, None, host.ctypes.data))
