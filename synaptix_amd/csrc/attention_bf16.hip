@@ -1055,31 +1055,35 @@ attn_decode_split_kernel(const bf16* __restrict__ q, bf16* __restrict__ k_pages,
     const int head = kvh * g + chunk * 16 + c;
     const float* p = partial + ((size_t)first * nh + head) * PART;
     const size_t step = (size_t)nh * PART;   // from one split of the head to the next
-    float m = -INFINITY;
-    for (int s0 = 0; s0 < n_splits; s0 += 8) {
-      float ms[8];
+    // all of up to 16 splits' values are asked for together (one trip to memory); further splits join a running
+    // state, in their order
+    constexpr int BATCH = 16;
+    float m = -INFINITY, acc = 0.f, lsum = 0.f;
+    for (int s0 = 0; s0 < n_splits; s0 += BATCH) {
+      float ms[BATCH], ls[BATCH], vs[BATCH];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) ms[u] = s0 + u < n_splits ? load_through(p + (s0 + u) * step) : -INFINITY;
-#pragma unroll
-      for (int u = 0; u < 8; ++u) m = fmaxf(m, ms[u]);
-    }
-    float acc = 0.f, lsum = 0.f;
-    for (int s0 = 0; s0 < n_splits; s0 += 8) {   // eight splits' values in flight together, added in their order
-      float ms[8], ls[8], vs[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
+      for (int u = 0; u < BATCH; ++u) {
         const bool on = s0 + u < n_splits;
-        ms[u] = on ? load_through(p + (s0 + u) * step) : -INFINITY;
-        ls[u] = on ? load_through(p + (s0 + u) * step + 1) : 0.f;
-        vs[u] = on ? load_through(p + (s0 + u) * step + 2 + d) : 0.f;
+        const float* ps = p + (size_t)min(s0 + u, n_splits - 1) * step;
+        ms[u] = load_through(ps);
+        ls[u] = load_through(ps + 1);
+        vs[u] = load_through(ps + 2 + d);
+        if (!on) ms[u] = -INFINITY;
       }
+      float m_new = m;
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        if (ms[u] == -INFINITY) continue;   // a split that had no keys weighs nothing and may hold anything
-        const float f = __expf(ms[u] - m);
+      for (int u = 0; u < BATCH; ++u) m_new = fmaxf(m_new, ms[u]);
+      if (m_new == -INFINITY) continue;        // (no split of this batch had keys)
+      const float keep = m == -INFINITY ? 0.f : __expf(m - m_new);
+      acc *= keep, lsum *= keep;
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u) {
+        if (ms[u] == -INFINITY) continue;       // a split that had no keys weighs nothing and may hold anything
+        const float f = __expf(ms[u] - m_new);
         acc += f * vs[u];
         lsum += f * ls[u];
       }
+      m = m_new;
     }
     out[((size_t)seq * nh + head) * HD + d] = (bf16)(acc / lsum);
   }
