@@ -60,9 +60,10 @@ class Engine:
         self._runners = {}
         from ..parts.base import StateNeed
         # a captured step is run more than once while it is recorded: only steps that write the
-        # same values again may be captured, which a mixer with a running state is not
+        # same values again may be captured, which a mixer with a running state is not; and every part has
+        # to say of itself that it only launches kernels (Part.capturable)
         self.has_states = any(isinstance(n, StateNeed) for n in model.cache_needs())
-        self.graph_ok = not self.has_states
+        self.graph_ok = not self.has_states and bool(getattr(model, "capturable", lambda: False)())
         self.prompt_graphs = True        # short prompt steps are replayed from graphs (see _prompt_runner)
 
     # ------------------------------------------------------------------ construction

@@ -31,6 +31,7 @@ class LayerRun:
 
 class TokenEmbedding(Part):
     """x[n, :] = E[id[n], :] (crates/synaptix-ops/src/embed/token_embed.rs:4-15)."""
+    capturable = True
 
     def __init__(self, name: str, vocab: int, hidden: int):
         self.name, self.vocab, self.hidden = name, vocab, hidden
@@ -51,6 +52,7 @@ class TokenEmbedding(Part):
 class OutputHead(Part):
     """logits = h . W^T in float; tied: W is the embedding table
     (crates/synaptix-models/llm/common/src/model.rs:757-764)."""
+    capturable = True
 
     def __init__(self, name: str, vocab: int, hidden: int, tied_to: TokenEmbedding | None = None):
         self.name, self.vocab, self.hidden, self.tied_to = name, vocab, hidden, tied_to
@@ -115,6 +117,10 @@ class DecoderModel:
         """Every part is asked whether its kernels take its sizes in `dtype`."""
         for p in self._parts():
             p.check(dtype)
+
+    def capturable(self) -> bool:
+        """Whether a step of this model may be captured into a graph: every part says so of itself."""
+        return all(getattr(p, "capturable", False) for p in self._parts())
 
     # ------------------------------------------------------------------ cache
     def cache_needs(self) -> list:

@@ -16,6 +16,12 @@ import torch
 class Part:
     """Base of norms, position encodings, mixers, feed-forwards and blocks."""
 
+    # True: the part's forward only launches kernels on the current stream (no wait for the device, no shape that
+    # depends on device data) and writes the same values when it is run again, so that a step that contains it
+    # may be captured into a graph and replayed.  False (the default, for parts from elsewhere): the steps of a
+    # model that contains it are launched one by one.
+    capturable = False
+
     def tensor_specs(self) -> dict:
         """name -> TensorSpec of every tensor this part reads from the weight source."""
         return {}

@@ -37,6 +37,10 @@ class PreNormBlock(Block):
     def _parts(self):
         return (self.norm1, self.mixer, self.norm2, self.feed_forward)
 
+    @property
+    def capturable(self):
+        return all(getattr(p, "capturable", False) for p in self._parts())
+
     def tensor_specs(self):
         specs = {}
         for p in self._parts():

@@ -24,6 +24,7 @@ class FeedForward(Part):
 
 class GatedMlp(FeedForward):
     takes_scaled_rows = True
+    capturable = True
 
     def __init__(self, prefix: str, hidden: int, intermediate: int, activation: str = "silu"):
         try:

@@ -42,6 +42,7 @@ class Mixer(Part):
 
 class GqaAttention(Mixer):
     takes_scaled_rows = True
+    capturable = True
 
     def __init__(self, prefix: str, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, *,
                  position: Position | None = None, qk_norm_eps: float | None = None, scale: float | None = None,

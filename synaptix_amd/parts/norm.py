@@ -17,6 +17,7 @@ from .linear import DeferredProduct, ScaledRows
 
 
 class RmsNorm(Part):
+    capturable = True
     takes_deferred_product = True     # add_apply accepts a parts.linear.DeferredProduct as delta and may return ScaledRows
 
     def __init__(self, name: str, dim: int, eps: float, gain_offset: float = 0.0):
