@@ -725,10 +725,12 @@ def test_attention_with_terms_on_the_scores(ops, nh, nkv, hd, past, new, window,
             close(outd, want[last], 2e-2, 1e-2, what=f"attention decode bf16 with terms, {splits} splits")
 
 
-def merged_in_kernel(run, two_kernels, want, lens, splits, window, nh, nkv):
+def merged_in_kernel(run, two_kernels, want, lens, splits, window, nh, nkv, work):
     """The same call with the merge of the splits inside the one launch, by the workgroup that finishes last:
     first with every sequence in `splits` splits, then with the host's work list, which gives long sequences
-    more of them; twice each with the same counters, which the kernel has to leave at zero."""
+    more of them; twice each with the same counters, which the kernel has to leave at zero.  Before every run
+    the partial results' memory is filled with NaN by another kernel: a workgroup that merged what an earlier
+    launch left in its cache, and not what the other workgroups of this launch have written, would show it."""
     if splits == 1:
         return
     chunks = -(-(nh // nkv) // 16)
@@ -740,6 +742,7 @@ def merged_in_kernel(run, two_kernels, want, lens, splits, window, nh, nkv):
         outs = []
         for _ in range(2):
             got = torch.full_like(two_kernels, float("nan"))
+            work.fill_(float("nan"))
             run(got, **kw)
             close(got, want, 2e-2, 1e-2, what=f"decode attention {what}")
             outs.append(got.cpu())
@@ -789,7 +792,45 @@ def test_attention_decode_bf16(ops, nh, nkv, hd, lens, window, splits):
     close(out, want, 2e-2, 1e-2, what="attention decode bf16")
     merged_in_kernel(lambda out2, **kw: ops.attention_decode_bf16(
         d(q), d(k), dv(v), d(table), d(torch.tensor(lens, dtype=I32)), out2, work, splits, scale, window, nh, nkv, hd, **kw),
-        out, want, lens, splits, window, nh, nkv)
+        out, want, lens, splits, window, nh, nkv, work)
+
+
+@pytest.mark.parametrize("lens,splits", [([2061] * 8, 4), ([2061], 16), ([3908, 457, 1200, 2500], 8)])
+def test_merge_inside_the_launch_reads_what_this_launch_wrote(ops, lens, splits):
+    """The workgroup that merges the splits reads partial results that workgroups on other XCDs, each with a
+    second-level cache of its own, wrote within the same launch.  200 launches at a decode step's shapes, the
+    memory of the partial results filled with NaN by another kernel before each and the keys of other launches
+    read in between: every output equals the first, none is NaN."""
+    nh, nkv, hd = 32, 8, 128
+    B = len(lens)
+    width = max((T + 63) // 64 for T in lens) + 1
+    table = shuffled_table(B, width, 6)
+    k, v = make_cache(B * width, nkv, hd, BF16, 70)
+    fill_sequences(k, v, table, lens, nkv, hd, BF16, 71)
+    q = rnd((B, nh * hd), 72, BF16)
+    d = lambda t: t.to(DEV)
+    qd, kd, vd, td, ld = d(q), d(k), dv(v), d(table), d(torch.tensor(lens, dtype=I32))
+    work = torch.empty(B * nh * splits * (hd + 2), dtype=F32, device=DEV)
+    counters = torch.zeros(B * nkv, dtype=I32, device=DEV)
+    items = torch.tensor(rt.decode_items(lens, splits), dtype=I32, device=DEV)
+    other = torch.randn(64 << 20, device=DEV)          # 256 MB that a kernel in between reads
+    first = None
+    for i in range(200):
+        out = torch.full((B, nh * hd), float("nan"), dtype=BF16, device=DEV)
+        work.fill_(float("nan"))
+        if i % 3 == 0:
+            other.sum()
+        ops.attention_decode_bf16(qd, kd, vd, td, ld, out, work, splits, 1 / math.sqrt(hd), 0, nh, nkv, hd,
+                                  counters=counters, items=items if i % 2 else None)
+        if first is None:
+            first = {}
+        key = i % 2
+        if key not in first:
+            assert torch.isfinite(out.float()).all()
+            first[key] = out.clone()
+        else:
+            assert torch.equal(out, first[key]), f"launch {i} differs from the first of its kind"
+    assert int(counters.abs().sum()) == 0
 
 
 @pytest.mark.parametrize("nh,nkv,hd,rot,norm,lens,window,splits,parts,own", [
@@ -841,7 +882,7 @@ def test_attention_decode_with_qkv_intake(ops, nh, nkv, hd, rot, norm, lens, win
     close(out, want, 2e-2, 1e-2, what="decode attention with q/k/v intake")
     merged_in_kernel(lambda out2, **kw: ops.attention_decode_fused_bf16(
         d(qkv), kd, vd, d(table), d(seq_len), out2, work, splits, scale, window, nh, nkv, hd, d(qg), d(kg), 1e-5, d(cos),
-        d(sin), write_kv=own, **kw), out, want, lens, splits, window, nh, nkv)
+        d(sin), write_kv=own, **kw), out, want, lens, splits, window, nh, nkv, work)
     # the cache afterwards: the new rows written (or nothing touched)
     close(kd, k_ref.float(), 2e-2, 1e-2, what="k pages after the step")
     close(hv(vd), v_ref.float(), 2e-2, 1e-2, what="v pages after the step")
