@@ -1200,8 +1200,9 @@ SYN_EXPORT int syn_gemm_packed_norm(const void* x, const void* wp, void* out, in
   else if (paired) launch_packed<2, 8, 4, true>(xb, wb, out, ep, M, N, K, stream, 1, rn);
   else if (N <= 8192) launch_packed<1, 16, 2>(xb, wb, out, ep, M, N, K, stream, slices, rn);
   // very wide (the output head): from 5 rows of x on two groups of rows a wave as well (N = 151936, K = 4096 at 8 rows:
-  // 193 -> 182 us; at one row 175 -> 179; three or four groups a wave, or deeper, lose again)
-  else if (M >= 5) launch_packed2<8, 4>(xb, wb, out, ep, M, N, K, stream, slices, rn);
+  // 193 -> 182 us; at one row 175 -> 179; three or four groups a wave, or deeper, lose again; N = 10240 in two slices
+  // of K: 18.9 -> 20.0 us, so only where W is very wide)
+  else if (M >= 5 && N >= 32768) launch_packed2<8, 4>(xb, wb, out, ep, M, N, K, stream, slices, rn);
   else launch_packed<1, 8, 8>(xb, wb, out, ep, M, N, K, stream, slices, rn);
   SYN_LAUNCH_CHECK("gemm_packed");
   return 0;
