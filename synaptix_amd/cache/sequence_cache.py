@@ -7,7 +7,7 @@ group has storage and a page pool of its own:
     v_pages [layers, pages, kv_heads, head_dim, 64]      (transposed inside the page; a bf16 page in the
                                                           order of its kernels, ops.v_pages_to_kernel_order)
 A group that keeps a window gives pages back as soon as every position in them has left the
-window.  Layers with a StateNeed get `state[layer] : [slots, *shape]`, zeroed when a slot is
+window.  Layers with a StateNeed get `state[layer] : [slots + 1, *shape]`, zeroed when a slot is
 taken (the reference keeps such state in the same per-layer vector as the keys and values,
 crates/synaptix-models/llm/common/src/model.rs:359-362,377-492).
 
@@ -38,8 +38,26 @@ class KvLayerView:
 
 @dataclass
 class StateLayerView:
-    """What a mixer with a StateNeed is handed: state [slots, *shape]; row = slot id."""
+    """What a mixer with a StateNeed is handed: state [slots + 1, *shape]; row = slot id, and the last
+    row belongs to the padding rows of a captured step (no sequence owns it, as with the spare page).
+
+    A mixer whose steps are to be replayed from graphs reads and writes its state through row indices
+    that lie on the device (`seq_rows`, `token_rows`: index_select / index_copy_ with them), because
+    a captured step does not know its slots on the host."""
     state: torch.Tensor
+
+    @property
+    def spare_row(self) -> int:
+        return self.state.shape[0] - 1
+
+    def seq_rows(self, ctx) -> torch.Tensor:
+        """int64 [n_seqs] on the device: the state row of each sequence of the step (padding: the spare row)."""
+        slot = ctx.seq_slot
+        return torch.where(slot < 0, torch.full_like(slot, self.spare_row), slot).long()
+
+    def token_rows(self, ctx) -> torch.Tensor:
+        """int64 [n_tokens] on the device: the state row of the sequence that each token of the step is in."""
+        return self.seq_rows(ctx).index_select(0, ctx.tok_seq.long())
 
 
 @dataclass
@@ -106,7 +124,8 @@ class SequenceCache:
                 self._layer_index[i] = len(self.groups[gi].layers)
                 self.groups[gi].layers.append(i)
             elif isinstance(need, StateNeed):
-                self._state[i] = torch.zeros((self.max_slots,) + tuple(need.shape), dtype=need.dtype,
+                # one row more than slots: the padding rows of a captured step keep their state there
+                self._state[i] = torch.zeros((self.max_slots + 1,) + tuple(need.shape), dtype=need.dtype,
                                              device=self.device)
             elif need is not None:
                 raise CacheError(f"cache layer {i}: unknown need {need!r}")
@@ -220,6 +239,16 @@ class SequenceCache:
         self.truncate(snap.slot, snap.length)
         for i, saved in snap.states.items():
             self._state[i][snap.slot].copy_(saved)
+
+    def states_of(self, sids: list) -> dict:
+        """Copies of the fixed-size states of these slots alone (lengths and pages are not touched)."""
+        rows = torch.tensor([self._sid(s) for s in sids], dtype=torch.long, device=self.device)
+        return {"rows": rows, "states": {i: st.index_select(0, rows) for i, st in self._state.items()}}
+
+    def put_states(self, saved: dict) -> None:
+        """The states as `states_of` found them."""
+        for i, rows in saved["states"].items():
+            self._state[i].index_copy_(0, saved["rows"], rows)
 
     # ------------------------------------------------------------------ what a step needs
     def table_width(self, gi: int, sids: list) -> int:

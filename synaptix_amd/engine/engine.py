@@ -59,11 +59,11 @@ class Engine:
         self._dev = None
         self._runners = {}
         from ..parts.base import StateNeed
-        # a captured step is run more than once while it is recorded: only steps that write the
-        # same values again may be captured, which a mixer with a running state is not; and every part has
-        # to say of itself that it only launches kernels (Part.capturable)
+        # steps are replayed from graphs only if every part says of itself that it only launches kernels and
+        # finds its sequences through arrays on the device (Part.capturable).  A step is run before it is
+        # captured; where sequences have running states the runner puts them back after each such run.
         self.has_states = any(isinstance(n, StateNeed) for n in model.cache_needs())
-        self.graph_ok = not self.has_states and bool(getattr(model, "capturable", lambda: False)())
+        self.graph_ok = bool(getattr(model, "capturable", lambda: False)())
         self.prompt_graphs = True        # short prompt steps are replayed from graphs (see _prompt_runner)
 
     # ------------------------------------------------------------------ construction

@@ -39,14 +39,18 @@ def bucket_for(n: int) -> int:
     return (n + 31) // 32 * 32
 
 
-def _captured(forward, scratch):
-    """Run `forward` twice on a side stream (a step that may be captured writes the same values again), freeze
-    its scratch pool, then capture it; returns (graph, what forward returned)."""
+def _captured(forward, scratch, rewind=None):
+    """Run `forward` twice on a side stream, freeze its scratch pool, then capture it; returns (graph, what
+    forward returned).  Keys and values are written to the same places with the same values every time; what a
+    run changes for good (running states) `rewind` puts back after each of the two runs, so that the first
+    replay finds the sequences where the step found them."""
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side), torch.no_grad():
         for _ in range(2):
             forward()
+            if rewind is not None:
+                rewind()
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     scratch.frozen = True
@@ -65,6 +69,14 @@ def _captured(forward, scratch):
         if was_enabled:
             gc.enable()
     return graph, out
+
+
+def _state_rewind(engine, slots):
+    """What puts the running states of these slots back to where they are now, or None if there are none."""
+    if not engine.has_states:
+        return None
+    saved = engine.cache.states_of(slots)
+    return lambda: engine.cache.put_states(saved)
 
 
 class DecodeRunner:
@@ -139,7 +151,7 @@ class DecodeRunner:
                               self.scratch)
             ctx.max_position = eng.max_positions - 1 if eng.max_positions else 0   # checked on the host each step
             ctx.items = self.items
-            self.graph, self.logits = _captured(lambda: self._forward(ctx), self.scratch)
+            self.graph, self.logits = _captured(lambda: self._forward(ctx), self.scratch, _state_rewind(eng, slots))
         self.graph.replay()
         out = self.out_tokens[:B].cpu().tolist()      # waits for the step
         for s in slots:
@@ -164,7 +176,7 @@ class PromptRunner:
     """A prompt step of up to `rows` tokens in up to `seqs - 1` sequences, each with one wanted row,
     replayed from a graph.  The step's own tokens come first; the rows behind them are padding: token 0
     at positions 0, 1, ... of one more sequence that owns no slot and whose page table names only the
-    spare page.  A prompt step writes the same values when it is run again, so it may be captured."""
+    spare page (and whose running state, where there is one, is the spare row)."""
 
     def __init__(self, engine, rows: int, seqs: int, widths: list):
         self.engine, self.rows, self.seqs, self.widths = engine, rows, seqs, list(widths)
@@ -199,6 +211,6 @@ class PromptRunner:
                               [self.rows] + [0] * (self.seqs - 1), self.scratch)
             ctx.max_position = eng.max_positions - 1 if eng.max_positions else 0   # checked on the host each step
             self.graph, self.logits = _captured(lambda: eng.model.forward(ctx, ctx.tokens, ctx.want, eng.cache),
-                                                self.scratch)
+                                                self.scratch, _state_rewind(eng, slots))
         self.graph.replay()
         return self.logits[:len(want_rows)].clone()     # the next replay writes the same rows again

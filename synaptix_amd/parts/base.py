@@ -17,9 +17,11 @@ class Part:
     """Base of norms, position encodings, mixers, feed-forwards and blocks."""
 
     # True: the part's forward only launches kernels on the current stream (no wait for the device, no shape that
-    # depends on device data) and writes the same values when it is run again, so that a step that contains it
-    # may be captured into a graph and replayed.  False (the default, for parts from elsewhere): the steps of a
-    # model that contains it are launched one by one.
+    # depends on device data), finds the step's sequences through the context's device arrays alone (a captured
+    # step's `ctx.slots`, `ctx.past` and `ctx.new_counts` are placeholders; a running state is reached with
+    # StateLayerView.seq_rows / token_rows) and, apart from such a state, writes the same values when it is run
+    # again, so that a step that contains it may be captured into a graph and replayed.  False (the default, for
+    # parts from elsewhere): the steps of a model that contains it are launched one by one.
     capturable = False
 
     def tensor_specs(self) -> dict:

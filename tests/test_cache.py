@@ -20,7 +20,7 @@ def test_groups_and_storage():
     assert c.groups[1].k.shape == (1, 11, 1, 64, 32) and c.groups[1].spare_page == 10
     v0, v2, v3 = c.layer_view(0), c.layer_view(2), c.layer_view(3)
     assert v0.group == v2.group == 0 and v0.k_pages.data_ptr() != v2.k_pages.data_ptr()
-    assert v3.state.shape == (10, 3, 5) and c.layer_view(4) is None
+    assert v3.state.shape == (10 + 1, 3, 5) and v3.spare_row == 10 and c.layer_view(4) is None   # a row for padding
     assert c.bytes_per_token() == 2 * 4 * (2 * 2 * 16 + 1 * 32 + 2 * 16)
 
 
@@ -157,6 +157,29 @@ def test_random_walk_keeps_every_invariant():
         c.release(s)
     c.check()
     assert c.free_slots == 12 and all(g.pool.free_pages == 40 for g in c.groups)
+
+
+def test_states_of_some_slots_are_copied_and_put_back_and_padding_has_a_row_of_its_own():
+    """What a captured step needs of the states: the rows of its slots alone can be saved and put back without a
+    touch to lengths or to other slots; and a step's sequences map to rows through the step's own slot array, the
+    padding (slot -1) to the spare row behind the slots."""
+    from types import SimpleNamespace
+    c = make(needs=[StateNeed((3,)), KvNeed(2, 16)], max_slots=3)
+    a, b, d = c.acquire(), c.acquire(), c.acquire()
+    st = c.layer_view(0).state
+    st[a] += 1.0
+    st[b] += 2.0
+    st[d] += 3.0
+    saved = c.states_of([a, d])
+    st += 10.0
+    c.put_states(saved)
+    assert st[a].tolist() == [1.0] * 3 and st[d].tolist() == [3.0] * 3 and st[b].tolist() == [12.0] * 3
+    view = c.layer_view(0)
+    ctx = SimpleNamespace(seq_slot=torch.tensor([d, -1, a], dtype=torch.int32), tok_seq=torch.tensor([0, 0, 2, 1], dtype=torch.int32))
+    assert view.seq_rows(ctx).tolist() == [d, 3, a] and view.spare_row == 3
+    assert view.token_rows(ctx).tolist() == [d, d, a, 3]
+    with pytest.raises(CacheError):
+        c.states_of([7.5])
 
 
 def test_going_back_to_a_snapshot():

@@ -251,6 +251,121 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
         assert (first - whole[4:7]).abs().max() <= tolerance
 
 
+def test_toy_mixer_with_state_is_replayed_from_graphs(tmp_path):
+    """The same running mean, written so that its steps may be captured: it finds the state rows of the step's
+    sequences through the device arrays of the step (StateLayerView.token_rows), never through slots on the host,
+    and says so (capturable).  Prompt steps and decode steps then come from graphs like any other model's: the
+    runs that precede a capture must leave no trace in the states (the first replay is checked), every replay
+    must advance them once (later replays are checked), padding rows must keep to the spare row (a fourth
+    sequence that takes no part in the replayed steps goes on afterwards with the right state), and a slot that
+    is used again starts from zero."""
+    from dataclasses import dataclass, asdict
+    import json
+    from synaptix_amd import register_architecture, Engine
+    from synaptix_amd.models import DecoderModel, LayerRun, TokenEmbedding, OutputHead
+    from synaptix_amd.parts import Mixer, StateNeed, RmsNorm, GatedMlp, PreNormBlock, GqaAttention, RotaryHalfSplit
+    from synaptix_amd.weights import TensorSpec, save_file, RandomSource
+
+    class RunningMeanOnDevice(Mixer):
+        capturable = True
+
+        def __init__(self, prefix, hidden, decay):
+            self.prefix, self.hidden, self.decay = prefix, hidden, decay
+            self.scale = None
+
+        def tensor_specs(self):
+            return {self.prefix + "scale": TensorSpec((self.hidden,), "gain")}
+
+        def load(self, get):
+            self.scale = get(self.prefix + "scale").float()
+
+        def cache_need(self):
+            return StateNeed((self.hidden,), torch.float32)
+
+        def forward(self, h, ctx, cache, owner=True):
+            rows = cache.token_rows(ctx)                        # on the device; padding tokens: the spare row
+            out = torch.empty(h.shape, dtype=torch.float32, device=h.device)
+            for t in range(h.shape[0]):                         # tokens of a sequence lie in order
+                r = rows[t:t + 1]
+                s = cache.state.index_select(0, r) * self.decay + h[t:t + 1].float()
+                cache.state.index_copy_(0, r, s)
+                out[t:t + 1] = s * self.scale
+            return out
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        vocab_size: int = 97
+        hidden_size: int = 48
+        intermediate_size: int = 80
+        decay: float = 0.5
+        max_position_embeddings: int = 128
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(**{k: d[k] for k in cls.__dataclass_fields__ if k in d})
+
+        def to_dict(self):
+            return {**asdict(self), "architectures": ["ToyRunningMeanOnDevice"]}
+
+    def build(cfg, max_positions=None):
+        emb = TokenEmbedding("emb", cfg.vocab_size, cfg.hidden_size)
+        rope = RotaryHalfSplit(1e4, 16, cfg.max_position_embeddings)
+        blocks = [
+            PreNormBlock(RmsNorm("l0.n1", cfg.hidden_size, 1e-5), RunningMeanOnDevice("l0.mix.", cfg.hidden_size, cfg.decay),
+                         RmsNorm("l0.n2", cfg.hidden_size, 1e-5), GatedMlp("l0.ff.", cfg.hidden_size, cfg.intermediate_size)),
+            PreNormBlock(RmsNorm("l1.n1", cfg.hidden_size, 1e-5),
+                         GqaAttention("l1.att.", cfg.hidden_size, 3, 1, 16, position=rope),
+                         RmsNorm("l1.n2", cfg.hidden_size, 1e-5), GatedMlp("l1.ff.", cfg.hidden_size, cfg.intermediate_size)),
+        ]
+        schedule = [LayerRun(0, 0), LayerRun(1, 1), LayerRun(0, 2)]
+        return DecoderModel(cfg, emb, blocks, schedule, RmsNorm("norm", cfg.hidden_size, 1e-5),
+                            OutputHead("head", cfg.vocab_size, cfg.hidden_size))
+
+    register_architecture("ToyRunningMeanOnDevice", ToyConfig, build)
+    cfg = ToyConfig()
+    src = RandomSource(build(cfg).tensor_specs(), 5, std=0.2)
+    save_file({n: src.tensor(n) for n in src.names()}, str(tmp_path / "model.safetensors"))
+    (tmp_path / "config.json").write_text(json.dumps(cfg.to_dict()))
+
+    seqs = [[5, 9, 33, 2, 70, 11, 8, 41, 3], [90, 1, 4, 17, 60, 2, 2], [7, 7, 52, 13, 88, 21, 30, 6], [64, 12, 95, 3, 18, 44]]
+    heads = [5, 3, 4, 3]                                         # tokens that come as prompts
+    for dtype in ("float32", "bfloat16"):
+        eng = Engine.load(str(tmp_path), dtype=dtype, max_tokens=1024, max_slots=4)
+        assert eng.has_states and eng.graph_ok
+        tolerance = 1e-4 if dtype == "float32" else 5e-2
+        # what every position should give: each sequence whole and alone, launched one by one
+        eng.prompt_graphs = False
+        whole = []
+        for toks in seqs:
+            s = eng.acquire()
+            whole.append(eng.step([(s, toks)], want="all").clone())
+            eng.release(s)
+        eng.prompt_graphs = True
+        for round_ in range(2):                                  # the second round takes the same slots again
+            slots = [eng.acquire() for _ in seqs]
+            # the fourth sequence starts before the others and waits while their steps are replayed
+            lg = eng.step([(slots[3], seqs[3][:heads[3]])], want="last")
+            assert (lg - whole[3][heads[3] - 1:heads[3]]).abs().max() <= tolerance
+            live = [0, 1, 2]
+            lg = eng.step([(slots[i], seqs[i][:heads[i]]) for i in live], want="last")     # bfloat16: a captured prompt step
+            for j, i in enumerate(live):
+                assert (lg[j] - whole[i][heads[i] - 1]).abs().max() <= tolerance, (dtype, round_, "prompt", i)
+            assert (dtype == "bfloat16") == any(k[0] == "prompt" for k in eng._runners)
+            runner = eng.decode_runner(3, 64)                    # 4 rows: one of padding
+            d = 0
+            while live:
+                _, lg = runner.step([slots[i] for i in live], [seqs[i][heads[i] + d] for i in live])
+                for j, i in enumerate(live):
+                    assert (lg[j] - whole[i][heads[i] + d]).abs().max() <= tolerance, (dtype, round_, "decode", d, i)
+                d += 1
+                live = [i for i in live if heads[i] + d < len(seqs[i])]      # shorter sequences end earlier
+            lg = eng.step([(slots[3], seqs[3][heads[3]:])], want="all")
+            assert (lg - whole[3][heads[3]:]).abs().max() <= tolerance, (dtype, round_, "the sequence that waited")
+            for s in slots:
+                eng.release(s)
+        eng.cache.check()
+
+
 # ----------------------------------------------------------------------------- more toy parts
 def test_toy_position_encoding_plugs_into_attention():
     """Another position encoding, defined here: angles that grow linearly with the index of the
