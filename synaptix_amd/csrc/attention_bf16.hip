@@ -128,15 +128,20 @@ constexpr int PF_CHUNKS = (8 * HD + PF_THREADS - 1) / PF_THREADS;  // 16-byte ch
 // sequence.  Two workgroups share a compute unit, and a tile's work grows with its number: the first
 // half of the grid takes the tiles from the last downwards, the second half from the first upwards,
 // so that the pairs that meet on a unit have about equal work.  False: the grid is an upper bound.
-__device__ __forceinline__ bool prefill_tile(const int* __restrict__ seq_start, int n_seqs, int& seq, int& q0) {
+// Sequences with fewer new tokens than skip_below have no tiles (their rows of `out` are left as they are).
+__device__ __forceinline__ bool prefill_tile(const int* __restrict__ seq_start, int n_seqs, int skip_below, int& seq, int& q0) {
+  auto tiles_of = [&](int s) {
+    const int n = seq_start[s + 1] - seq_start[s];
+    return n < skip_below ? 0 : (n + PF_ROWS - 1) / PF_ROWS;
+  };
   int total = 0;
-  for (int s = 0; s < n_seqs; ++s) total += (seq_start[s + 1] - seq_start[s] + PF_ROWS - 1) / PF_ROWS;
+  for (int s = 0; s < n_seqs; ++s) total += tiles_of(s);
   const int y = blockIdx.y, half = (total + 1) / 2;
   if (y >= total) return false;
   const int tile = y < half ? total - 1 - y : y - half;
   int t_acc = 0;
   for (int s = 0; s < n_seqs; ++s) {
-    const int nt = (seq_start[s + 1] - seq_start[s] + PF_ROWS - 1) / PF_ROWS;
+    const int nt = tiles_of(s);
     if (tile < t_acc + nt) {
       seq = s;
       q0 = (tile - t_acc) * PF_ROWS;
@@ -151,12 +156,12 @@ __global__ void __launch_bounds__(PF_THREADS)
 attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
                     const int* __restrict__ page_table, int table_stride, const int* __restrict__ seq_start,
                     const int* __restrict__ seq_past, int n_seqs, bf16* __restrict__ out, float scale,
-                    int window, int nh, int nkv, ScoreTerms terms) {
+                    int window, int nh, int nkv, ScoreTerms terms, int skip_below) {
   extern __shared__ __attribute__((aligned(16))) bf16 lds[];  // [2][PF_TILE]
   // Heads run fastest through the grid; workgroups go round the eight dies in turn, and the heads are
   // dealt so that each die gets neighbouring heads, which share their K and V.
   int seq, q0;
-  if (!prefill_tile(seq_start, n_seqs, seq, q0)) return;
+  if (!prefill_tile(seq_start, n_seqs, skip_below, seq, q0)) return;
   const int tid = threadIdx.x, wave = tid / SYN_WAVE, lane = tid % SYN_WAVE;
   const int r16 = lane % 16, g4 = lane / 16;
   const int hx = blockIdx.x;
@@ -370,10 +375,10 @@ __global__ void __launch_bounds__(PF2_THREADS, 2)
 attn_prefill32_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
                       const int* __restrict__ page_table, int table_stride, const int* __restrict__ seq_start,
                       const int* __restrict__ seq_past, int n_seqs, bf16* __restrict__ out, float scale,
-                      int window, int nh, int nkv) {
+                      int window, int nh, int nkv, int skip_below) {
   extern __shared__ __attribute__((aligned(16))) char lds2[];  // [2][K block | V block]
   int seq, q0;
-  if (!prefill_tile(seq_start, n_seqs, seq, q0)) return;
+  if (!prefill_tile(seq_start, n_seqs, skip_below, seq, q0)) return;
   const int tid = threadIdx.x, lane = tid % SYN_WAVE;
   const int wave = __builtin_amdgcn_readfirstlane(tid / SYN_WAVE);
   const int n32 = lane % 32, hh = lane / 32;
@@ -557,10 +562,12 @@ SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, co
                                           const int* page_table, int table_stride, const int* seq_start,
                                           const int* seq_past, int n_seqs, int n_tokens, void* out, float scale,
                                           int window, int nh, int nkv, int hd, int variant, const float* slopes,
-                                          float softcap, hipStream_t stream) {
+                                          float softcap, int skip_below, hipStream_t stream) {
   // variant: 0 = whichever is faster for this head size, 1 = waves of 16 query rows (every head size),
   // 2 = waves of 32 query rows (head sizes 64 and 128, a positive scale, no terms on the scores)
   // slopes [nh] float or null, softcap (0: none): see ScoreTerms; the kernel with waves of 16 rows applies them
+  // skip_below: sequences that bring fewer new tokens than this are left out (2: those with a single token, which
+  // the caller hands to the decode kernel); 0 or 1: none
   SYN_CHECK(variant >= 0 && variant <= 2, "attention_prefill: unknown variant %d", variant);
   SYN_CHECK(softcap >= 0.f, "attention_prefill: a soft cap of %g", (double)softcap);
   const ScoreTerms terms = {slopes, softcap};
@@ -584,14 +591,14 @@ SYN_EXPORT int syn_attention_prefill_bf16(const void* q, const void* k_pages, co
     if (variant == 2 || (variant == 0 && scale > 0.f && !with_terms)) {
       attn_prefill32_kernel<<<dim3(nh, tiles), PF2_THREADS, 2 * PF2_BUF, stream>>>(
           (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, page_table, table_stride, seq_start, seq_past,
-          n_seqs, (bf16*)out, scale, window, nh, nkv);
+          n_seqs, (bf16*)out, scale, window, nh, nkv, skip_below);
       SYN_LAUNCH_CHECK("attention_prefill32");
       return 0;
     }
   }
   attn_prefill_kernel<<<dim3(nh, tiles), PF_THREADS, lds, stream>>>(
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, page_table, table_stride, seq_start, seq_past, n_seqs,
-      (bf16*)out, scale, window, nh, nkv, terms);
+      (bf16*)out, scale, window, nh, nkv, terms, skip_below);
   SYN_LAUNCH_CHECK("attention_prefill");
   return 0;
 }

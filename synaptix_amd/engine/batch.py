@@ -95,6 +95,20 @@ class StepContext:
         """The group's work list for decode attention (int32 [n_seqs * decode_splits, 4]) or None."""
         return None if self.items is None else self.items[group]
 
+    def single_token_rows(self):
+        """In a step that brings whole prompts for some sequences and one token for others: (the token rows, the
+        sequence indices) of those with one token, as int64 tensors on the device; None in every other step.  A
+        mixer may hand these sequences to its kernel for single tokens (one workgroup a tile of query rows would
+        walk a long sequence's keys alone)."""
+        if not hasattr(self, "_singles"):
+            self._singles = None
+            seqs = [i for i, n in enumerate(self.new_counts) if n == 1]
+            if seqs and len(seqs) < len(self.new_counts):
+                starts = np.concatenate([[0], np.cumsum(self.new_counts)])
+                self._singles = (torch.tensor([int(starts[i]) for i in seqs], dtype=torch.long, device=self.device),
+                                 torch.tensor(seqs, dtype=torch.long, device=self.device))
+        return self._singles
+
     def scratch(self, name: str, numel: int) -> torch.Tensor:
         """Float scratch memory that lives as long as its pool's owner; contents are undefined."""
         return self._scratch.get(name, numel)

@@ -557,12 +557,13 @@ def _attn_lib(hd):
 
 
 def attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, seq_past, out, scale, window, n_heads,
-                           n_kv_heads, head_dim, variant=0, slopes=None, softcap=0.0):
+                           n_kv_heads, head_dim, variant=0, slopes=None, softcap=0.0, skip_below=0):
     """Causal attention of the new tokens of each sequence over its cache (which already holds them).
     seq_start [B+1]: offsets of the sequences' new tokens in q; seq_past [B]: tokens cached before.
     variant: 0 = the kernel's own choice, 1 = waves of 16 query rows (every head size), 2 = waves of 32
     query rows (head sizes 64 and 128); for comparisons.  slopes, softcap: see _score_terms (they take the kernel
-    with waves of 16 rows)."""
+    with waves of 16 rows).  skip_below: sequences with fewer new tokens than this are left out and their rows of
+    `out` stay as they are (2: single tokens, which the caller hands to attention_decode_bf16)."""
     nh, nkv, hd = n_heads, n_kv_heads, head_dim
     _need(q, "attention_prefill.q", _BF16, (None, nh * hd))
     N = q.shape[0]
@@ -576,7 +577,8 @@ def attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, seq_past,
     _need(out, "attention_prefill.out", _BF16, (N, nh * hd))
     _call(_attn_lib(hd), "syn_attention_prefill_bf16", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
           page_table.shape[1], _ptr(seq_start), _ptr(seq_past), B, N, _ptr(out), ctypes.c_float(scale),
-          int(window or 0), nh, nkv, hd, int(variant), *_score_terms("attention_prefill", slopes, softcap, nh), _stream())
+          int(window or 0), nh, nkv, hd, int(variant), *_score_terms("attention_prefill", slopes, softcap, nh),
+          int(skip_below), _stream())
 
 
 def decode_splits(n_seqs, n_kv_heads, max_pages):

@@ -157,6 +157,19 @@ class GqaAttention(Mixer):
             ops.attention_decode_bf16(q, cache.k_pages, cache.v_pages, table, ctx.seq_len, o, work, splits,
                                       self.scale, window, nh, nkv, hd, **terms, **merge)
         else:
+            # a step of prompts and single tokens: the prompts' kernel leaves the single tokens out, and the kernel
+            # for single tokens takes them (gathered, since it counts one row a sequence)
+            singles = ctx.single_token_rows()
             ops.attention_prefill_bf16(q, cache.k_pages, cache.v_pages, table, ctx.seq_start, ctx.seq_past, o,
-                                       self.scale, window, nh, nkv, hd, **terms)
+                                       self.scale, window, nh, nkv, hd, skip_below=2 if singles is not None else 0, **terms)
+            if singles is not None:
+                rows, seqs = singles
+                n1 = rows.numel()
+                q1, o1 = q.index_select(0, rows), torch.empty((n1, nh * hd), dtype=act, device=h.device)
+                splits = ops.decode_splits(n1, nkv, table.shape[1])
+                work = ctx.scratch("attention_decode", n1 * nh * splits * (hd + 2))
+                ops.attention_decode_bf16(q1, cache.k_pages, cache.v_pages, table.index_select(0, seqs),
+                                          ctx.seq_len.index_select(0, seqs), o1, work, splits, self.scale, window,
+                                          nh, nkv, hd, **terms)
+                o.index_copy_(0, rows, o1)
         return deferred_product(o, self.w_o)

@@ -189,10 +189,12 @@ def attention_f32(q, k_pages, v_pages, page_table, tok_seq, tok_pos, out, scale,
 
 
 def attention_prefill_bf16(q, k_pages, v_pages, page_table, seq_start, seq_past, out, scale, window, n_heads,
-                           n_kv_heads, head_dim, variant=0, slopes=None, softcap=0.0):
+                           n_kv_heads, head_dim, variant=0, slopes=None, softcap=0.0, skip_below=0):
     N = q.shape[0]
     qf = q.to(F32).view(N, n_heads, head_dim)
     for b in range(seq_past.shape[0]):
+        if int(seq_start[b + 1]) - int(seq_start[b]) < skip_below:
+            continue
         for n in range(int(seq_start[b]), int(seq_start[b + 1])):
             pos = int(seq_past[b]) + n - int(seq_start[b])
             o = _attend(qf[n], k_pages, v_pages, page_table[b], pos, scale, window, n_heads, n_kv_heads, head_dim,

@@ -272,6 +272,30 @@ def test_graph_replays_equal_eager_steps(dtype):
         e.cache.check()
 
 
+def test_single_tokens_beside_prompts_take_the_kernel_for_single_tokens():
+    """A step of two sequences that go on by one token over some hundred cached tokens and one prompt that starts:
+    the prompts' attention kernel runs once a layer and leaves the single tokens to the kernel for single tokens,
+    which runs once a layer as well; the logits are those of the plain implementation (with peaked attention, so
+    that a key out of reach or a row handed to the wrong sequence shows)."""
+    from synaptix_amd.kernels import ops
+    name, sharp = "C", True
+    V, L = CONFIGS[name]["vocab_size"], CONFIGS[name]["num_hidden_layers"]
+    olds = [random_tokens(V, 300 + 1, 61), random_tokens(V, 130 + 1, 62)]
+    fresh = random_tokens(V, 90, 63)
+    eng = make_engine(name, "bfloat16", 2048, sharp)
+    a, b, c = eng.acquire(), eng.acquire(), eng.acquire()
+    eng.step([(a, olds[0][:300]), (b, olds[1][:130])], want=None)
+    with ops.op_timing() as times:
+        lg = eng.step([(a, olds[0][300:]), (c, fresh), (b, olds[1][130:])], want="all")
+    assert times["syn_attention_prefill_bf16"][1] == L and times["syn_attention_decode_bf16"][1] == L
+    assert_logits_close(lg[:1], plain_logits(name, olds[0], sharp)[300:], "bfloat16", "the first single token", sharp)
+    assert_logits_close(lg[1:91], plain_logits(name, fresh, sharp), "bfloat16", "the prompt between them", sharp)
+    assert_logits_close(lg[91:], plain_logits(name, olds[1], sharp)[130:], "bfloat16", "the second single token", sharp)
+    for s_ in (a, b, c):
+        eng.release(s_)
+    eng.cache.check()
+
+
 @pytest.mark.parametrize("name", ["B", "C"])
 def test_captured_prompt_steps_equal_eager_ones(name):
     """Short prompt steps are replayed from graphs with padding rows behind their own: every replay against

@@ -672,6 +672,15 @@ def test_attention_prefill(ops, dtype, nh, nkv, hd, past, new, window):
             ops.attention_prefill_bf16(d(q), d(k), dv(v), d(table), d(starts), d(past_t), out, scale, window, nh, nkv,
                                        hd, variant=variant)
             close(out, want, 2e-2, 1e-2, what=f"attention prefill bf16, variant {variant}")
+            # sequences with a single new token left out (a step of prompts and single tokens hands them to the
+            # kernel for single tokens): their rows stay as they were, the others are computed as before
+            if 1 in new and any(n > 1 for n in new):
+                out.fill_(7.0)
+                ops.attention_prefill_bf16(d(q), d(k), dv(v), d(table), d(starts), d(past_t), out, scale, window, nh, nkv,
+                                           hd, variant=variant, skip_below=2)
+                single = torch.tensor([n == 1 for n in new])[tok_seq.long()]
+                assert bool((out.cpu()[single] == 7.0).all()), "a single token's row was written"
+                close(out.cpu()[~single], want[~single], 2e-2, 1e-2, what=f"prompts beside skipped single tokens, variant {variant}")
 
 
 @pytest.mark.parametrize("nh,nkv,hd,past,new,window,softcap,sloped", [
