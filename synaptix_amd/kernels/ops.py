@@ -296,6 +296,13 @@ def gemm_swiglu(x, w_paired, out, activation="silu"):
 PACKED_BLOCK_ROWS = 16   # the most rows that a product of gemm_packed takes
 PACKED_MAX_ROWS = 8   # up to this many rows of x the products over packed weights are the faster ones
 PACKED_MAX_ROWS_GATED = 16   # the gated product, whose waves take two groups of rows of W for every fragment of x
+PACKED_WIDE_N = 32768   # from this many rows of W on (an output head) the products over packed weights stay the faster
+                        # ones up to 16 rows of x (151,936 x 4,096 at 16 rows: 222 us on tiles, as at 8 rows in fragments)
+
+
+def packed_max_rows(n_out: int) -> int:
+    """Up to how many rows of x a plain product with a packed weight of n_out rows takes the kernels for few rows."""
+    return PACKED_BLOCK_ROWS if n_out >= PACKED_WIDE_N else PACKED_MAX_ROWS
 
 
 def pack_weight(w):

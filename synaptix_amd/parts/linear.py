@@ -36,7 +36,7 @@ class Matrix:
 
 
 def _use_packed(x, m):
-    return m.packed is not None and x.dtype == torch.bfloat16 and x.shape[0] <= ops.PACKED_MAX_ROWS
+    return m.packed is not None and x.dtype == torch.bfloat16 and x.shape[0] <= ops.packed_max_rows(m.shape[0])
 
 
 def _matrix(w):

@@ -291,7 +291,7 @@ def test_gemm_with_the_gated_activation_inside(ops, M, I, K):
 @pytest.mark.parametrize("out_dtype", [BF16, F32])
 @pytest.mark.parametrize("M,N,K", [(1, 16, 32), (1, 4096, 4096), (8, 6144, 4096), (3, 48, 96), (5, 1008, 1120), (8, 16400, 160),
                                    (16, 64, 12288), (7, 80, 2080),
-                                   (8, 32784, 96), (5, 40000, 4096)])   # very wide from 5 rows on: two groups of rows a wave, an odd number of groups
+                                   (8, 32784, 96), (5, 40000, 4096), (13, 32784, 96)])   # very wide from 5 rows on: two groups of rows a wave, an odd number of groups
 def test_gemm_over_weights_in_fragment_order(ops, out_dtype, M, N, K):
     """The products for few rows over pack_weight(W): every k-step and every row tile lands where the
     plain product has it, also where K is no multiple of the waves' turns and N of the workgroup's rows."""
