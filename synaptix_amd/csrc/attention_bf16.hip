@@ -413,29 +413,33 @@ attn_prefill32_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pag
     for (int e = 0; e < 16; ++e) o[d][e] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  auto fetch = [&](int kb, int buf) {
+  // Load j of a wave for a block: its share of K (even j) or of V (odd j), 1 KB straight into LDS.
+  constexpr int NLOAD = 2 * (PF2_KBYTES / 1024 / PF2_WAVES);
+  auto views_of = [&](int kb, BufferView& vk, BufferView& vv) {
     const size_t base =
         ((size_t)__builtin_amdgcn_readfirstlane(page_table[(size_t)seq * table_stride + kb]) * nkv + kvh) * SYN_PAGE * HD;
-    const BufferView vk = buffer_view(k_pages + base, PF2_KBYTES), vv = buffer_view(v_pages + base, PF2_KBYTES);
+    vk = buffer_view(k_pages + base, PF2_KBYTES), vv = buffer_view(v_pages + base, PF2_KBYTES);
+  };
+  auto fetch_one = [&](const BufferView& vk, const BufferView& vv, int buf, int j) {
     char* dst = lds2 + buf * PF2_BUF;
-#pragma unroll
-    for (int it = 0; it < PF2_KBYTES / 1024 / PF2_WAVES; ++it) {
-      const int i = it * PF2_WAVES + wave;                 // which 1 KB of the block this wave's load fills
-      const int at = 64 * i + lane, krow = at / PF2_CPR, slot = at % PF2_CPR;
-      buffer_to_lds16(vk, dst + 1024 * i, (unsigned)((krow * PF2_CPR + (slot ^ pf2_swizzle(krow))) * 16), 0);
-      buffer_to_lds16(vv, dst + PF2_KBYTES + 1024 * i, (unsigned)(at * 16), 0);
-    }
+    const int i = (j / 2) * PF2_WAVES + wave;              // which 1 KB of the block this load fills
+    const int at = 64 * i + lane, krow = at / PF2_CPR, slot = at % PF2_CPR;
+    if (j % 2 == 0) buffer_to_lds16(vk, dst + 1024 * i, (unsigned)((krow * PF2_CPR + (slot ^ pf2_swizzle(krow))) * 16), 0);
+    else buffer_to_lds16(vv, dst + PF2_KBYTES + 1024 * i, (unsigned)(at * 16), 0);
   };
   auto landed = [&]() {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's loads have written LDS; behind the barrier all have
     __syncthreads();
   };
 
-  fetch(kb_lo, 0);
-  landed();
-  for (int kb = kb_lo; kb <= kb_hi; ++kb) {
-    const int buf = (kb - kb_lo) & 1;
-    if (kb < kb_hi) fetch(kb + 1, buf ^ 1);   // that buffer was last read before the previous barrier
+  // One block of keys.  MORE: a next block exists, and its loads are issued here, one behind every second MFMA of
+  // the scores: issued in a burst at the block's top, the loads of four waves queue at the texture addresser
+  // (about 16 cycles for each KB) and every wave stands until its own are taken (measured: a sixth of a wave's time).
+  auto block = [&](int kb, auto more) {
+    constexpr bool MORE = decltype(more)::value;
+    const int buf = (kb - kb_lo) & 1;                    // the other buffer was last read before the previous barrier
+    BufferView nk, nv;
+    if constexpr (MORE) views_of(kb + 1, nk, nv);
     const int key0 = kb * SYN_PAGE;
     char* ks_ = lds2 + buf * PF2_BUF;
     char* vs_ = ks_ + PF2_KBYTES;
@@ -460,6 +464,7 @@ attn_prefill32_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pag
       // before the softmax, so that they arrive while its maxima are taken.
       constexpr int NQK = 2 * PF2_KS, NPV = 4 * PF2_DT;
       constexpr int AHEAD = NQK < PF2_AHEAD ? NQK : PF2_AHEAD, VAHEAD = NPV < PF2_AHEAD ? NPV : PF2_AHEAD;
+      static_assert(!PF2_OK || NLOAD <= NQK / 2, "a load behind every second MFMA of the scores");
       f32x16 s[2];
 #pragma unroll
       for (int t = 0; t < 2; ++t)
@@ -483,12 +488,14 @@ attn_prefill32_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pag
         s[i % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], qf[i / 2], s[i % 2], 0, 0, 0);
         if (i + AHEAD < NQK) kf[i + AHEAD] = k_frag(i + AHEAD);
         else if (i + AHEAD - NQK < VAHEAD) vf[i + AHEAD - NQK] = v_frag(i + AHEAD - NQK);
+        if (MORE && i % 2 == 1 && i / 2 < NLOAD) fetch_one(nk, nv, buf ^ 1, i / 2);
       }
       __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
 #pragma unroll
       for (int i = 0; i < NQK; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA,
-        if (i + AHEAD < NQK || i + AHEAD - NQK < VAHEAD) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one read behind it
+        if (i + AHEAD < NQK || i + AHEAD - NQK < VAHEAD) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one read behind it,
+        if (MORE && i % 2 == 1 && i / 2 < NLOAD) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);           // a load behind every second
       }
       __builtin_amdgcn_sched_barrier(0);
       // a block needs masking if some row of the wave does not see all of it
@@ -539,9 +546,22 @@ attn_prefill32_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pag
         }
       }
       l_run += lsum;
+    } else if constexpr (MORE) {
+#pragma unroll
+      for (int j = 0; j < NLOAD; ++j) fetch_one(nk, nv, buf ^ 1, j);
     }
     landed();
+  };
+
+  {
+    BufferView vk, vv;
+    views_of(kb_lo, vk, vv);
+#pragma unroll
+    for (int j = 0; j < NLOAD; ++j) fetch_one(vk, vv, 0, j);
   }
+  landed();
+  for (int kb = kb_lo; kb < kb_hi; ++kb) block(kb, std::true_type{});
+  block(kb_hi, std::false_type{});
   if (!wave_on) return;
   float l = l_run + __shfl_xor(l_run, 32, SYN_WAVE);
   if (!valid) return;
