@@ -208,8 +208,9 @@ class Engine:
         one, the kernels of a few dozen tokens take the host longer than the GPU."""
         if not (self.prompt_graphs and self.graph_ok and self.dtype == torch.bfloat16) or ops.timing_active():
             return None
-        if len(want_rows) != len(slots) or all(c == 1 for c in counts):
-            return None
+        if len(want_rows) != len(slots) or any(c == 1 for c in counts):
+            return None         # (single tokens beside prompts go to their own attention kernel, which a captured
+                                # prompt step, knowing no counts on the host, cannot arrange)
         starts = np.concatenate([[0], np.cumsum(counts)])
         if any(not (starts[i] <= r < starts[i + 1]) for i, r in enumerate(want_rows)):
             return None

@@ -333,10 +333,13 @@ def test_captured_prompt_steps_equal_eager_ones(name):
     more = [random_tokens(V, n, 950 + n) for n in (40, 9)]
     got = both(lambda e: list(zip(slots[id(e)][3:5], more)), [[17], [8]])
     assert_logits_close(got[0:1], plain_logits(name, more[0])[17:18], dtype, "a wanted place that is not the last")
-    # second pieces of two prompts (tokens cached before), beside a fresh one-token sequence
+    # second pieces of two prompts (tokens cached before), beside a fresh sequence of two tokens (one of a single
+    # token would send the step to the kernels launched one by one, where single tokens have a kernel of their own)
     acquire(1)
     tails = [random_tokens(V, n, 970 + n) for n in (30, 12)]
-    got = both(lambda e: [(slots[id(e)][0], tails[0]), (slots[id(e)][3], tails[1]), (slots[id(e)][5], [7])], "last")
+    runners = len(graph._runners)
+    got = both(lambda e: [(slots[id(e)][0], tails[0]), (slots[id(e)][3], tails[1]), (slots[id(e)][5], [7, 9])], "last")
+    assert len(graph._runners) == runners                      # the graph of 64 rows again
     assert_logits_close(got[0:1], plain_logits(name, prompts[0] + tails[0])[-1:], dtype, "second piece of a prompt")
     assert_logits_close(got[1:2], plain_logits(name, more[0] + tails[1])[-1:], dtype, "second piece of a prompt")
     # a slot that is given back and used again; exactly as many tokens as the graph has rows (no padding rows)
