@@ -716,6 +716,34 @@ def sample_rows(logits, temperature, uniform, out):
           _ptr(uniform if temperature is not None else None), _ptr(out), R, V, _stream())
 
 
+def filter_rows(logits, out, temperature, top_k, top_p, min_p, repetition, presence, frequency,
+                ids=None, id_start=None, counts=None):
+    """The processors in front of the sampler, one workgroup a row of logits [R, V] (float): repetition penalty,
+    presence / frequency penalty, temperature, top-k, top-p, min-p, in this order; what is dropped becomes -inf
+    in `out` (which may be `logits`).  Every option is an array with one entry a row: temperature (<= 0 or 1:
+    the row is not divided), top_k (int32; 0: off), top_p (>= 1: off), min_p (0: off), repetition (1: off),
+    presence, frequency (0: off).  ids (int32, flat) and id_start (int32 [R + 1]) give each row the tokens that
+    the penalties look at; counts (int32 [R * V], zero) is their scratch memory, left zero."""
+    _need(logits, "filter_rows.logits", _F32, (None, None))
+    R, V = logits.shape
+    _need(out, "filter_rows.out", _F32, (R, V))
+    for name, t, dt in (("temperature", temperature, _F32), ("top_k", top_k, _I32), ("top_p", top_p, _F32),
+                        ("min_p", min_p, _F32), ("repetition", repetition, _F32), ("presence", presence, _F32),
+                        ("frequency", frequency, _F32)):
+        _need(t, f"filter_rows.{name}", dt, (R,))
+    if (ids is None) != (id_start is None):
+        raise KernelError("filter_rows: ids and id_start come together")
+    if ids is not None:
+        _need(ids, "filter_rows.ids", _I32, (None,))
+        _need(id_start, "filter_rows.id_start", _I32, (R + 1,))
+        _need(counts, "filter_rows.counts", _I32)
+        if counts.numel() < R * V:
+            raise KernelError(f"filter_rows: {counts.numel()} counters for {R} rows of {V}")
+    _call(load_library("core"), "syn_filter_rows", _ptr(logits), _ptr(out), R, V, _ptr(temperature), _ptr(top_k),
+          _ptr(top_p), _ptr(min_p), _ptr(repetition), _ptr(presence), _ptr(frequency), _ptr(ids), _ptr(id_start),
+          _ptr(counts), _stream())
+
+
 # ----------------------------------------------------------------------------- what the machine gives
 
 def measure_ceilings(device="cuda:0", read_bytes=1 << 30, repeats=5):

@@ -3,8 +3,8 @@
 Order of the reference's pipeline (crates/synaptix-models/llm/common/src/generate.rs:304-340):
 repetition penalty, presence/frequency penalty, temperature, top-k, top-p, min-p, then greedy
 (temperature <= 0) or multinomial.  The reference does all of it on the host from a downloaded
-vector (generate.rs:124-144); here the logits stay on the device.  Greedy and temperature
-sampling are one hand-written kernel; the filters run as device tensor operations in front of it.
+vector (generate.rs:124-144); here the logits stay on the device: the processors are one kernel for
+the batch (ops.filter_rows), greedy and temperature sampling another (ops.sample_rows).
 """
 from __future__ import annotations
 
@@ -33,44 +33,45 @@ class SequenceSampler:
             self.context.append(token)
 
 
-def apply_filters(row: torch.Tensor, cfg: GenerationConfig, penalty_ids) -> torch.Tensor:
-    """One row of float logits through the processors that are switched on; returns a new row."""
-    x = row.clone()
-    V = x.numel()
-    if cfg.penalties_on and len(penalty_ids):
-        ids = torch.as_tensor([t for t in penalty_ids if 0 <= t < V], dtype=torch.long, device=x.device)
-        counts = torch.bincount(ids, minlength=V).to(torch.float32)
-        seen = counts > 0
-        if cfg.repetition_penalty != 1.0:
-            # applied once for each occurrence: positive logits are divided, the others multiplied
-            # (crates/synaptix-infer/src/sampling/repetition.rs:27-45)
-            f = torch.pow(torch.tensor(cfg.repetition_penalty, dtype=torch.float32, device=x.device), counts)
-            x = torch.where(seen, torch.where(x > 0, x / f, x * f), x)
-        if cfg.presence_penalty != 0.0 or cfg.frequency_penalty != 0.0:
-            # repetition.rs:59-77
-            x = torch.where(seen, x - (cfg.presence_penalty + cfg.frequency_penalty * counts), x)
-    if cfg.temperature > 0.0 and cfg.temperature != 1.0:
-        x = x / torch.tensor(cfg.temperature, dtype=torch.float32, device=x.device)
-    if 0 < cfg.top_k < V:
-        # keep the k largest (crates/synaptix-infer/src/sampling/top_k.rs:8-24); equal values at the
-        # k-th place are all kept, where the reference keeps an arbitrary k of them
-        kth = torch.topk(x, cfg.top_k).values[-1]
-        x = torch.where(x < kth, torch.full_like(x, float("-inf")), x)
-    if cfg.top_p < 1.0:
-        # sorted by probability, a candidate stays while the sum before it is <= p * total
-        # (crates/synaptix-infer/src/sampling/top_p.rs:8-44)
-        probs = torch.exp(x - x.max())
-        order = torch.argsort(probs, descending=True, stable=True)
-        sp = probs[order]
-        before = torch.cumsum(sp, 0) - sp
-        drop = order[(before > cfg.top_p * probs.sum()) & torch.isfinite(x[order])]
-        x[drop] = float("-inf")
-    if cfg.min_p > 0.0:
-        # crates/synaptix-infer/src/sampling/min_p.rs:8-24
-        e = torch.exp(x - x.max())
-        pr = e / e.sum()
-        x = torch.where(pr < cfg.min_p * pr.max(), torch.full_like(x, float("-inf")), x)
-    return x
+_ZEROED = {}      # device -> int32 counters of the penalties, zero between calls
+
+
+def _counters(device, n: int) -> torch.Tensor:
+    t = _ZEROED.get(str(device))
+    if t is None or t.numel() < n:
+        t = _ZEROED[str(device)] = torch.zeros(n, dtype=torch.int32, device=device)
+    return t
+
+
+def filter_batch(logits: torch.Tensor, configs: list, penalty_ids: list) -> torch.Tensor:
+    """logits [B, V] float on the device through the processors that each row's GenerationConfig switches on
+    (ops.filter_rows: one kernel for the batch); returns new rows, divided by the temperature where it is
+    positive.  penalty_ids[r]: the tokens that row r's penalties look at."""
+    B, V = logits.shape
+    dev = logits.device
+
+    def column(values, dtype):
+        return torch.tensor(values, dtype=dtype).to(dev)
+
+    ids, starts = [], [0]
+    for cfg, row_ids in zip(configs, penalty_ids):
+        if cfg.penalties_on:
+            ids += [int(t) for t in row_ids]
+        starts.append(len(ids))
+    out = torch.empty_like(logits)
+    ops.filter_rows(
+        logits, out,
+        column([float(c.temperature) for c in configs], torch.float32),
+        column([int(c.top_k) if 0 < c.top_k < V else 0 for c in configs], torch.int32),
+        column([float(c.top_p) for c in configs], torch.float32),
+        column([float(c.min_p) for c in configs], torch.float32),
+        column([float(c.repetition_penalty) if c.penalties_on else 1.0 for c in configs], torch.float32),
+        column([float(c.presence_penalty) if c.penalties_on else 0.0 for c in configs], torch.float32),
+        column([float(c.frequency_penalty) if c.penalties_on else 0.0 for c in configs], torch.float32),
+        column(ids, torch.int32) if ids else None,
+        column(starts, torch.int32) if ids else None,
+        _counters(dev, B * V) if ids else None)
+    return out
 
 
 def sample_batch(logits: torch.Tensor, samplers: list) -> list:
@@ -78,11 +79,7 @@ def sample_batch(logits: torch.Tensor, samplers: list) -> list:
     B = logits.shape[0]
     assert B == len(samplers)
     if not all(s.config.plain for s in samplers):
-        rows = []
-        for r, s in enumerate(samplers):
-            rows.append(logits[r] if s.config.plain and not (s.config.temperature > 0 and s.config.temperature != 1.0)
-                        else apply_filters(logits[r], s.config, s.penalty_ids()))
-        logits = torch.stack(rows).contiguous()
+        logits = filter_batch(logits.contiguous(), [s.config for s in samplers], [s.penalty_ids() for s in samplers])
         temps = [1.0 if s.config.temperature > 0 else 0.0 for s in samplers]   # already divided
     else:
         temps = [float(s.config.temperature) for s in samplers]

@@ -244,8 +244,43 @@ def sample_rows(logits, temperature, uniform, out):
         out[r] = int(hit[0]) if hit.numel() else x.numel() - 1
 
 
+def filter_rows(logits, out, temperature, top_k, top_p, min_p, repetition, presence, frequency,
+                ids=None, id_start=None, counts=None):
+    R, V = logits.shape
+    for r in range(R):
+        x = logits[r].clone()
+        row_ids = [] if ids is None else [int(t) for t in ids[int(id_start[r]):int(id_start[r + 1])]]
+        rep, pres, freq = float(repetition[r]), float(presence[r]), float(frequency[r])
+        if row_ids and (rep != 1.0 or pres != 0.0 or freq != 0.0):
+            cnt = torch.bincount(torch.tensor([t for t in row_ids if 0 <= t < V], dtype=torch.long), minlength=V).to(F32)
+            seen = cnt > 0
+            if rep != 1.0:
+                f = torch.pow(torch.tensor(rep, dtype=F32), cnt)
+                x = torch.where(seen, torch.where(x > 0, x / f, x * f), x)
+            if pres != 0.0 or freq != 0.0:
+                x = torch.where(seen, x - (pres + freq * cnt), x)
+        T = float(temperature[r])
+        if T > 0.0 and T != 1.0:
+            x = x / torch.tensor(T, dtype=F32)
+        k = int(top_k[r])
+        if 0 < k < V:
+            order = torch.argsort(x, descending=True, stable=True)        # equal values: the first in index order
+            x[order[k:]] = float("-inf")
+        if float(top_p[r]) < 1.0:
+            probs = torch.exp(x - x.max())
+            order = torch.argsort(probs, descending=True, stable=True)
+            sp = probs[order]
+            before = torch.cumsum(sp, 0) - sp
+            drop = order[(before > float(top_p[r]) * probs.sum()) & torch.isfinite(x[order])]
+            x[drop] = float("-inf")
+        if float(min_p[r]) > 0.0:
+            e = torch.exp(x - x.max())
+            x = torch.where(torch.isfinite(x) & (e < float(min_p[r])), torch.full_like(x, float("-inf")), x)
+        out[r] = x
+
+
 ALL = ["embed", "add_rmsnorm", "rmsnorm_rows", "swiglu", "gemm", "gemm_swiglu", "gemm_packed", "stream_scope", "gemm_slices", "qk_norm_rope_kv_write", "attention_f32",
-       "attention_prefill_bf16", "decode_splits", "attention_decode_bf16", "attention_decode_fused_bf16", "sample_rows"]
+       "attention_prefill_bf16", "decode_splits", "attention_decode_bf16", "attention_decode_fused_bf16", "sample_rows", "filter_rows"]
 
 
 def install(monkeypatch):

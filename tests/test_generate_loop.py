@@ -7,7 +7,7 @@ import cpu_kernels
 from synaptix_amd.cache import SequenceCache
 from synaptix_amd.engine.generate import generate, plan_batch, GenerationConfig
 from synaptix_amd.parts import KvNeed
-from synaptix_amd.sampling import Philox4x32, SequenceSampler, apply_filters
+from synaptix_amd.sampling import Philox4x32, SequenceSampler, filter_batch
 import plain_qwen3 as P
 
 V = 50
@@ -182,26 +182,37 @@ def test_philox_matches_the_known_answer_and_the_plain_stream():
     assert 0.0 <= u < 1.0
 
 
-def test_filters_equal_the_plain_ones():
+def test_options_reach_the_filters_as_the_plain_ones_apply_them(monkeypatch):
+    """What a GenerationConfig and a context become on their way to the filter kernel (here its stand-in on the
+    CPU): which tokens the penalties see (the last repeat_last_n), which options are on, row by row of a batch
+    whose rows have different options."""
+    import cpu_kernels
+    cpu_kernels.install(monkeypatch)
     g = torch.Generator().manual_seed(0)
-    for trial in range(20):
-        x = torch.randn(200, generator=g) * 3
-        ids = torch.randint(0, 200, (30,), generator=g).tolist()
-        cfg = GenerationConfig(temperature=0.8, top_k=[0, 17][trial % 2], top_p=[1.0, 0.85][(trial // 2) % 2],
-                               min_p=[0.0, 0.02][(trial // 4) % 2], repetition_penalty=1.2, presence_penalty=0.3,
-                               frequency_penalty=0.1, repeat_last_n=[0, 10][trial % 2])
-        s = SequenceSampler(cfg, ids)
-        got = apply_filters(x, cfg, s.penalty_ids())
-        want = x.clone()
-        want = P.repetition_penalty(want, ids, 1.2, cfg.repeat_last_n)
-        want = P.presence_frequency(want, ids, 0.3, 0.1, cfg.repeat_last_n)
-        want = want / torch.tensor(0.8)
-        if cfg.top_k:
-            want = P.top_k(want, cfg.top_k)
-        if cfg.top_p < 1:
-            want = P.top_p(want, cfg.top_p)
-        if cfg.min_p > 0:
-            want = P.min_p(want, cfg.min_p)
-        assert torch.equal(torch.isinf(got), torch.isinf(want))
-        keep = ~torch.isinf(want)
-        assert torch.allclose(got[keep], want[keep], atol=1e-6)
+    for trial in range(10):
+        rows, cfgs, ctxs = [], [], []
+        for r in range(3):
+            t = 3 * trial + r
+            rows.append(torch.randn(200, generator=g) * 3)
+            ctxs.append(torch.randint(0, 200, (30,), generator=g).tolist())
+            cfgs.append(GenerationConfig(temperature=[0.8, 1.0, 0.0][r], top_k=[0, 17][t % 2], top_p=[1.0, 0.85][(t // 2) % 2],
+                                         min_p=[0.0, 0.02][(t // 4) % 2], repetition_penalty=[1.2, 1.0][r % 2],
+                                         presence_penalty=0.3, frequency_penalty=[0.1, 0.0][t % 2], repeat_last_n=[0, 10][t % 2]))
+        samplers = [SequenceSampler(c, ids) for c, ids in zip(cfgs, ctxs)]
+        got = filter_batch(torch.stack(rows), cfgs, [s.penalty_ids() for s in samplers])
+        for r, (x, cfg, ids) in enumerate(zip(rows, cfgs, ctxs)):
+            want = x.clone()
+            if cfg.repetition_penalty != 1.0:
+                want = P.repetition_penalty(want, ids, cfg.repetition_penalty, cfg.repeat_last_n)
+            want = P.presence_frequency(want, ids, cfg.presence_penalty, cfg.frequency_penalty, cfg.repeat_last_n)
+            if cfg.temperature > 0 and cfg.temperature != 1.0:
+                want = want / torch.tensor(cfg.temperature)
+            if cfg.top_k:
+                want = P.top_k(want, cfg.top_k)
+            if cfg.top_p < 1:
+                want = P.top_p(want, cfg.top_p)
+            if cfg.min_p > 0:
+                want = P.min_p(want, cfg.min_p)
+            assert torch.equal(torch.isinf(got[r]), torch.isinf(want)), (trial, r)
+            keep = ~torch.isinf(want)
+            assert torch.allclose(got[r][keep], want[keep], atol=1e-6)

@@ -1016,6 +1016,156 @@ def test_sample_rows_frequencies(ops):
     assert (freq - p).abs().max() < 0.012
 
 
+def _filter(ops, x, options, ids=None, in_place=False):
+    """ops.filter_rows over rows x [R, V] with options = list of dicts (k, p, mp, T, rep, pres, freq) and ids = list of lists."""
+    R, V = x.shape
+    col = lambda key, default, dt: torch.tensor([o.get(key, default) for o in options], dtype=dt).to(DEV)
+    flat, starts = [], [0]
+    for r in range(R):
+        flat += list(ids[r]) if ids else []
+        starts.append(len(flat))
+    xd = x.to(DEV).contiguous()
+    out = xd if in_place else torch.full_like(xd, float("nan"))
+    counts = torch.zeros(R * V, dtype=I32, device=DEV) if flat else None
+    ops.filter_rows(xd, out, col("T", 1.0, F32), col("k", 0, I32), col("p", 1.0, F32), col("mp", 0.0, F32),
+                    col("rep", 1.0, F32), col("pres", 0.0, F32), col("freq", 0.0, F32),
+                    torch.tensor(flat, dtype=I32).to(DEV) if flat else None,
+                    torch.tensor(starts, dtype=I32).to(DEV) if flat else None, counts)
+    torch.cuda.synchronize()
+    if counts is not None:
+        assert int(counts.abs().sum()) == 0, "the penalties' counters are not left zero"
+    return out.cpu()
+
+
+def _plain_filter(x, o, ids):
+    """The plain processors in the reference's order (tests/plain_qwen3.py)."""
+    import plain_qwen3 as P
+    want = x.clone()
+    if o.get("rep", 1.0) != 1.0:
+        want = P.repetition_penalty(want, ids, o["rep"], 0)
+    if o.get("pres", 0.0) != 0.0 or o.get("freq", 0.0) != 0.0:
+        want = P.presence_frequency(want, ids, o.get("pres", 0.0), o.get("freq", 0.0), 0)
+    T = o.get("T", 1.0)
+    if T > 0 and T != 1.0:
+        want = want / torch.tensor(T, dtype=F32)
+    if o.get("k", 0):
+        want = P.top_k(want, o["k"])
+    if o.get("p", 1.0) < 1.0:
+        want = P.top_p(want, o["p"]) if o["p"] <= 0.9 else _top_p_in_64_bit(want, o["p"])
+    if o.get("mp", 0.0) > 0.0:
+        want = P.min_p(want, o["mp"])
+    return want
+
+
+def _top_p_in_64_bit(x, p):
+    """The rule of the plain top_p (a candidate stays while the sum of those before it is at most p * the sum of
+    all; sorted by probability, equal ones in index order) with sums in 64-bit.  The reference adds up in 32-bit,
+    one candidate after the other (crates/synaptix-infer/src/sampling/top_p.rs:31-40): deep in the tail of a large
+    vocabulary a candidate is less than half a unit in the last place of that sum, the sum stands still and the
+    cut is never reached; the kernel's sums are exact, so for p near 1 it is held against the rule, not against
+    that rounding."""
+    probs = torch.exp(x.double() - x.max().double())
+    order = torch.argsort(probs, descending=True, stable=True)
+    sp = probs[order]
+    before = torch.cumsum(sp, 0) - sp
+    out = x.clone()
+    out[order[(before > p * probs.sum()) & torch.isfinite(x[order])]] = float("-inf")
+    return out
+
+
+@pytest.mark.parametrize("V", [97, 1000, 40000])
+def test_filter_rows_against_the_plain_processors(ops, V):
+    """Every processor alone and all together, rows with different options in one launch, against the plain
+    processors: the same entries dropped, the kept ones equal up to the rounding of the penalty's power."""
+    options = [dict(k=1), dict(k=17), dict(k=V - 1), dict(k=V), dict(p=0.9), dict(p=0.3), dict(p=0.999), dict(mp=0.05),
+               dict(T=0.7), dict(T=0.0, k=5), dict(rep=1.3), dict(pres=0.4, freq=0.2), dict(rep=0.8, pres=-0.1),
+               dict(T=0.8, k=40, p=0.85, mp=0.02, rep=1.2, pres=0.3, freq=0.1), dict(T=1.5, k=300, p=0.5), dict()]
+    R = len(options)
+    x = rnd((R, V), 90, scale=3.0)
+    g = torch.Generator().manual_seed(V)
+    ids = [torch.randint(-2, V + 3, (60,), generator=g).tolist() for _ in range(R)]       # some ids lie outside the vocabulary
+    for r in range(R):
+        ids[r] += ids[r][:20]                                                              # and some come several times
+    got = _filter(ops, x, options, ids)
+    for r, o in enumerate(options):
+        want = _plain_filter(x[r], o, [t for t in ids[r] if t >= 0])
+        differ = torch.isinf(got[r]) != torch.isinf(want)
+        if o.get("p", 1.0) > 0.9 and bool(differ.any()):
+            # deep in the tail neighbours in the sorted order lie 1e-8 of the mass apart, less than the rounding of
+            # a 32-bit exponential: an entry may fall on the other side only if it stands that close to the cut
+            probs = torch.exp(x[r].double() - x[r].max().double())
+            above = torch.stack([probs[probs > probs[j]].sum() for j in differ.nonzero().flatten()]) / probs.sum()
+            assert int(differ.sum()) <= 2 and bool(((above - o["p"]).abs() < 1e-6).all()), (r, o, above)
+            want = torch.where(differ, got[r], want)
+        assert torch.equal(torch.isinf(got[r]), torch.isinf(want)), (r, o, int(differ.sum()))
+        keep = ~torch.isinf(want)
+        close(got[r][keep], want[keep], 1e-5, 1e-5, what=f"kept logits of row {r}")
+    again = _filter(ops, x, options, ids, in_place=True)
+    assert torch.equal(torch.nan_to_num(again, neginf=-1e30), torch.nan_to_num(got, neginf=-1e30)), "in place, and the same bits twice"
+
+
+def test_filter_rows_with_equal_values(ops):
+    """Equal values at the k-th place and at the boundary of the probability mass: of equal entries the first in
+    index order stay, so that top-k keeps exactly k; rows of one value only; rows that are -inf but for a few."""
+    V = 5000
+    g = torch.Generator().manual_seed(3)
+    coarse = torch.randint(-4, 5, (V,), generator=g).float()              # nine values, hundreds of each
+    flat = torch.full((V,), 1.5)
+    few = torch.full((V,), float("-inf"))
+    few[[7, 4000, 123]] = torch.tensor([2.0, 1.0, 2.0])
+    x = torch.stack([coarse, coarse, coarse, flat, flat, few, few, coarse])
+    options = [dict(k=50), dict(k=900), dict(p=0.6), dict(k=3), dict(p=0.5), dict(k=2), dict(p=0.7), dict(k=700, p=0.8, mp=0.2)]
+    got = _filter(ops, x, options)
+
+    def first_k(row, k):
+        order = torch.argsort(row, descending=True, stable=True)
+        keep = torch.zeros(V, dtype=torch.bool)
+        keep[order[:k]] = True
+        return keep
+
+    def first_by_mass(row, p):
+        probs = torch.exp(row.double() - row.max().double())
+        order = torch.argsort(probs, descending=True, stable=True)
+        sp = probs[order]
+        before = torch.cumsum(sp, 0) - sp
+        keep = torch.zeros(V, dtype=torch.bool)
+        keep[order[(before <= p * probs.sum()) & torch.isfinite(row[order])]] = True
+        return keep
+
+    kept = ~torch.isinf(got)
+    assert torch.equal(kept[0], first_k(coarse, 50)) and int(kept[0].sum()) == 50
+    assert torch.equal(kept[1], first_k(coarse, 900)) and int(kept[1].sum()) == 900
+    assert torch.equal(kept[2], first_by_mass(coarse, 0.6))
+    assert kept[3].nonzero().flatten().tolist() == [0, 1, 2]
+    assert torch.equal(kept[4], first_by_mass(flat, 0.5)) and int(kept[4].sum()) == V // 2 + 1
+    assert kept[5].nonzero().flatten().tolist() == [7, 123]
+    assert kept[6].nonzero().flatten().tolist() == [7, 123]            # 2/(2e^2+e) of the mass before the second, 0.84 before the third
+    both = first_k(coarse, 700)
+    row = torch.where(both, coarse, torch.full_like(coarse, float("-inf")))
+    both &= first_by_mass(row, 0.8)
+    both &= torch.exp(coarse - coarse.max()) >= 0.2
+    assert torch.equal(kept[7], both)
+    assert torch.equal(got[kept], x[kept])                                # what stays is untouched
+
+
+def test_filter_rows_at_the_vocabulary_of_the_large_models(ops):
+    """151,936 logits a row, as the models' output head gives them; a sampled token after the filters lies among
+    the entries that were kept."""
+    import plain_qwen3 as P
+    V = 151936
+    x = rnd((3, V), 95, scale=2.5)
+    options = [dict(T=0.7, k=50, p=0.9), dict(p=0.95, mp=0.001), dict(T=0.9, k=2000, rep=1.1)]
+    ids = [list(range(100, 400)) * 2, [], [5, 5, 5, 9]]
+    got = _filter(ops, x, options, ids)
+    for r, o in enumerate(options):
+        want = _plain_filter(x[r], o, ids[r])
+        assert torch.equal(torch.isinf(got[r]), torch.isinf(want)), (r, int((torch.isinf(got[r]) != torch.isinf(want)).sum()))
+    out = torch.empty(3, dtype=I32, device=DEV)
+    ops.sample_rows(got.to(DEV), torch.ones(3).to(DEV), torch.tensor([0.3, 0.999, 0.0]).to(DEV), out)
+    for r, t in enumerate(out.cpu().tolist()):
+        assert math.isfinite(float(got[r, t]))
+
+
 def test_measured_ceilings_are_plausible(ops):
     """The two probes run and report rates of the right order for this kind of machine."""
     read_gbs, mfma_tflops = ops.measure_ceilings(DEV, read_bytes=1 << 28, repeats=2)
