@@ -297,6 +297,26 @@ def check_greedy_path(plain, prompt, got, want, margin=2e-2):
             return
 
 
+def generation_with_every_processor(make_engine, name):
+    """Penalties over the last tokens, temperature, top-k, top-p and min-p together, two requests with streams of
+    their own, in 32-bit: the tokens are the plain implementation's (its processors in the reference's order on
+    the plain logits, the same uniform numbers).  What a request's penalties see grows with the tokens it has
+    drawn, and a wrong window, a processor out of order or a row's options given to its neighbour changes the
+    draws within a few tokens."""
+    V = CONFIGS[name]["vocab_size"]
+    options = dict(temperature=0.9, k=12, p=0.9, mp=0.02, repetition=1.3, last_n=6, presence=0.2, frequency=0.1)
+    cfg = GenerationConfig(max_new_tokens=14, temperature=0.9, top_k=12, top_p=0.9, min_p=0.02, repetition_penalty=1.3,
+                           repeat_last_n=6, presence_penalty=0.2, frequency_penalty=0.1, seed=5)
+    prompts = [random_tokens(V, n, 400 + i) for i, n in enumerate((9, 30))]
+    plain = plain_model(name)
+    eng = make_engine(name, "float32", 1024, False)
+    outs, _ = generate(eng, prompts, cfg)
+    for i, (p, o) in enumerate(zip(prompts, outs)):
+        want = P.generate(plain, p, 14, seed=5 + i, **options)
+        assert o.tokens == want, f"request {i}: {o.tokens} vs {want}"
+    eng.cache.check()
+
+
 def sampled_generation(make_engine, name, dtype):
     """Temperature sampling with per-sequence streams: the tiny configuration B at temperature 0.7 and seed 1.
     In float32 the tokens are the plain implementation's.  In bfloat16 a draw may fall on the other

@@ -51,6 +51,7 @@ def test_decode_beside_a_fresh_prompt_and_prompts_in_chunks():
 def test_greedy_and_sampled_generation():
     scenarios.greedy_generation(make_engine, "A", "float32", n_new=5)
     scenarios.sampled_generation(make_engine, "B", "float32")
+    scenarios.generation_with_every_processor(make_engine, "A")
 
 
 def test_step_errors():

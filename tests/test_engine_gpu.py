@@ -127,6 +127,11 @@ def test_sampled_generation(dtype):
     scenarios.sampled_generation(make_engine, "B", dtype)
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_generation_with_every_processor(name):
+    scenarios.generation_with_every_processor(make_engine, name)
+
+
 def test_batch_rows_do_not_depend_on_their_neighbours():
     """The same request alone, and between others in another slot and other pages."""
     for dtype in DTYPES:
