@@ -144,6 +144,7 @@ SYN_EXPORT int syn_sample_rows(const float* logits, const float* temperature, co
 // passes over the row with a histogram of 256 bins in LDS), and the sums are integers (probabilities in 44-bit
 // fixed point), so that a row gives the same result whatever the order in which threads arrive.
 #define FILTER_THREADS 1024
+#define FILTER_LIST 2048
 typedef unsigned long long u64;
 
 // the float's bits as an unsigned number that grows with the float
@@ -163,6 +164,9 @@ struct FilterShared {
   int bin;
   unsigned need;
   u64 above;
+  // what top-k has left, if that is little: the processors behind it then walk this list, not the row
+  int cand_j[FILTER_LIST];
+  int n_cand;
 };
 
 __device__ __forceinline__ float block_max_all(float v, float* red) {
@@ -188,6 +192,25 @@ __device__ __forceinline__ u64 block_sum_all(u64 v, u64* red) {
   return t;
 }
 
+// For the lanes of one wave, lane l holding bins 4 l .. 4 l + 3 of a histogram: above[i] = the sum of all bins above
+// bin 4 l + i.
+template <typename T>
+__device__ __forceinline__ void sums_above(const T* hist, int lane, T (&mine)[4], T (&above)[4]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) mine[i] = hist[4 * lane + i];
+  const T own = mine[0] + mine[1] + mine[2] + mine[3];
+  T from_here = own;   // becomes the sum over this lane and all higher ones
+#pragma unroll
+  for (int off = 1; off < SYN_WAVE; off <<= 1) {
+    const T o = __shfl_down(from_here, off, SYN_WAVE);
+    if (lane + off < SYN_WAVE) from_here += o;
+  }
+  above[3] = from_here - own;
+  above[2] = above[3] + mine[3];
+  above[1] = above[2] + mine[2];
+  above[0] = above[1] + mine[1];
+}
+
 // A thread's additions to the histogram go through one bin kept in registers: logits share their top bytes, and
 // a thousand threads adding to the same few LDS words one by one would take longer than the pass itself.
 struct BinCache {
@@ -210,7 +233,7 @@ struct BinCache {
   }
 };
 
-// A pass over a row: f(j, x[j]) for every entry, 16 bytes a load and four loads of a thread under way where the row
+// A pass over a row: f(j, x[j]) for every entry, 16 bytes a load and eight loads of a thread under way where the row
 // allows it (one entry at a time, a pass of one workgroup over 150,000 entries waits 150 times for memory).
 template <typename F>
 __device__ __forceinline__ void for_each_entry(const float* x, int V, F f) {
@@ -218,12 +241,12 @@ __device__ __forceinline__ void for_each_entry(const float* x, int V, F f) {
   if (V % 4 == 0 && (uintptr_t)x % 16 == 0) {
     const float4* x4 = (const float4*)x;
     const int V4 = V / 4;
-    for (int i0 = tid; i0 < V4; i0 += 4 * nt) {
-      float4 v[4];
+    for (int i0 = tid; i0 < V4; i0 += 8 * nt) {
+      float4 v[8];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) v[q] = i0 + q * nt < V4 ? x4[i0 + q * nt] : make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int q = 0; q < 8; ++q) v[q] = i0 + q * nt < V4 ? x4[i0 + q * nt] : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
+      for (int q = 0; q < 8; ++q)
         if (i0 + q * nt < V4) {
           const int j = 4 * (i0 + q * nt);
           f(j, v[q].x), f(j + 1, v[q].y), f(j + 2, v[q].z), f(j + 3, v[q].w);
@@ -233,7 +256,7 @@ __device__ __forceinline__ void for_each_entry(const float* x, int V, F f) {
     for (int j = tid; j < V; j += nt) f(j, x[j]);
   }
 }
-// The same with a new value for every entry: dst[j] = f(src[j]) (dst may be src).
+// The same with a new value for every entry: dst[j] = f(j, src[j]) (dst may be src).
 template <typename F>
 __device__ __forceinline__ void map_entries(const float* src, float* dst, int V, F f) {
   const int tid = threadIdx.x, nt = blockDim.x;
@@ -247,10 +270,13 @@ __device__ __forceinline__ void map_entries(const float* src, float* dst, int V,
       for (int q = 0; q < 4; ++q) v[q] = i0 + q * nt < V4 ? s4[i0 + q * nt] : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
       for (int q = 0; q < 4; ++q)
-        if (i0 + q * nt < V4) d4[i0 + q * nt] = make_float4(f(v[q].x), f(v[q].y), f(v[q].z), f(v[q].w));
+        if (i0 + q * nt < V4) {
+          const int j = 4 * (i0 + q * nt);
+          d4[i0 + q * nt] = make_float4(f(j, v[q].x), f(j + 1, v[q].y), f(j + 2, v[q].z), f(j + 3, v[q].w));
+        }
     }
   } else {
-    for (int j = tid; j < V; j += nt) dst[j] = f(src[j]);
+    for (int j = tid; j < V; j += nt) dst[j] = f(j, src[j]);
   }
 }
 
@@ -292,7 +318,7 @@ filter_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int V,
   const float rep = repetition[row], pres = presence[row], freq = frequency[row];
   if (n_ids > 0 && (rep != 1.f || pres != 0.f || freq != 0.f)) {
     if (src != x) {
-      map_entries(src, x, V, [](float v) { return v; });
+      map_entries(src, x, V, [](int, float v) { return v; });
       src = x;
       __syncthreads();
     }
@@ -330,7 +356,7 @@ filter_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int V,
   const bool scale = T > 0.f && T != 1.f;
   float m = -INFINITY;
   if (scale || src != x) {
-    map_entries(src, x, V, [&](float v) {
+    map_entries(src, x, V, [&](int, float v) {
       if (scale) v = v / T;
       m = fmaxf(m, v);
       return v;
@@ -342,6 +368,7 @@ filter_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int V,
 
   // ---- top-k: the key of the k-th largest, a byte at a time
   const int k = top_k[row];
+  bool listed = false;
   if (k > 0 && k < V) {
     unsigned prefix = 0, need = (unsigned)k, ties = 0;
     for (int shift = 24; shift >= 0; shift -= 8) {
@@ -355,30 +382,60 @@ filter_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int V,
       });
       cache.flush(sh, false);
       __syncthreads();
-      if (tid == 0) {
-        unsigned seen = 0;
-        int b = 255;
-        for (; b > 0; --b) {
-          if (seen + sh.cnt[b] >= need) break;
-          seen += sh.cnt[b];
-        }
-        sh.bin = b, sh.need = need - seen;
+      if (tid < SYN_WAVE) {
+        // the bin in which the need-th largest of the matching entries lies (there are at least `need` of them)
+        unsigned mine[4], above[4];
+        sums_above(sh.cnt, tid, mine, above);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (above[i] < need && need <= above[i] + mine[i]) sh.bin = 4 * tid + i, sh.need = need - above[i];
       }
       __syncthreads();
       prefix |= (unsigned)sh.bin << shift, need = sh.need, ties = sh.cnt[sh.bin];
       __syncthreads();
     }
-    // below the k-th key everything goes; of its equals the first `need` stay
-    map_entries(x, x, V, [&](float v) { return order_key(v) < prefix ? -INFINITY : v; });
+    // below the k-th key everything goes; of its equals the first `need` stay.  If processors follow and little is
+    // left, what stays is listed in LDS (in no order) for them.
+    const bool list = (top_p[row] < 1.f || min_p[row] > 0.f) && (unsigned)k - need + ties <= FILTER_LIST;
+    if (tid == 0) sh.n_cand = 0;
+    __syncthreads();
+    map_entries(x, x, V, [&](int j, float v) {
+      if (order_key(v) < prefix) return -INFINITY;
+      if (list) {
+        const int i = atomicAdd(&sh.n_cand, 1);
+        sh.cand_j[i] = j;
+      }
+      return v;
+    });
     __syncthreads();
     if (need < ties) drop_later_ties(x, V, prefix, need, sh);
+    listed = list;
   }
+  // a pass over what is left: f(j, value) for the listed entries or for the whole row
+  const int n_listed = listed ? sh.n_cand : 0;
+  auto each_left = [&](auto f) {
+    if (listed) {
+      for (int i = tid; i < n_listed; i += nt) f(sh.cand_j[i], x[sh.cand_j[i]]);
+    } else {
+      for_each_entry(x, V, f);
+    }
+  };
+  auto drop_left = [&](auto gone) {   // gone(value): whether the entry goes
+    if (listed) {
+      for (int i = tid; i < n_listed; i += nt) {
+        const int j = sh.cand_j[i];
+        if (gone(x[j])) x[j] = -INFINITY;
+      }
+    } else {
+      map_entries(x, x, V, [&](int, float v) { return gone(v) ? -INFINITY : v; });
+    }
+  };
 
   // ---- top-p: the lowest key whose mass above it is at most p * all mass
   const float p = top_p[row];
   if (p < 1.f) {
     u64 mine = 0;
-    for_each_entry(x, V, [&](int, float v) {
+    each_left([&](int, float v) {
       if (is_finite(v)) mine += mass_of(v, m);
     });
     const u64 total = block_sum_all(mine, sh.red64);
@@ -390,24 +447,30 @@ filter_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int V,
       for (int b = tid; b < 256; b += nt) sh.cnt[b] = 0, sh.sum[b] = 0;
       __syncthreads();
       BinCache cache;
-      for_each_entry(x, V, [&](int, float v) {
+      each_left([&](int, float v) {
         if (!is_finite(v)) return;
         const unsigned key = order_key(v);
         if ((key & himask) == prefix) cache.add(sh, (key >> shift) & 255, mass_of(v, m), true);
       });
       cache.flush(sh, true);
       __syncthreads();
-      if (tid == 0) {
-        // from the top: a bin's largest entry has exactly the mass of the bins above it before it
-        u64 running = above, chosen_above = above;
-        int chosen = -1;
-        for (int b = 255; b >= 0; --b) {
-          if (!sh.cnt[b]) continue;
-          if (running > limit) break;
-          chosen = b, chosen_above = running;
-          running += sh.sum[b];
+      if (tid < SYN_WAVE) {
+        // a bin's largest entry has exactly the mass of the bins above it before it: the lowest bin that holds
+        // entries and has at most `limit` above it is where the boundary lies (every such bin above it stays whole)
+        u64 mine[4], over[4];
+        sums_above(sh.sum, tid, mine, over);
+        int lowest = 256;
+#pragma unroll
+        for (int i = 3; i >= 0; --i)
+          if (sh.cnt[4 * tid + i] && above + over[i] <= limit) lowest = 4 * tid + i;
+        int first = lowest;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) first = min(first, __shfl_xor(first, off, SYN_WAVE));
+        if (first == 256) {
+          if (tid == 0) sh.bin = -1;
+        } else if (first == lowest) {
+          sh.bin = first, sh.above = above + over[first % 4];
         }
-        sh.bin = chosen, sh.above = chosen_above;
       }
       __syncthreads();
       if (sh.bin < 0) break;   // no finite entry at all
@@ -415,7 +478,7 @@ filter_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int V,
       __syncthreads();
     }
     if (ties > 0) {
-      map_entries(x, x, V, [&](float v) { return is_finite(v) && order_key(v) < prefix ? -INFINITY : v; });
+      drop_left([&](float v) { return is_finite(v) && order_key(v) < prefix; });
       __syncthreads();
       // the j-th of equal entries has (j - 1) of them before it as well
       const u64 each = tie_mass / ties;
@@ -426,7 +489,7 @@ filter_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int V,
 
   // ---- min-p: the largest probability belongs to the largest logit, exp(0) = 1 before the division by the sum
   const float mp = min_p[row];
-  if (mp > 0.f) map_entries(x, x, V, [&](float v) { return is_finite(v) && expf(v - m) < mp ? -INFINITY : v; });
+  if (mp > 0.f) drop_left([&](float v) { return is_finite(v) && expf(v - m) < mp; });
 }
 
 // in, out [n_rows, V] float (may be the same); one entry a row of every option (top_k 0 and top_p >= 1: off);
