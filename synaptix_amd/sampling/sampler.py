@@ -49,28 +49,24 @@ def filter_batch(logits: torch.Tensor, configs: list, penalty_ids: list) -> torc
     positive.  penalty_ids[r]: the tokens that row r's penalties look at."""
     B, V = logits.shape
     dev = logits.device
-
-    def column(values, dtype):
-        return torch.tensor(values, dtype=dtype).to(dev)
-
     ids, starts = [], [0]
     for cfg, row_ids in zip(configs, penalty_ids):
         if cfg.penalties_on:
             ids += [int(t) for t in row_ids]
         starts.append(len(ids))
+    # two copies to the device: the float options column after column, and top_k, the rows' offsets and the tokens
+    floats = ([float(c.temperature) for c in configs] + [float(c.top_p) for c in configs] + [float(c.min_p) for c in configs]
+              + [float(c.repetition_penalty) if c.penalties_on else 1.0 for c in configs]
+              + [float(c.presence_penalty) if c.penalties_on else 0.0 for c in configs]
+              + [float(c.frequency_penalty) if c.penalties_on else 0.0 for c in configs])
+    ints = [int(c.top_k) if 0 < c.top_k < V else 0 for c in configs] + starts + ids
+    f = torch.tensor(floats, dtype=torch.float32).to(dev)
+    i = torch.tensor(ints, dtype=torch.int32).to(dev)
+    temperature, top_p, min_p, repetition, presence, frequency = (f[c * B:(c + 1) * B] for c in range(6))
     out = torch.empty_like(logits)
-    ops.filter_rows(
-        logits, out,
-        column([float(c.temperature) for c in configs], torch.float32),
-        column([int(c.top_k) if 0 < c.top_k < V else 0 for c in configs], torch.int32),
-        column([float(c.top_p) for c in configs], torch.float32),
-        column([float(c.min_p) for c in configs], torch.float32),
-        column([float(c.repetition_penalty) if c.penalties_on else 1.0 for c in configs], torch.float32),
-        column([float(c.presence_penalty) if c.penalties_on else 0.0 for c in configs], torch.float32),
-        column([float(c.frequency_penalty) if c.penalties_on else 0.0 for c in configs], torch.float32),
-        column(ids, torch.int32) if ids else None,
-        column(starts, torch.int32) if ids else None,
-        _counters(dev, B * V) if ids else None)
+    ops.filter_rows(logits, out, temperature, i[:B], top_p, min_p, repetition, presence, frequency,
+                    i[2 * B + 1:] if ids else None, i[B:2 * B + 1] if ids else None,
+                    _counters(dev, B * V) if ids else None)
     return out
 
 
