@@ -590,3 +590,139 @@ def test_toy_feed_forward_with_routing_registers_builds_and_steps(tmp_path):
     a = eng.acquire()
     cut = [eng.step([(a, ids[:4])], want="all")] + [eng.step([(a, [t])], want="last") for t in ids[4:]]
     assert (torch.cat(cut).cpu() - whole16).abs().max() <= 5e-2 * max(1.0, float(whole16.abs().max()))
+
+
+def test_toy_block_arrangement_and_toy_norm_register_build_and_step(tmp_path):
+    """Another arrangement of a layer and another norm, both defined here: a block in which mixer and feed-forward
+    read the same normed rows and their sums are added together (x <- x + mixer(n(x)) + ff(n(x))), beside a pre-norm
+    block in the same model; and a norm that takes the mean away before it scales (with a gain and a bias).  The
+    block keeps to the interface of blocks (the delta it is handed is added by its norm, the delta it returns is added by
+    whoever runs next), the norm to that of norms (add_apply with and without rows).  Registered, built from its own
+    config.json, loaded and stepped without a change to the package; whole prompts, pieces and single tokens agree
+    with a plain statement of the same model in both types."""
+    from dataclasses import dataclass, asdict
+    import json
+    from synaptix_amd import register_architecture, Engine
+    from synaptix_amd.models import DecoderModel, LayerRun, TokenEmbedding, OutputHead
+    from synaptix_amd.parts import Part, Block, RmsNorm, GatedMlp, PreNormBlock, GqaAttention, RotaryHalfSplit, as_delta
+    from synaptix_amd.weights import TensorSpec, save_file, RandomSource
+
+    class CenteredNorm(Part):
+        """y = gain * (x - mean) / sqrt(var + eps) + bias, in 32-bit; the residual sum in front of it as the package's norms have it."""
+        def __init__(self, name, dim, eps):
+            self.name, self.dim, self.eps = name, dim, eps
+
+        def tensor_specs(self):
+            return {self.name + ".gain": TensorSpec((self.dim,), "gain"), self.name + ".bias": TensorSpec((self.dim,))}
+
+        def load(self, get):
+            self.gain, self.bias = get(self.name + ".gain").float(), get(self.name + ".bias").float()
+
+        def add_apply(self, resid, delta, out_dtype, rows=None):
+            delta = as_delta(delta)
+            if delta is not None and delta.dim() == 3:
+                delta = delta.sum(0)
+            if rows is None:
+                if delta is not None:
+                    resid += delta
+                x = resid
+            else:
+                x = resid[rows.long()] + (0 if delta is None else delta[rows.long()])
+            c = x - x.mean(-1, keepdim=True)
+            return (self.gain * c * torch.rsqrt(c.square().mean(-1, keepdim=True) + self.eps) + self.bias).to(out_dtype)
+
+    class ParallelBlock(Block):
+        def __init__(self, norm, mixer, feed_forward):
+            self.norm, self.mixer, self.feed_forward = norm, mixer, feed_forward
+
+        def _parts(self):
+            return (self.norm, self.mixer, self.feed_forward)
+
+        def tensor_specs(self):
+            return {k: v for p in self._parts() for k, v in p.tensor_specs().items()}
+
+        def load(self, get):
+            for p in self._parts():
+                p.load(get)
+
+        def forward(self, resid, pending, ctx, cache, owner=True):
+            h = self.norm.add_apply(resid, pending, ctx.act_dtype)              # the delta of the layer before is added here
+            both = [as_delta(self.mixer.forward(h, ctx, cache, owner)), as_delta(self.feed_forward.forward(h, ctx))]
+            both = [d.sum(0) if d.dim() == 3 else d for d in both]                # (products may come as partial sums)
+            return both[0] + both[1]                                              # added by the norm that runs next
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        vocab_size: int = 83
+        hidden_size: int = 48
+        intermediate_size: int = 64
+        max_position_embeddings: int = 128
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(**{k: d[k] for k in cls.__dataclass_fields__ if k in d})
+
+        def to_dict(self):
+            return {**asdict(self), "architectures": ["ToyParallel"]}
+
+    def build(cfg, max_positions=None):
+        H = cfg.hidden_size
+        rope = RotaryHalfSplit(1e4, 16, cfg.max_position_embeddings)
+        blocks = [ParallelBlock(CenteredNorm("l0.n", H, 1e-5), GqaAttention("l0.att.", H, 3, 1, 16, position=rope),
+                                GatedMlp("l0.ff.", H, cfg.intermediate_size)),
+                  PreNormBlock(RmsNorm("l1.n1", H, 1e-5), GqaAttention("l1.att.", H, 3, 3, 16, position=rope),
+                               CenteredNorm("l1.n2", H, 1e-5), GatedMlp("l1.ff.", H, cfg.intermediate_size)),
+                  ParallelBlock(RmsNorm("l2.n", H, 1e-5), GqaAttention("l2.att.", H, 3, 1, 16, position=rope),
+                                GatedMlp("l2.ff.", H, cfg.intermediate_size))]
+        return DecoderModel(cfg, TokenEmbedding("emb", cfg.vocab_size, H), blocks, [LayerRun(l, l) for l in range(3)],
+                            CenteredNorm("norm", H, 1e-5), OutputHead("head", cfg.vocab_size, H))
+
+    register_architecture("ToyParallel", ToyConfig, build)
+    cfg = ToyConfig()
+    src = RandomSource(build(cfg).tensor_specs(), 21, std=0.25)
+    tensors = {n: src.tensor(n) for n in src.names()}
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    (tmp_path / "config.json").write_text(json.dumps(cfg.to_dict()))
+
+    def plain(ids):
+        t = {n: v.float() for n, v in tensors.items()}
+        S, cos_sin = len(ids), P.rope_tables(16, len(ids), 1e4)
+
+        def centered(x, name):
+            c = x - x.mean(-1, keepdim=True)
+            return t[name + ".gain"] * c * torch.rsqrt(c.square().mean(-1, keepdim=True) + 1e-5) + t[name + ".bias"]
+
+        def attend(xn, pre, nkv):
+            q = (xn @ t[pre + "q_proj.weight"].T).view(S, 3, 16)
+            k = (xn @ t[pre + "k_proj.weight"].T).view(S, nkv, 16)
+            v = (xn @ t[pre + "v_proj.weight"].T).view(S, nkv, 16)
+            q, k = P.apply_rope(q, *cos_sin, range(S)), P.apply_rope(k, *cos_sin, range(S))
+            return P.attention(q, k, v, 0.25, list(range(S))).reshape(S, 48) @ t[pre + "o_proj.weight"].T
+
+        def mlp(xn, pre):
+            return P.swiglu_mlp(xn, t[pre + "gate_proj.weight"], t[pre + "up_proj.weight"], t[pre + "down_proj.weight"])
+
+        x = t["emb"][ids]
+        n = centered(x, "l0.n")
+        x = x + attend(n, "l0.att.", 1) + mlp(n, "l0.ff.")
+        x = x + attend(P.rms_norm(x, t["l1.n1"], 1e-5), "l1.att.", 3)
+        x = x + mlp(centered(x, "l1.n2"), "l1.ff.")
+        n = P.rms_norm(x, t["l2.n"], 1e-5)
+        x = x + attend(n, "l2.att.", 1) + mlp(n, "l2.ff.")
+        return centered(x, "norm") @ t["head"].T
+
+    ids = [3, 17, 44, 9, 60, 21, 5, 38, 12, 50, 7, 80, 2]
+    want = plain(ids)
+    for dtype, tol in (("float32", 3e-4), ("bfloat16", 6e-2)):
+        eng = Engine.load(str(tmp_path), dtype=dtype, max_tokens=256, max_slots=2)
+        assert not eng.graph_ok                        # parts from elsewhere: every step is launched one by one
+        a = eng.acquire()
+        whole = eng.step([(a, ids)], want="all").cpu()
+        assert (whole - want).abs().max() <= tol * max(1.0, float(want.abs().max())), dtype
+        last = eng.step([(eng.acquire(), ids)], want=[[4, 12]]).cpu()             # wanted rows: the last norm with rows
+        assert (last - whole[[4, 12]]).abs().max() <= (1e-5 if dtype == "float32" else 2e-2)
+        eng.release(a)
+        a = eng.acquire()
+        cut = [eng.step([(a, ids[:5])], want="all"), eng.step([(a, ids[5:9])], want="all")]
+        cut += [eng.step([(a, [tok])], want="last") for tok in ids[9:]]
+        assert (torch.cat(cut).cpu() - whole).abs().max() <= (1e-4 if dtype == "float32" else 5e-2 * max(1.0, float(whole.abs().max())))
