@@ -61,6 +61,16 @@ def test_command_line_run_and_bench():
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert [int(t) for t in proc.stdout.split()] == want
     assert "12 prompt + 7 new tokens" in proc.stderr and "tok/s" in proc.stderr
+    # every sampling option of the command line, in 32-bit: the plain implementation's tokens for the same seed
+    want = P.generate(plain, prompt, 9, seed=4, temperature=0.8, k=15, p=0.9, mp=0.01, repetition=1.2, last_n=8,
+                      presence=0.1, frequency=0.05)
+    cmd = [sys.executable, "-m", "synaptix_amd", "run", folder, "--prompt-ids", ",".join(map(str, prompt)),
+           "--max-tokens", "9", "--temperature", "0.8", "--top-k", "15", "--top-p", "0.9", "--min-p", "0.01",
+           "--repetition-penalty", "1.2", "--repeat-last-n", "8", "--presence-penalty", "0.1",
+           "--frequency-penalty", "0.05", "--seed", "4", "--compute-dtype", "f32"]
+    proc = subprocess.run(cmd, capture_output=True, text=True, cwd=ROOT, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [int(t) for t in proc.stdout.split()] == want
     # no folder: a config.json alone with weights drawn from --seed, and the prompt several times in one batch
     cmd = [sys.executable, "-m", "synaptix_amd", "run", "--random", os.path.join(folder, "config.json"), "--seed", "3",
            "--prompt-ids", "5,6,7,8,9", "--max-tokens", "4", "--temperature", "0", "--batch", "3"]
