@@ -432,14 +432,10 @@ filter_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int V,
   };
 
   // ---- top-p: the lowest key whose mass above it is at most p * all mass
-  const float p = top_p[row];
+  const float p = top_p[row], mp = min_p[row];
+  bool min_p_done = false;
   if (p < 1.f) {
-    u64 mine = 0;
-    each_left([&](int, float v) {
-      if (is_finite(v)) mine += mass_of(v, m);
-    });
-    const u64 total = block_sum_all(mine, sh.red64);
-    const u64 limit = (u64)((double)p * (double)total);
+    u64 limit = 0;       // p * all mass; all mass is what the first histogram adds up to
     unsigned prefix = 0, ties = 0;
     u64 above = 0, tie_mass = 0;
     for (int shift = 24; shift >= 0; shift -= 8) {
@@ -459,6 +455,11 @@ filter_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int V,
         // entries and has at most `limit` above it is where the boundary lies (every such bin above it stays whole)
         u64 mine[4], over[4];
         sums_above(sh.sum, tid, mine, over);
+        if (shift == 24) {
+          const u64 total = __shfl(over[0] + mine[0], 0, SYN_WAVE);
+          limit = (u64)((double)p * (double)total);
+          if (tid == 0) sh.red64[0] = limit;
+        }
         int lowest = 256;
 #pragma unroll
         for (int i = 3; i >= 0; --i)
@@ -474,11 +475,14 @@ filter_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int V,
       }
       __syncthreads();
       if (sh.bin < 0) break;   // no finite entry at all
+      limit = sh.red64[0];
       prefix |= (unsigned)sh.bin << shift, above = sh.above, ties = sh.cnt[sh.bin], tie_mass = sh.sum[sh.bin];
       __syncthreads();
     }
     if (ties > 0) {
-      drop_left([&](float v) { return is_finite(v) && order_key(v) < prefix; });
+      // (min-p looks at each entry alone, so it goes along in this pass)
+      drop_left([&](float v) { return is_finite(v) && (order_key(v) < prefix || (mp > 0.f && expf(v - m) < mp)); });
+      min_p_done = true;
       __syncthreads();
       // the j-th of equal entries has (j - 1) of them before it as well
       const u64 each = tie_mass / ties;
@@ -488,8 +492,7 @@ filter_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int V,
   }
 
   // ---- min-p: the largest probability belongs to the largest logit, exp(0) = 1 before the division by the sum
-  const float mp = min_p[row];
-  if (mp > 0.f) drop_left([&](float v) { return is_finite(v) && expf(v - m) < mp; });
+  if (mp > 0.f && !min_p_done) drop_left([&](float v) { return is_finite(v) && expf(v - m) < mp; });
 }
 
 // in, out [n_rows, V] float (may be the same); one entry a row of every option (top_k 0 and top_p >= 1: off);
