@@ -70,6 +70,47 @@ def test_awkward_sizes(dtype):
     scenarios.unequal_batches(make_engine, "E", dtype)
 
 
+@pytest.mark.parametrize("seed", [0, 1])
+def test_random_configurations(seed, tmp_path):
+    """Configurations drawn at random, every size odd where it may be (head sizes 16 to 256, groups of 1 to 7 heads,
+    widths and intermediate sizes that are multiples of 8 and 2 only, any vocabulary, tied or not): several prompts
+    of unequal lengths in one step, then single tokens, against the plain implementation in both types."""
+    import random
+    from synaptix_amd import Qwen3Config, write_random_model, Engine
+    from plain_qwen3 import PlainQwen3
+    rnd = random.Random(seed)
+    for trial in range(4):
+        nkv = rnd.choice([1, 2, 3, 5])
+        raw = dict(vocab_size=rnd.randint(20, 700), hidden_size=8 * rnd.randint(3, 40), intermediate_size=2 * rnd.randint(5, 150),
+                   num_hidden_layers=rnd.randint(1, 3), num_attention_heads=nkv * rnd.choice([1, 2, 3, 4, 7]),
+                   num_key_value_heads=nkv, head_dim=rnd.choice([16, 32, 48, 64, 80, 96, 112, 128, 160, 256]),
+                   max_position_embeddings=512, rope_theta=rnd.choice([1e4, 1e6]), rms_norm_eps=rnd.choice([1e-6, 1e-5]),
+                   tie_word_embeddings=rnd.random() < 0.5, eos_token_id=None)
+        folder = str(tmp_path / f"m{trial}")
+        write_random_model(folder, Qwen3Config(**raw), seed=100 * seed + trial)
+        plain = PlainQwen3.from_folder(folder)
+        lens = [rnd.randint(1, 150) for _ in range(rnd.randint(1, 5))]
+        seqs = [random_tokens(raw["vocab_size"], n + 3, 7 * trial + i) for i, n in enumerate(lens)]
+        want = [plain.forward(q) for q in seqs]
+        for dtype in DTYPES:
+            eng = Engine.load(folder, dtype=dtype, max_tokens=1024)
+            slots = [eng.acquire() for _ in seqs]
+            lg = eng.step([(sl, q[:n]) for sl, q, n in zip(slots, seqs, lens)], want="all")
+            got, off = [], 0
+            for n in lens:
+                got.append([lg[off:off + n]])
+                off += n
+            for d in range(3):
+                lg = eng.step([(sl, [q[n + d]]) for sl, q, n in zip(slots, seqs, lens)], want="last")
+                for i in range(len(seqs)):
+                    got[i].append(lg[i:i + 1].clone())
+            for i in range(len(seqs)):
+                assert_logits_close(torch.cat(got[i]), want[i], dtype, f"seed {seed} trial {trial} {raw} sequence {i}")
+            for sl in slots:
+                eng.release(sl)
+            eng.cache.check()
+
+
 def test_head_size_24_runs_in_32_bit_and_is_refused_in_bf16():
     scenarios.whole(make_engine, "F", "float32")
     scenarios.last_tokens_one_by_one(make_engine, "F", "float32", tail=8)
