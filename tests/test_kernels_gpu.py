@@ -1016,6 +1016,63 @@ def test_sample_rows_frequencies(ops):
     assert (freq - p).abs().max() < 0.012
 
 
+def test_products_of_random_shapes(ops):
+    """Shapes drawn at random over every kind of product (plain, as partial sums for a reader that adds them, gated)
+    through the entry points that the parts use (parts.linear): each lands in whichever kernel the sizes select, in
+    fragment order where the sizes allow it and in plain rows where they do not, and equals the 64-bit product."""
+    import random
+    from synaptix_amd.parts.linear import Matrix, linear, linear_for_sum
+    r = random.Random(11)
+    done = 0
+    while done < 48:
+        M = r.choice([1, 2, 5, 8, 9, 13, 16, 17, 32, 33, 64, 65, 100, 128, 129, 255, 257, 300, 513, 700])
+        K = r.choice([8, 24, 32, 40, 64, 96, 128, 136, 192, 256, 264, 512, 1000, 1024, 2080, 4096])
+        N = r.choice([8, 16, 24, 32, 48, 80, 96, 128, 160, 200, 384, 400, 1000, 1008, 2048, 4096, 6144, 32784])
+        kind = r.choice(["plain", "sum", "gated"])
+        if kind == "gated":
+            N = max(32, N // 32 * 32)
+        if M * N * K > 6e9:
+            continue
+        done += 1
+        x, w = rnd((M, K), 300 + done, BF16), rnd((N, K), 400 + done, BF16, 0.05)
+        full = x.double() @ w.double().T
+        atol = 4e-4 * math.sqrt(K) + 1e-3
+        if kind == "gated":
+            m = Matrix(ops.pair_rows(w[:N // 2].contiguous().to(DEV), w[N // 2:].contiguous().to(DEV)))
+            out = torch.full((M, N // 2), float("nan"), dtype=BF16, device=DEV)
+            ops.gemm_swiglu(x.to(DEV), m.data, out)
+            g, u = full[:, :N // 2], full[:, N // 2:]
+            close(out, (g / (1 + torch.exp(-g)) * u).float(), atol + 0.02, 1e-2, f"gated {M}x{N}x{K}")
+        else:
+            m = Matrix(w.to(DEV))
+            got = linear(x.to(DEV), m, F32) if kind == "plain" else linear_for_sum(x.to(DEV), m)
+            close(got.sum(0) if got.dim() == 3 else got, full.float(), atol, what=f"{kind} {M}x{N}x{K}")
+
+
+def test_attention_of_random_shapes(ops):
+    """The attention tests above at shapes drawn at random: head sizes 16 to 256, groups of 1 to 20 heads, sequences that
+    begin, end or are cut at page edges, windows down to one key, any number of splits."""
+    import random
+    r = random.Random(12)
+    for _ in range(10):
+        hd = r.choice([16, 32, 48, 64, 80, 96, 112, 128, 160, 256])
+        nkv = r.choice([1, 2, 3, 4, 8])
+        nh = nkv * r.choice([1, 2, 3, 4, 7, 8, 17, 20])
+        if nh * hd > 8192:
+            continue
+        B = r.randint(1, 4)
+        past = [r.choice([0, 0, 1, 63, 64, 65, 100, 200, 500]) for _ in range(B)]
+        new = [r.choice([1, 2, 31, 32, 33, 64, 100, 128, 129, 200, 300]) for _ in range(B)]
+        window = r.choice([0, 0, 0, 1, 37, 64, 70, 200])
+        lens = [r.choice([1, 2, 63, 64, 65, 130, 300, 700, 2100, 5000]) for _ in range(B)]
+        splits = r.choice([1, 2, 3, 4, 8, 16, 32])
+        rot = r.choice([0, hd, hd, hd // 2 if (hd // 2) % 2 == 0 else hd])
+        test_attention_prefill(ops, BF16, nh, nkv, hd, past, new, window)
+        test_attention_decode_bf16(ops, nh, nkv, hd, lens, window, splits)
+        test_attention_decode_with_qkv_intake(ops, nh, nkv, hd, rot, r.random() < 0.7, lens, window, splits,
+                                              r.choice([0, 0, 2, 4, 8]), r.random() < 0.8)
+
+
 def _filter(ops, x, options, ids=None, in_place=False):
     """ops.filter_rows over rows x [R, V] with options = list of dicts (k, p, mp, T, rep, pres, freq) and ids = list of lists."""
     R, V = x.shape
