@@ -221,7 +221,7 @@ def main() -> int:
 
     # ---- prefill of one 2,048-token prompt
     times = []
-    for i in range(5):
+    for i in range(8):       # (the clocks take some tens of milliseconds of work to settle)
         s = eng.acquire()
         toks = prompt()
         torch.cuda.synchronize()
@@ -230,7 +230,7 @@ def main() -> int:
         torch.cuda.synchronize()
         times.append(time.perf_counter() - t0)
         eng.release(s)
-    pre_s = statistics.median(times[2:])
+    pre_s = statistics.median(times[3:])
     pre_flops = prefill_flops(cfg, [prompt_len])
     prefill = {"value": round(prompt_len / pre_s, 1), "tokens": prompt_len, "ms": round(pre_s * 1e3, 3),
                "frac": round(pre_flops / pre_s / MFMA_PEAK["bf16"], 4)}
